@@ -1,0 +1,165 @@
+/*
+ * palimpsa_hip.h — C ABI of libpalimpsa_hip.so: the Palimpsa attention operator
+ * on AMD MI355X (gfx950), hand-written HIP kernels.
+ *
+ * The library is the drop-in for the device side of the reference's operator
+ * package palimpsa/ops/palimpsa/ (three Triton kernels and the Python that
+ * launches them).  Plain pointers and sizes only; no torch types.
+ *
+ * Conventions
+ *   - every buffer is owned by the caller, device-resident, densely packed:
+ *       q,k [B,T,H,dk]  v,b,o,o_var [B,T,H,dv]  gt [B,T,H]  g,Ip [H]
+ *       states [N,H,dv,dk] fp32 in (mu, I) form
+ *     (layouts enforced by the reference through .contiguous():
+ *      chunk_palimpsa_forgetting_scalar.py:14-20, and raw pointer arithmetic:
+ *      fused_recurrent_palimpsa.py:60-66, :89-90).
+ *   - varlen: B == 1, T == total tokens, cu_seqlens int32 [N+1] on the device.
+ *   - kernels are enqueued on the caller's stream (a hipStream_t passed as
+ *     void*); nothing synchronises, allocates or frees.
+ *   - return value: 0 = ok; < 0 = argument error found before any HIP call
+ *     (PAL_E_*); > 0 = a hipError_t from a launch.
+ *   - dk and dv must be multiples of 16 in [16, 256]; callers with other sizes
+ *     zero-pad (padding k,q,v,b with zeros leaves the valid outputs unchanged).
+ */
+#ifndef PALIMPSA_HIP_H
+#define PALIMPSA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PAL_ABI_VERSION 1
+
+/* element types of tensors handed over the boundary */
+#define PAL_DTYPE_F32 0
+#define PAL_DTYPE_BF16 1
+
+/* PalDims.flags */
+#define PAL_FLAG_VARLEN 1u      /* cu_seqlens given (B must be 1)            */
+#define PAL_FLAG_HAS_INIT 2u    /* init_mu / init_I given                    */
+#define PAL_FLAG_STORE_FINAL 4u /* final_mu / final_I requested              */
+#define PAL_FLAG_HAS_VAR 8u     /* o_var (fwd) / do_var (bwd) present        */
+
+/* error codes (negative) */
+#define PAL_OK 0
+#define PAL_E_NULL -1        /* required pointer is NULL                      */
+#define PAL_E_DIM -2         /* non-positive or out-of-range dimension        */
+#define PAL_E_HEADDIM -3     /* dk or dv not a multiple of 16 in [16,256]     */
+#define PAL_E_DTYPE -4       /* unsupported element type                      */
+#define PAL_E_VARLEN_BATCH -5 /* cu_seqlens given with B != 1                 */
+#define PAL_E_CU_SEQLENS -6  /* cu_seqlens not monotone / not starting at 0 / wrong total */
+#define PAL_E_WORKSPACE -7   /* workspace missing or too small                */
+#define PAL_E_CHUNK -8       /* unsupported chunk size                        */
+#define PAL_E_STATE -9       /* init/final state flags and pointers disagree  */
+#define PAL_E_CAPACITY -10   /* output table too small                        */
+#define PAL_E_ALIGN -11      /* pointer not aligned to 16 bytes               */
+
+/* Tokens per chunk tile of the chunked kernels (BASELINE chunk size). */
+#define PAL_CHUNK 64
+
+typedef struct PalDims {
+  int32_t batch;        /* B (1 when varlen)                                  */
+  int32_t seq_len;      /* T per batch row; total packed tokens when varlen   */
+  int32_t n_seqs;       /* N: B, or number of documents when varlen           */
+  int32_t n_heads;      /* H                                                  */
+  int32_t dk;           /* key/query head dim                                 */
+  int32_t dv;           /* value head dim                                     */
+  int32_t total_chunks; /* chunk path: sum over sequences of ceil(len/PAL_CHUNK) */
+  int32_t dtype;        /* PAL_DTYPE_* of q,k,v,b,o and of do,dq,dk,dv,db     */
+  int32_t gate_dtype;   /* PAL_DTYPE_* of gt                                  */
+  int32_t var_dtype;    /* PAL_DTYPE_* of o_var / do_var                      */
+  uint32_t flags;       /* PAL_FLAG_*                                         */
+  float scale;          /* output scale (reference default dk^-0.5)           */
+} PalDims;
+
+/* Forward-side tensors.  Unused optional pointers are NULL. */
+typedef struct PalFwdTensors {
+  const void *q, *k, *v, *b;      /* dtype                                    */
+  const void *gt;                 /* gate_dtype [B,T,H]                       */
+  const float *g, *Ip;            /* fp32 [H]                                 */
+  void *o;                        /* dtype [B,T,H,dv]                         */
+  void *o_var;                    /* var_dtype [B,T,H,dv] or NULL             */
+  const float *init_mu, *init_I;  /* fp32 [N,H,dv,dk] or NULL                 */
+  float *final_mu, *final_I;      /* fp32 [N,H,dv,dk] or NULL (may alias init_*) */
+  const int32_t *cu_seqlens;      /* device int32 [N+1] or NULL               */
+  const int32_t *chunk_table;     /* device int32 [total_chunks,4] (varlen chunk path) */
+  const int32_t *chunk_offsets;   /* device int32 [N+1] (varlen chunk path)   */
+  float *chunk_mu, *chunk_I;      /* fp32 [total_chunks,H,dv,dk]: state at the
+                                     start of every chunk (chunk path)        */
+} PalFwdTensors;
+
+/* Backward-side tensors. */
+typedef struct PalBwdTensors {
+  const void *d_o;                /* dtype [B,T,H,dv]                         */
+  const void *d_o_var;            /* var_dtype [B,T,H,dv] or NULL             */
+  void *dq, *dk;                  /* dtype [B,T,H,dk]                         */
+  void *dv, *db;                  /* dtype [B,T,H,dv]                         */
+  float *dgt;                     /* fp32 [B,T,H]                             */
+  float *dg, *dIp;                /* fp32 [H]                                 */
+  float *d_init_mu, *d_init_I;    /* fp32 [N,H,dv,dk] or NULL                 */
+} PalBwdTensors;
+
+/* ------------------------------------------------------------------ queries */
+
+/* Version of this interface (PAL_ABI_VERSION of the build). */
+int pal_abi_version(void);
+
+/* Text for a code returned by any pal_* function. */
+const char *pal_strerror(int code);
+
+/* Argument check shared by every entry point; no HIP call.  Replaces the
+ * reference's ValueErrors for varlen misuse
+ * (chunk_palimpsa_forgetting_scalar.py:629-630, fused_recurrent_palimpsa.py:273-277)
+ * and extends them to everything a raw-pointer interface can get wrong. */
+int pal_validate_dims(const PalDims *dims);
+
+/* ------------------------------------------------------------- host helpers */
+
+/* Chunk bookkeeping for packed variable-length batches, on the host.
+ * Replaces fla.ops.utils.prepare_chunk_offsets / prepare_chunk_indices as used
+ * at chunk_palimpsa_forgetting_scalar.py:633-641.
+ *   cu_seqlens_host  int64 [n_seqs+1], cu[0] == 0, non-decreasing
+ *   table_out        int32 [capacity,4] rows (seq, first_token, n_tokens, index_in_seq), or NULL to count only
+ *   offsets_out      int32 [n_seqs+1] cumulative chunk counts, or NULL
+ * Returns the total number of chunks (>= 0) or a PAL_E_* code. */
+int pal_build_chunk_table(const int64_t *cu_seqlens_host, int32_t n_seqs, int32_t *table_out,
+                          int32_t capacity, int32_t *offsets_out);
+
+/* ---------------------------------------------------------- recurrent path */
+
+/* Token-serial forward for any T >= 1 (T == 1 is single-step decode).
+ * Replaces fused_palimpsa_recurrent_fwd and its kernel
+ * (fused_recurrent_palimpsa.py:24-209), consuming bf16/fp32 rows directly
+ * instead of the host-side fp32 casts of :226-236. */
+int pal_recurrent_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
+
+/* Backward of pal_recurrent_fwd.  The reference has none
+ * (fused_recurrent_palimpsa.py:250-253 raises NotImplementedError); gradients
+ * follow the naive recurrence chunk_palimpsa_forgetting_scalar.py:669-725. */
+size_t pal_recurrent_bwd_workspace_bytes(const PalDims *dims);
+int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* -------------------------------------------------------------- chunked path */
+
+/* Chunked forward.  Replaces ChunkPalimpsa.forward + chunk_palimpsa_fwd_kernel
+ * (chunk_palimpsa_forgetting_scalar.py:66-218, :441-517).  Fills chunk_mu /
+ * chunk_I (the reference's intermediate_mu_state / intermediate_I_state,
+ * :187-188) for the backward. */
+int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
+
+/* Chunked backward.  Replaces ChunkPalimpsa.backward + chunk_palimpsa_bwd_kernel
+ * (chunk_palimpsa_forgetting_scalar.py:239-434, :519-620), including the host
+ * side .sum(0) reductions of :609-613.  Needs chunk_mu / chunk_I as written by
+ * pal_chunk_fwd on the same inputs. */
+size_t pal_chunk_bwd_workspace_bytes(const PalDims *dims);
+int pal_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PALIMPSA_HIP_H */

@@ -1,0 +1,124 @@
+"""ctypes binding of libpalimpsa_hip.so (the C ABI of include/palimpsa_hip.h).
+
+There is no fallback: if the library is missing the import fails with an
+instruction to build it, and if a kernel call returns an error it is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libpalimpsa_hip.so")
+
+PAL_ABI_VERSION = 1
+PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
+PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
+PAL_CHUNK = 64
+
+PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5
+PAL_E_CU_SEQLENS, PAL_E_WORKSPACE, PAL_E_CHUNK, PAL_E_STATE, PAL_E_CAPACITY, PAL_E_ALIGN = -6, -7, -8, -9, -10, -11
+
+# dk values the token-serial kernels are compiled for
+RECURRENT_DK = (16, 32, 48, 64, 96, 128, 192, 256)
+
+
+class PalDims(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("seq_len", C.c_int32), ("n_seqs", C.c_int32), ("n_heads", C.c_int32),
+        ("dk", C.c_int32), ("dv", C.c_int32), ("total_chunks", C.c_int32),
+        ("dtype", C.c_int32), ("gate_dtype", C.c_int32), ("var_dtype", C.c_int32),
+        ("flags", C.c_uint32), ("scale", C.c_float),
+    ]
+
+
+class PalFwdTensors(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "q", "k", "v", "b", "gt", "g", "Ip", "o", "o_var", "init_mu", "init_I", "final_mu", "final_I",
+        "cu_seqlens", "chunk_table", "chunk_offsets", "chunk_mu", "chunk_I")]
+
+
+class PalBwdTensors(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "d_o", "d_o_var", "dq", "dk", "dv", "db", "dgt", "dg", "dIp", "d_init_mu", "d_init_I")]
+
+
+class PalimpsaHipError(RuntimeError):
+    def __init__(self, code: int, where: str, text: str):
+        super().__init__(f"{where} failed with code {code}: {text}")
+        self.code = code
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library once; raises ImportError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build it with `python -m palimpsa_amd.build` "
+            "(needs hipcc; the kernels target gfx950). There is no CPU or eager fallback.")
+    lib = C.CDLL(LIB_PATH)
+    P = C.POINTER
+    lib.pal_abi_version.restype = C.c_int
+    lib.pal_abi_version.argtypes = []
+    lib.pal_strerror.restype = C.c_char_p
+    lib.pal_strerror.argtypes = [C.c_int]
+    lib.pal_validate_dims.restype = C.c_int
+    lib.pal_validate_dims.argtypes = [P(PalDims)]
+    lib.pal_build_chunk_table.restype = C.c_int
+    lib.pal_build_chunk_table.argtypes = [P(C.c_int64), C.c_int32, P(C.c_int32), C.c_int32, P(C.c_int32)]
+    for name in ("pal_recurrent_fwd", "pal_chunk_fwd"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [P(PalDims), P(PalFwdTensors), C.c_void_p]
+    for name in ("pal_recurrent_bwd", "pal_chunk_bwd"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [P(PalDims), P(PalFwdTensors), P(PalBwdTensors), C.c_void_p, C.c_size_t, C.c_void_p]
+    for name in ("pal_recurrent_bwd_workspace_bytes", "pal_chunk_bwd_workspace_bytes"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_size_t
+        fn.argtypes = [P(PalDims)]
+    if lib.pal_abi_version() != PAL_ABI_VERSION:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.pal_abi_version()} != expected {PAL_ABI_VERSION}; rebuild")
+    _lib = lib
+    return lib
+
+
+def strerror(code: int) -> str:
+    return load().pal_strerror(int(code)).decode()
+
+
+def check(code: int, where: str) -> None:
+    """Map a pal_* return code to the Python exception the reference would raise."""
+    if code == 0:
+        return
+    text = strerror(code)
+    if code in (PAL_E_VARLEN_BATCH, PAL_E_CU_SEQLENS, PAL_E_HEADDIM, PAL_E_DIM, PAL_E_DTYPE, PAL_E_STATE):
+        raise ValueError(f"{where}: {text} (code {code})")
+    raise PalimpsaHipError(code, where, text)
+
+
+def build_chunk_table(cu_seqlens_host):
+    """Host chunk bookkeeping for packed batches: returns (table int32 [n,4], offsets int32 [N+1])."""
+    import numpy as np
+
+    lib = load()
+    cu = np.ascontiguousarray(np.asarray(cu_seqlens_host, dtype=np.int64))
+    n_seqs = int(cu.shape[0]) - 1
+    cu_p = cu.ctypes.data_as(C.POINTER(C.c_int64))
+    total = lib.pal_build_chunk_table(cu_p, n_seqs, None, 0, None)
+    if total < 0:
+        check(total, "pal_build_chunk_table")
+    table = np.zeros((max(total, 1), 4), dtype=np.int32)
+    offsets = np.zeros((n_seqs + 1,), dtype=np.int32)
+    rc = lib.pal_build_chunk_table(cu_p, n_seqs, table.ctypes.data_as(C.POINTER(C.c_int32)), int(table.shape[0]),
+                                   offsets.ctypes.data_as(C.POINTER(C.c_int32)))
+    if rc < 0:
+        check(rc, "pal_build_chunk_table")
+    return table[:total], offsets

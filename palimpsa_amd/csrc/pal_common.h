@@ -1,0 +1,132 @@
+// Shared device/host helpers for the Palimpsa HIP kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/palimpsa_hip.h"
+
+namespace pal {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ------------------------------------------------------------------ scalars
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return (float)x; }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
+
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// gate tensor element i, fp32 or bf16 storage chosen at run time
+__device__ __forceinline__ float load_gate(const void* p, int64_t i, int is_bf16) {
+  return is_bf16 ? (float)((const bf16_t*)p)[i] : ((const float*)p)[i];
+}
+
+// store to an output whose element type is chosen at run time
+__device__ __forceinline__ void store_rt(void* p, int64_t i, float x, int is_bf16) {
+  if (is_bf16) ((bf16_t*)p)[i] = (bf16_t)x;
+  else ((float*)p)[i] = x;
+}
+__device__ __forceinline__ float load_rt(const void* p, int64_t i, int is_bf16) {
+  return is_bf16 ? (float)((const bf16_t*)p)[i] : ((const float*)p)[i];
+}
+
+// ---------------------------------------------------------- vector loads
+// VW consecutive elements starting at p (aligned to VW*sizeof(T)) -> fp32
+template <int VW>
+__device__ __forceinline__ void load_vec(const float* p, float* out) {
+  if constexpr (VW == 4) {
+    f32x4 x = *(const f32x4*)p;
+    out[0] = x[0]; out[1] = x[1]; out[2] = x[2]; out[3] = x[3];
+  } else if constexpr (VW == 2) {
+    f32x2 x = *(const f32x2*)p;
+    out[0] = x[0]; out[1] = x[1];
+  } else {
+    out[0] = *p;
+  }
+}
+template <int VW>
+__device__ __forceinline__ void load_vec(const bf16_t* p, float* out) {
+  if constexpr (VW == 4) {
+    bf16x4 x = *(const bf16x4*)p;
+    out[0] = (float)x[0]; out[1] = (float)x[1]; out[2] = (float)x[2]; out[3] = (float)x[3];
+  } else if constexpr (VW == 2) {
+    bf16x2 x = *(const bf16x2*)p;
+    out[0] = (float)x[0]; out[1] = (float)x[1];
+  } else {
+    out[0] = (float)*p;
+  }
+}
+template <int VW>
+__device__ __forceinline__ void store_vec(float* p, const float* in) {
+  if constexpr (VW == 4) {
+    f32x4 x = {in[0], in[1], in[2], in[3]};
+    *(f32x4*)p = x;
+  } else if constexpr (VW == 2) {
+    f32x2 x = {in[0], in[1]};
+    *(f32x2*)p = x;
+  } else {
+    *p = in[0];
+  }
+}
+
+// ------------------------------------------------------- cross-lane helpers
+// rotate within each row of 16 lanes (DPP row_ror:N)
+template <int N>
+__device__ __forceinline__ float row_ror(float x) {
+  int v = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + N, 0xf, 0xf, false);
+  return __builtin_bit_cast(float, v);
+}
+// sum over the 16 lanes of a row; every lane of the row gets the total
+__device__ __forceinline__ float row16_sum(float x) {
+  x += row_ror<8>(x);
+  x += row_ror<4>(x);
+  x += row_ror<2>(x);
+  x += row_ror<1>(x);
+  return x;
+}
+// sum over the four 16-lane rows of a wave (same lane-in-row); all lanes get it
+__device__ __forceinline__ float rows4_sum(float x) {
+  x += __shfl_xor(x, 16);
+  x += __shfl_xor(x, 32);
+  return x;
+}
+__device__ __forceinline__ float wave_sum(float x) { return rows4_sum(row16_sum(x)); }
+
+// ------------------------------------------------------------------- MFMA
+// D[16x16] += A[16x32] * B[32x16], bf16 operands, fp32 accumulate.
+// lane l holds: A row (l%16), k = 8*(l/16)+j ; B col (l%16), same k ;
+// D col (l%16), rows 4*(l/16)+r.
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x2 pack2(float lo, float hi) {
+  f32x2 x = {lo, hi};
+  return __builtin_convertvector(x, bf16x2);
+}
+
+// ------------------------------------------------------------------ host
+#define PAL_HIP_LAUNCH_CHECK()                 \
+  do {                                         \
+    hipError_t e__ = hipGetLastError();        \
+    if (e__ != hipSuccess) return (int)e__;    \
+  } while (0)
+
+inline bool is_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+}  // namespace pal

@@ -1,0 +1,237 @@
+// Token-serial Palimpsa forward (any T >= 1; T == 1 is single-step decode).
+//
+// Replaces fused_palimpsa_recurrent_fwd_kernel of the reference
+// (palimpsa/ops/palimpsa/fused_recurrent_palimpsa.py:24-154).  Same arithmetic:
+//   f = exp(-gt*g); M = f*M + v k^T; Jbar = f*Jbar + b (k*k)^T; I = Jbar + Ip;
+//   o = scale * (M/I) q ; o_var = scale * (1/I) (q*q)
+// with the (mu, I) external state form of :88-96 and :145-154.
+//
+// Mapping (wave64): one wave per (sequence, head, tile of 4*RD value rows).
+// A row of the dv x dk state is spread over the 16 lanes of a DPP row, NPL =
+// dk/16 entries per lane, so a wave covers 4 value rows at a time; each lane
+// keeps RD*NPL entries of M and of Jbar in registers for the whole sequence.
+// The sum over dk is a 4-step DPP rotation inside the row.  Memory access is
+// the only cost that matters at T == 1: every lane issues all its state loads
+// up front as 16-byte vectors that are contiguous across the row.
+#include "pal_common.h"
+#include "pal_host.h"
+
+namespace pal {
+
+struct RecArgs {
+  const void *q, *k, *v, *b, *gt;
+  const float *g, *Ip;
+  void *o, *o_var;
+  const float *init_mu, *init_I;
+  float *final_mu, *final_I;
+  const int32_t* cu_seqlens;
+  int32_t T, H, dk, dv, n_seqs;
+  int32_t gate_bf16, var_bf16;
+  uint32_t flags;
+  float scale;
+};
+
+// n index of element e of lane j (j = lane % 16); VW-wide vectors interleaved across the row
+template <int NPL>
+struct NMap {
+  static constexpr int VW = (NPL % 4 == 0) ? 4 : ((NPL % 2 == 0) ? 2 : 1);
+  static constexpr int NV = NPL / VW;
+  __device__ static __forceinline__ int vec_start(int j, int iv) { return 16 * VW * iv + VW * j; }
+};
+
+template <typename TIn, int NPL, int RD>
+__global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
+  using Map = NMap<NPL>;
+  constexpr int VW = Map::VW;
+  constexpr int NV = Map::NV;
+  const int lane = threadIdx.x;
+  const int j = lane & 15;
+  const int grp = lane >> 4;
+  const int n_dtiles = a.dv / (4 * RD);
+  const int tile = blockIdx.x % n_dtiles;
+  const int nh = blockIdx.x / n_dtiles;
+  const int h = nh % a.H;
+  const int n = nh / a.H;
+  const int dk = a.dk, dv = a.dv, H = a.H;
+
+  int64_t bos;
+  int T;
+  if (a.cu_seqlens) {
+    bos = a.cu_seqlens[n];
+    T = a.cu_seqlens[n + 1] - (int)bos;
+  } else {
+    bos = (int64_t)n * a.T;
+    T = a.T;
+  }
+  const float gh = a.g[h] * kLog2e;
+  const float Ip = a.Ip[h];
+  const float scale = a.scale;
+  const bool has_var = a.flags & PAL_FLAG_HAS_VAR;
+
+  int drow[RD];
+#pragma unroll
+  for (int rr = 0; rr < RD; ++rr) drow[rr] = tile * (4 * RD) + rr * 4 + grp;
+
+  float M[RD][NPL], J[RD][NPL];
+  if (a.init_mu) {
+#pragma unroll
+    for (int rr = 0; rr < RD; ++rr) {
+      const int64_t base = ((int64_t)nh * dv + drow[rr]) * dk;
+#pragma unroll
+      for (int iv = 0; iv < NV; ++iv) {
+        float mu[VW], I[VW];
+        load_vec<VW>(a.init_mu + base + Map::vec_start(j, iv), mu);
+        load_vec<VW>(a.init_I + base + Map::vec_start(j, iv), I);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) {
+          M[rr][iv * VW + e] = mu[e] * I[e];
+          J[rr][iv * VW + e] = I[e] - Ip;
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int rr = 0; rr < RD; ++rr)
+#pragma unroll
+      for (int e = 0; e < NPL; ++e) { M[rr][e] = 0.f; J[rr][e] = 0.f; }
+  }
+
+  const TIn* qp = (const TIn*)a.q + (bos * H + h) * dk;
+  const TIn* kp = (const TIn*)a.k + (bos * H + h) * dk;
+  const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv;
+  const TIn* bp = (const TIn*)a.b + (bos * H + h) * dv;
+  TIn* op = (TIn*)a.o + (bos * H + h) * dv;
+  const int64_t gt_base = bos * H + h;
+  const int64_t var_base = (bos * H + h) * dv;
+
+  float kc[NPL], qc[NPL], vc[RD], bc[RD], gtc;
+  auto load_token = [&](int t, float* kk_, float* qq_, float* vv_, float* bb_, float& gt_) {
+    const int64_t off_k = (int64_t)t * H * dk;
+    const int64_t off_v = (int64_t)t * H * dv;
+#pragma unroll
+    for (int iv = 0; iv < NV; ++iv) {
+      load_vec<VW>(kp + off_k + Map::vec_start(j, iv), kk_ + iv * VW);
+      load_vec<VW>(qp + off_k + Map::vec_start(j, iv), qq_ + iv * VW);
+    }
+#pragma unroll
+    for (int rr = 0; rr < RD; ++rr) {
+      vv_[rr] = to_f32(vp[off_v + drow[rr]]);
+      bb_[rr] = to_f32(bp[off_v + drow[rr]]);
+    }
+    gt_ = load_gate(a.gt, gt_base + (int64_t)t * H, a.gate_bf16);
+  };
+
+  if (T > 0) load_token(0, kc, qc, vc, bc, gtc);
+  for (int t = 0; t < T; ++t) {
+    float kn[NPL], qn[NPL], vn[RD], bn[RD], gtn = 0.f;
+    const bool more = (t + 1 < T);
+    if (more) load_token(t + 1, kn, qn, vn, bn, gtn);
+
+    const float f = fast_exp2(-gtc * gh);
+    float kk[NPL];
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) kk[e] = kc[e] * kc[e];
+#pragma unroll
+    for (int rr = 0; rr < RD; ++rr) {
+      float acc = 0.f, accv = 0.f;
+#pragma unroll
+      for (int e = 0; e < NPL; ++e) {
+        M[rr][e] = fmaf(f, M[rr][e], vc[rr] * kc[e]);
+        J[rr][e] = fmaf(f, J[rr][e], bc[rr] * kk[e]);
+        const float rI = fast_rcp(J[rr][e] + Ip);
+        acc = fmaf(M[rr][e] * rI, qc[e], acc);
+        if (has_var) accv = fmaf(qc[e] * qc[e], rI, accv);
+      }
+      acc = row16_sum(acc) * scale;
+      if (j == 0) op[(int64_t)t * H * dv + drow[rr]] = from_f32<TIn>(acc);
+      if (has_var) {
+        accv = row16_sum(accv) * scale;
+        if (j == 0) store_rt(a.o_var, var_base + (int64_t)t * H * dv + drow[rr], accv, a.var_bf16);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int e = 0; e < NPL; ++e) { kc[e] = kn[e]; qc[e] = qn[e]; }
+#pragma unroll
+      for (int rr = 0; rr < RD; ++rr) { vc[rr] = vn[rr]; bc[rr] = bn[rr]; }
+      gtc = gtn;
+    }
+  }
+
+  if (a.final_mu) {
+#pragma unroll
+    for (int rr = 0; rr < RD; ++rr) {
+      const int64_t base = ((int64_t)nh * dv + drow[rr]) * dk;
+#pragma unroll
+      for (int iv = 0; iv < NV; ++iv) {
+        float mu[VW], I[VW];
+#pragma unroll
+        for (int e = 0; e < VW; ++e) {
+          I[e] = J[rr][iv * VW + e] + Ip;
+          mu[e] = M[rr][iv * VW + e] * fast_rcp(I[e]);
+        }
+        store_vec<VW>(a.final_mu + base + Map::vec_start(j, iv), mu);
+        store_vec<VW>(a.final_I + base + Map::vec_start(j, iv), I);
+      }
+    }
+  }
+}
+
+template <typename TIn, int NPL>
+static int launch_npl(const RecArgs& a, int rd, hipStream_t s) {
+  const int64_t blocks = (int64_t)a.n_seqs * a.H * (a.dv / (4 * rd));
+  if (blocks > 0x7fffffff) return PAL_E_DIM;
+  if (rd == 4) hipLaunchKernelGGL((recurrent_fwd_kernel<TIn, NPL, 4>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+  else hipLaunchKernelGGL((recurrent_fwd_kernel<TIn, NPL, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+template <typename TIn>
+static int launch_dtype(const RecArgs& a, int rd, hipStream_t s) {
+  switch (a.dk / 16) {
+    case 1: return launch_npl<TIn, 1>(a, rd, s);
+    case 2: return launch_npl<TIn, 2>(a, rd, s);
+    case 3: return launch_npl<TIn, 3>(a, rd, s);
+    case 4: return launch_npl<TIn, 4>(a, rd, s);
+    case 6: return launch_npl<TIn, 6>(a, rd, s);
+    case 8: return launch_npl<TIn, 8>(a, rd, s);
+    case 12: return launch_npl<TIn, 12>(a, rd, s);
+    case 16: return launch_npl<TIn, 16>(a, rd, s);
+    default: return PAL_E_HEADDIM;
+  }
+}
+
+bool recurrent_dk_supported(int dk) {
+  switch (dk) {
+    case 16: case 32: case 48: case 64: case 96: case 128: case 192: case 256: return true;
+    default: return false;
+  }
+}
+
+}  // namespace pal
+
+extern "C" int pal_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
+  using namespace pal;
+  int rc = check_fwd_common(d, t);
+  if (rc) return rc;
+  if (!recurrent_dk_supported(d->dk)) return PAL_E_HEADDIM;
+  RecArgs a;
+  a.q = t->q; a.k = t->k; a.v = t->v; a.b = t->b; a.gt = t->gt;
+  a.g = t->g; a.Ip = t->Ip; a.o = t->o;
+  a.o_var = (d->flags & PAL_FLAG_HAS_VAR) ? t->o_var : nullptr;
+  a.init_mu = t->init_mu; a.init_I = t->init_I;
+  a.final_mu = t->final_mu; a.final_I = t->final_I;
+  a.cu_seqlens = t->cu_seqlens;
+  a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv; a.n_seqs = d->n_seqs;
+  a.gate_bf16 = d->gate_dtype == PAL_DTYPE_BF16;
+  a.var_bf16 = d->var_dtype == PAL_DTYPE_BF16;
+  a.flags = d->flags;
+  a.scale = d->scale;
+  // 16 value rows per wave once that still gives every SIMD of the chip two waves
+  const int64_t waves16 = (int64_t)d->n_seqs * d->n_heads * (d->dv / 16);
+  const int rd = (waves16 >= 2048) ? 4 : 1;
+  hipStream_t s = (hipStream_t)stream;
+  if (d->dtype == PAL_DTYPE_BF16) return launch_dtype<bf16_t>(a, rd, s);
+  return launch_dtype<float>(a, rd, s);
+}

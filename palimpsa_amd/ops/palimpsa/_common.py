@@ -1,0 +1,156 @@
+"""Host-side plumbing shared by the two operator entry points: dtype and layout
+normalisation, zero-padding of head dims the kernels are not compiled for, and
+filling the C structs.  PyTorch is used for device memory and streams only."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from ... import _lib as L
+
+
+def _require_gpu(*tensors) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError(
+            "palimpsa_amd runs on an AMD GPU only (hand-written HIP kernels for gfx950); "
+            f"got a tensor on '{dev}'. There is no CPU fallback: use palimpsa_ref for a CPU evaluation.")
+    for t in tensors:
+        if t is not None and t.device != dev:
+            raise ValueError(f"all tensors must be on {dev}, found {t.device}")
+    return dev
+
+
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
+def padded_dk(dk: int, recurrent: bool) -> int:
+    if dk > 256:
+        raise ValueError(f"head dim {dk} > 256 is not supported")
+    if recurrent:
+        for c in L.RECURRENT_DK:
+            if c >= dk:
+                return c
+    return _round_up(dk, 16)
+
+
+def padded_dv(dv: int) -> int:
+    if dv > 256:
+        raise ValueError(f"value head dim {dv} > 256 is not supported")
+    return _round_up(dv, 16)
+
+
+def _pal_dtype(dt: torch.dtype) -> int:
+    return L.PAL_DTYPE_BF16 if dt == torch.bfloat16 else L.PAL_DTYPE_F32
+
+
+@dataclass
+class Prepared:
+    """Kernel-ready views of the operator inputs (contiguous, padded, supported dtypes)."""
+    q: torch.Tensor
+    k: torch.Tensor
+    v: torch.Tensor
+    b: torch.Tensor
+    gt: torch.Tensor
+    g: torch.Tensor
+    Ip: torch.Tensor
+    init_mu: Optional[torch.Tensor]
+    init_I: Optional[torch.Tensor]
+    cu_seqlens: Optional[torch.Tensor]
+    dk: int          # logical dims
+    dv: int
+    dk_p: int        # padded dims handed to the kernels
+    dv_p: int
+    n_seqs: int
+    compute_dtype: torch.dtype
+
+
+def prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens, recurrent: bool) -> Prepared:
+    dev = _require_gpu(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state)
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or b.shape != v.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError("expected q,k [B,T,H,dk] and v,b [B,T,H,dv]")
+    if tuple(gt.shape) != tuple(q.shape[:3]):
+        raise ValueError(f"gt must be [B,T,H]={tuple(q.shape[:3])}, got {tuple(gt.shape)}")
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    if g.numel() != H or Ip.numel() != H:
+        raise ValueError("g and Ip must have one entry per head")
+    # one element type for q,k,v,b: bf16 stays bf16, everything else computes from fp32 rows
+    cd = torch.bfloat16 if all(x.dtype == torch.bfloat16 for x in (q, k, v, b)) else torch.float32
+    q, k, v, b = [x.to(cd).contiguous() for x in (q, k, v, b)]
+    if gt.dtype not in (torch.float32, torch.bfloat16):
+        gt = gt.float()
+    gt = gt.contiguous()
+    g = g.reshape(H).float().contiguous()
+    Ip = Ip.reshape(H).float().contiguous()
+    n_seqs = B
+    if cu_seqlens is not None:
+        n_seqs = int(cu_seqlens.numel()) - 1
+        cu_seqlens = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+    dk_p, dv_p = padded_dk(dk, recurrent), padded_dv(dv)
+    if dk_p != dk:
+        q = F.pad(q, (0, dk_p - dk))
+        k = F.pad(k, (0, dk_p - dk))
+    if dv_p != dv:
+        v = F.pad(v, (0, dv_p - dv))
+        b = F.pad(b, (0, dv_p - dv))
+    if (initial_mu_state is None) != (initial_I_state is None):
+        # the layer may hand over a bare recurrent state (layers/palimpsa.py:305-306 of the
+        # reference); the kernels need both halves
+        raise ValueError("initial_mu_state and initial_I_state must be given together")
+    if initial_mu_state is not None:
+        exp = (n_seqs, H, dv, dk)
+        if tuple(initial_mu_state.shape) != exp or tuple(initial_I_state.shape) != exp:
+            raise ValueError(f"Initial states mismatch: expected {exp}, got "
+                             f"{tuple(initial_mu_state.shape)} / {tuple(initial_I_state.shape)}")
+        initial_mu_state = initial_mu_state.float().contiguous()
+        initial_I_state = initial_I_state.float().contiguous()
+        if dk_p != dk or dv_p != dv:
+            pad = (0, dk_p - dk, 0, dv_p - dv)
+            initial_mu_state = F.pad(initial_mu_state, pad, value=0.0)
+            initial_I_state = F.pad(initial_I_state, pad, value=1.0)
+    return Prepared(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens,
+                    dk, dv, dk_p, dv_p, n_seqs, cd)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def make_dims(p: Prepared, scale: float, flags: int, total_chunks: int = 0, var_dtype: torch.dtype = torch.float32) -> L.PalDims:
+    B, T, H, _ = p.q.shape
+    return L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=p.dk_p, dv=p.dv_p,
+                     total_chunks=total_chunks, dtype=_pal_dtype(p.compute_dtype),
+                     gate_dtype=_pal_dtype(p.gt.dtype), var_dtype=_pal_dtype(var_dtype),
+                     flags=flags, scale=float(scale))
+
+
+def make_fwd_tensors(p: Prepared, o, o_var, final_mu, final_I, chunk_table=None, chunk_offsets=None,
+                     chunk_mu=None, chunk_I=None) -> L.PalFwdTensors:
+    return L.PalFwdTensors(
+        q=_ptr(p.q), k=_ptr(p.k), v=_ptr(p.v), b=_ptr(p.b), gt=_ptr(p.gt), g=_ptr(p.g), Ip=_ptr(p.Ip),
+        o=_ptr(o), o_var=_ptr(o_var), init_mu=_ptr(p.init_mu), init_I=_ptr(p.init_I),
+        final_mu=_ptr(final_mu), final_I=_ptr(final_I), cu_seqlens=_ptr(p.cu_seqlens),
+        chunk_table=_ptr(chunk_table), chunk_offsets=_ptr(chunk_offsets),
+        chunk_mu=_ptr(chunk_mu), chunk_I=_ptr(chunk_I))
+
+
+def current_stream_ptr(dev: torch.device):
+    return C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def unpad_state(x: Optional[torch.Tensor], p: Prepared):
+    if x is None or (p.dk_p == p.dk and p.dv_p == p.dv):
+        return x
+    return x[:, :, :p.dv, :p.dk].contiguous()
+
+
+def unpad_last(x: Optional[torch.Tensor], n: int):
+    if x is None or x.shape[-1] == n:
+        return x
+    return x[..., :n].contiguous()

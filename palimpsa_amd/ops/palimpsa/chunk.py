@@ -1,0 +1,196 @@
+"""Chunk-parallel Palimpsa operator (training / prefill path) on HIP kernels.
+
+Mirrors palimpsa/ops/palimpsa/chunk_palimpsa_forgetting_scalar.py of the
+reference: ``chunk_palimpsa`` (:623-667) and the 17-argument
+``ChunkPalimpsa`` autograd Function (:437-620) keep their names, argument
+order, defaults, return packing and ValueError.  Deliberate differences:
+
+* the kernels always work on tiles of 64 tokens; ``chunk_size`` is accepted for
+  signature compatibility and validated, but results do not depend on it (the
+  chunked form is exact for any tile size) and the chunk-state buffers are
+  sized for 64-token tiles;
+* ``chunk_offsets`` (argument 15 of the Function) carries this build's packed
+  chunk metadata for varlen batches: ``[N+1]`` cumulative chunk counts followed
+  by ``[total_chunks,4]`` rows (sequence, first token, length, index in
+  sequence);
+* gradients of fp32 inputs (gt, g, Ip) come back in fp32 instead of being
+  rounded to q.dtype (:617-620), and gradients for the initial states are
+  returned instead of None;
+* no ``torch.autocast`` wrapper (:440, :521).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from ... import _lib as L
+from . import _common as cm
+
+
+def _chunk_meta(cu_seqlens: torch.Tensor):
+    """cu_seqlens (any int dtype/device) -> (packed int32 metadata tensor on CPU, total_chunks)."""
+    cu_host = cu_seqlens.detach().to("cpu", torch.int64).numpy()
+    table, offsets = L.build_chunk_table(cu_host)
+    packed = torch.cat([torch.from_numpy(offsets), torch.from_numpy(table.reshape(-1))]).to(torch.int32)
+    return packed, int(table.shape[0])
+
+
+def _count_chunks(T: int, B: int) -> int:
+    return (T + L.PAL_CHUNK - 1) // L.PAL_CHUNK * B
+
+
+class ChunkPalimpsa(torch.autograd.Function):
+    """forward(ctx, q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
+    output_final_state, output_uncertainty, cu_seqlens, chunk_offsets, int_mu, int_I)
+    -> (o, o_var | None, final_mu, final_I); argument order of chunk...py:441."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
+                output_final_state, output_uncertainty, cu_seqlens, chunk_offsets, int_mu, int_I):
+        p = cm.prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens,
+                              recurrent=False)
+        dev = p.q.device
+        B, T, H, _ = p.q.shape
+        table = offsets = None
+        if p.cu_seqlens is not None:
+            if chunk_offsets is None:
+                chunk_offsets, _ = _chunk_meta(cu_seqlens)
+            meta = chunk_offsets.to(device=dev, dtype=torch.int32).contiguous()
+            offsets = meta[: p.n_seqs + 1]
+            table = meta[p.n_seqs + 1:]
+            total_chunks = int(table.numel()) // 4
+        else:
+            total_chunks = _count_chunks(T, B)
+        need = (total_chunks, H, p.dv_p, p.dk_p)
+        if (int_mu is None or int_I is None or tuple(int_mu.shape) != need or tuple(int_I.shape) != need
+                or int_mu.dtype != torch.float32 or int_I.dtype != torch.float32
+                or int_mu.device != dev or not int_mu.is_contiguous() or not int_I.is_contiguous()):
+            int_mu = torch.empty(need, dtype=torch.float32, device=dev)
+            int_I = torch.empty(need, dtype=torch.float32, device=dev)
+        o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
+        # the reference hands o_var back in q.dtype (chunk...py:515)
+        o_var = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev) if output_uncertainty else None
+        # final states are always produced, as in the reference (chunk...py:475-476)
+        final_mu = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+        final_I = torch.empty_like(final_mu)
+        flags = L.PAL_FLAG_STORE_FINAL
+        if p.cu_seqlens is not None:
+            flags |= L.PAL_FLAG_VARLEN
+        if p.init_mu is not None:
+            flags |= L.PAL_FLAG_HAS_INIT
+        if output_uncertainty:
+            flags |= L.PAL_FLAG_HAS_VAR
+        dims = cm.make_dims(p, scale, flags, total_chunks, var_dtype=p.compute_dtype)
+        tens = cm.make_fwd_tensors(p, o, o_var, final_mu, final_I, table, offsets, int_mu, int_I)
+        with torch.cuda.device(dev):
+            rc = L.load().pal_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
+        L.check(rc, "pal_chunk_fwd")
+
+        ctx.save_for_backward(p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens,
+                              table, offsets, int_mu, int_I)
+        ctx.meta = dict(dk=p.dk, dv=p.dv, dk_p=p.dk_p, dv_p=p.dv_p, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype,
+                        scale=float(scale), flags=flags & ~L.PAL_FLAG_STORE_FINAL, total_chunks=total_chunks,
+                        in_dtypes=(q.dtype, k.dtype, v.dtype, b.dtype, gt.dtype, g.dtype, Ip.dtype),
+                        g_shape=tuple(g.shape), Ip_shape=tuple(Ip.shape), has_init=p.init_mu is not None,
+                        output_uncertainty=bool(output_uncertainty))
+        o = cm.unpad_last(o, p.dv).to(q.dtype)
+        o_var = cm.unpad_last(o_var, p.dv).to(q.dtype) if output_uncertainty else None
+        return o, o_var, cm.unpad_state(final_mu, p), cm.unpad_state(final_I, p)
+
+    @staticmethod
+    def backward(ctx, do, do_var=None, d_mu=None, d_I=None):
+        # incoming gradients of the final states are ignored, as in the reference (chunk...py:522)
+        (q, k, v, b, gt, g, Ip, init_mu, init_I, cu, table, offsets, int_mu, int_I) = ctx.saved_tensors
+        m = ctx.meta
+        dev = q.device
+        B, T, H, dk_p = q.shape
+        dv_p = v.shape[-1]
+        cd = m["compute_dtype"]
+        has_var = m["output_uncertainty"] and do_var is not None
+
+        def prep_grad(x):
+            x = x.to(cd)
+            if dv_p != m["dv"]:
+                x = torch.nn.functional.pad(x, (0, dv_p - m["dv"]))
+            return x.contiguous()
+
+        do_p = prep_grad(do)
+        dovar_p = prep_grad(do_var) if has_var else None
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        db = torch.empty_like(b)
+        dgt = torch.empty(B, T, H, dtype=torch.float32, device=dev)
+        dg = torch.empty(H, dtype=torch.float32, device=dev)
+        dIp = torch.empty(H, dtype=torch.float32, device=dev)
+        d_init_mu = d_init_I = None
+        if m["has_init"]:
+            d_init_mu = torch.empty_like(init_mu)
+            d_init_I = torch.empty_like(init_I)
+        flags = m["flags"]
+        if has_var:
+            flags |= L.PAL_FLAG_HAS_VAR
+        else:
+            flags &= ~L.PAL_FLAG_HAS_VAR
+        dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p,
+                         total_chunks=m["total_chunks"], dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype),
+                         var_dtype=cm._pal_dtype(cd), flags=flags, scale=m["scale"])
+        pt = cm._ptr
+        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
+                               o_var=None, init_mu=pt(init_mu), init_I=pt(init_I), final_mu=None, final_I=None,
+                               cu_seqlens=pt(cu), chunk_table=pt(table), chunk_offsets=pt(offsets),
+                               chunk_mu=pt(int_mu), chunk_I=pt(int_I))
+        grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk), dv=pt(dv), db=pt(db),
+                                dgt=pt(dgt), dg=pt(dg), dIp=pt(dIp), d_init_mu=pt(d_init_mu), d_init_I=pt(d_init_I))
+        lib = L.load()
+        ws_bytes = int(lib.pal_chunk_bwd_workspace_bytes(dims))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.pal_chunk_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, cm.current_stream_ptr(dev))
+        L.check(rc, "pal_chunk_bwd")
+        dts = m["in_dtypes"]
+        dq = cm.unpad_last(dq, m["dk"]).to(dts[0])
+        dk = cm.unpad_last(dk, m["dk"]).to(dts[1])
+        dv = cm.unpad_last(dv, m["dv"]).to(dts[2])
+        db = cm.unpad_last(db, m["dv"]).to(dts[3])
+        dgt = dgt.to(dts[4])
+        dg = dg.reshape(m["g_shape"]).to(dts[5])
+        dIp = dIp.reshape(m["Ip_shape"]).to(dts[6])
+        if d_init_mu is not None and (dk_p != m["dk"] or dv_p != m["dv"]):
+            d_init_mu = d_init_mu[:, :, :m["dv"], :m["dk"]].contiguous()
+            d_init_I = d_init_I[:, :, :m["dv"], :m["dk"]].contiguous()
+        return (dq, dk, dv, db, dgt, dg, dIp, d_init_mu, d_init_I,
+                None, None, None, None, None, None, None, None)
+
+
+def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state=None, scale=None,
+                   chunk_size=16, output_final_state=False, output_uncertainty=False, cu_seqlens=None):
+    """Chunked Palimpsa attention; calling convention of chunk_palimpsa in the reference
+    (chunk...py:623-667).  Returns ``o`` (or ``(o, o_var)``), plus the final ``(mu, I)``
+    states when ``output_final_state`` is set."""
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    if not isinstance(chunk_size, int) or chunk_size <= 0:
+        raise ValueError(f"chunk_size must be a positive int, got {chunk_size!r}")
+    chunk_offsets = None
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
+        chunk_offsets, total_chunks = _chunk_meta(cu_seqlens)
+        chunk_offsets = chunk_offsets.to(q.device)
+    else:
+        total_chunks = _count_chunks(q.shape[1], q.shape[0])
+    H = q.shape[-2]
+    dk_p, dv_p = cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1])
+    # chunk-start states, allocated outside the autograd Function as in the reference (chunk...py:652-653)
+    int_mu = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
+    int_I = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
+    o, o_var, final_mu_state, final_I_state = ChunkPalimpsa.apply(
+        q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
+        output_final_state, output_uncertainty, cu_seqlens, chunk_offsets, int_mu, int_I)
+    out = (o, o_var) if output_uncertainty else o
+    if output_final_state:
+        return out, final_mu_state, final_I_state
+    return out

@@ -1,0 +1,150 @@
+"""GPU parity of the token-serial (fused-recurrent / decode) HIP path against the CPU oracle.
+
+Every call goes through palimpsa_amd.ops.palimpsa -> ctypes -> the C ABI of
+libpalimpsa_hip.so.  Tolerances: fp32 max|x-ref|/max|ref| <= 1e-4; bf16 rows
+max|x-ref| <= 2e-2 on outputs (oracle fed the same bf16-rounded rows).
+"""
+import pytest
+import torch
+
+from oracle import palimpsa_oracle as po
+from tests import helpers as hp
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from palimpsa_amd.ops.palimpsa import fused_recurrent_palimpsa
+    return fused_recurrent_palimpsa
+
+
+def test_c0_fp32_forward_and_final_state(gpu_device):
+    """BASELINE config 0: B=2, T=256, H=4, dk=dv=32, fp32, seed 0, zero mean state, I0 = Ip."""
+    fr = _ops()
+    inp = po.make_inputs(2, 256, 4, 32, 32, seed=0)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp)
+    d = hp.to_device(inp, gpu_device)
+    o, mu, I = fr(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"], output_final_state=True)
+    assert o.dtype == torch.float32 and o.shape == (2, 256, 4, 32)
+    assert mu.shape == (2, 4, 32, 32) and I.dtype == torch.float32
+    assert hp.max_rel(o, o_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(mu, mu_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(I, I_ref) <= hp.FP32_REL_TOL
+
+
+@pytest.mark.parametrize("dk,dv", [(16, 16), (48, 96), (64, 64), (96, 96), (128, 128), (192, 48), (256, 32)])
+def test_fp32_all_compiled_head_dims_with_state_and_var(gpu_device, dk, dv):
+    fr = _ops()
+    B, T, H = 2, 37, 3
+    inp = po.make_inputs(B, T, H, dk, dv, seed=dk + dv, g_value=2.0)
+    inp["g"] = torch.linspace(1.0, 16.0, H)
+    inp["Ip"] = torch.tensor([0.5, 1.0, 2.5])
+    gen = torch.Generator().manual_seed(5)
+    mu0 = torch.randn(B, H, dv, dk, generator=gen) * 0.1
+    I0 = inp["Ip"].view(1, H, 1, 1) + torch.nn.functional.softplus(torch.randn(B, H, dv, dk, generator=gen))
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, scale=0.7, mu0=mu0, I0=I0, want_var=True)
+    d = hp.to_device(inp, gpu_device)
+    (o, ov), mu, I = fr(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"], scale=0.7,
+                        initial_mu_state=mu0.to(gpu_device), initial_I_state=I0.to(gpu_device),
+                        output_final_state=True, output_uncertainty=True)
+    assert hp.max_rel(o, o_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(ov, ov_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(mu, mu_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(I, I_ref) <= hp.FP32_REL_TOL
+
+
+def test_reference_check_script_shape_odd_dims(gpu_device):
+    """Topology of the reference's own check (check_palimpsa.py:43-59): dv=65, dk=31, L=511,
+    unnormalised q,k, g = |N|*10+1, Ip = |N|+0.1, scale=1; fewer batch rows to keep the CPU side short."""
+    fr = _ops()
+    gen = torch.Generator().manual_seed(42)
+    B, T, H, D, N = 2, 511, 4, 65, 31
+    v = torch.randn(B, T, H, D, generator=gen)
+    q = torch.randn(B, T, H, N, generator=gen)
+    k = torch.randn(B, T, H, N, generator=gen)
+    b = torch.sigmoid(torch.randn(B, T, H, D, generator=gen))
+    gt = torch.sigmoid(torch.randn(B, T, H, generator=gen))
+    g = torch.randn(H, generator=gen).abs() * 10 + 1
+    Ip = torch.randn(H, generator=gen).abs() + 0.1
+    inp = dict(q=q, k=k, v=v, b=b, gt=gt, g=g, Ip=Ip)
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, scale=1.0, want_var=True)
+    d = hp.to_device(inp, gpu_device)
+    (o, ov), mu, I = fr(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"], scale=1,
+                        output_final_state=True, output_uncertainty=True)
+    assert o.shape == (B, T, H, D) and mu.shape == (B, H, D, N)
+    assert hp.max_rel(o, o_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(ov, ov_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(mu, mu_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(I, I_ref) <= hp.FP32_REL_TOL
+
+
+def test_varlen_with_states(gpu_device):
+    fr = _ops()
+    H, dk, dv = 2, 32, 48
+    cu = [0, 1, 18, 19, 83, 200]
+    T = cu[-1]
+    N = len(cu) - 1
+    inp = po.make_inputs(1, T, H, dk, dv, seed=3)
+    gen = torch.Generator().manual_seed(6)
+    mu0 = torch.randn(N, H, dv, dk, generator=gen) * 0.1
+    I0 = 1.0 + torch.rand(N, H, dv, dk, generator=gen)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0, I0=I0, cu=cu)
+    d = hp.to_device(inp, gpu_device)
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=gpu_device)
+    o, mu, I = fr(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"],
+                  initial_mu_state=mu0.to(gpu_device), initial_I_state=I0.to(gpu_device),
+                  output_final_state=True, cu_seqlens=cu_t)
+    assert hp.max_rel(o, o_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(mu, mu_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(I, I_ref) <= hp.FP32_REL_TOL
+
+
+def test_bf16_rows_decode_steps(gpu_device):
+    """Config-3 style decode on a small batch: bf16 rows, fp32 states fed back for 16 steps."""
+    fr = _ops()
+    B, H, d, steps = 3, 2, 128, 16
+    inp = hp.rounded(po.make_inputs(B, steps, H, d, d, seed=0), torch.bfloat16)
+    gen = torch.Generator().manual_seed(1)
+    mu0 = torch.randn(B, H, d, d, generator=gen) * 0.1
+    I0 = torch.nn.functional.softplus(torch.randn(B, H, d, d, generator=gen))
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0, I0=I0)
+    dd = hp.to_device(inp, gpu_device)
+    mu, I = mu0.to(gpu_device), I0.to(gpu_device)
+    outs = []
+    for t in range(steps):
+        sl = slice(t, t + 1)
+        o, mu, I = fr(dd["q"][:, sl], dd["k"][:, sl], dd["v"][:, sl], dd["b"][:, sl], dd["gt"][:, sl],
+                      dd["g"], dd["Ip"], initial_mu_state=mu, initial_I_state=I, output_final_state=True)
+        assert o.dtype == torch.bfloat16
+        outs.append(o)
+    o = torch.cat(outs, dim=1)
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    # states are fp32 end to end: same bar as the fp32 kernels
+    assert hp.max_rel(mu, mu_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(I, I_ref) <= hp.FP32_REL_TOL
+
+
+def test_split_resume_property_full_width(gpu_device):
+    """Size-independent property at a decode-sized head (H=16, d=128): [0,T) == [0,T1) + [T1,T)."""
+    fr = _ops()
+    B, T, H, d = 4, 96, 16, 128
+    inp = hp.to_device(hp.rounded(po.make_inputs(B, T, H, d, d, seed=9), torch.bfloat16), gpu_device)
+    a = (inp["g"], inp["Ip"])
+    o, mu, I = fr(inp["q"], inp["k"], inp["v"], inp["b"], inp["gt"], *a, output_final_state=True)
+    T1 = 41
+    s1, s2 = slice(0, T1), slice(T1, T)
+    o1, mu1, I1 = fr(inp["q"][:, s1], inp["k"][:, s1], inp["v"][:, s1], inp["b"][:, s1], inp["gt"][:, s1], *a,
+                     output_final_state=True)
+    o2, mu2, I2 = fr(inp["q"][:, s2], inp["k"][:, s2], inp["v"][:, s2], inp["b"][:, s2], inp["gt"][:, s2], *a,
+                     initial_mu_state=mu1, initial_I_state=I1, output_final_state=True)
+    assert hp.max_abs(torch.cat([o1, o2], 1).float(), o.float()) <= 1e-2
+    assert hp.max_rel(mu2, mu) <= 1e-5
+    assert hp.max_rel(I2, I) <= 1e-5
+
+
+def test_error_paths_match_reference(gpu_device):
+    fr = _ops()
+    inp = hp.to_device(po.make_inputs(2, 8, 2, 16, 16, seed=0), gpu_device)
+    cu = torch.tensor([0, 8], device=gpu_device)
+    with pytest.raises(ValueError):
+        fr(inp["q"], inp["k"], inp["v"], inp["b"], inp["gt"], inp["g"], inp["Ip"], cu_seqlens=cu)
