@@ -1,0 +1,116 @@
+"""GPU parity of the chunked forward (bf16 MFMA kernels) against the CPU oracle.
+
+Calls go through palimpsa_amd.ops.palimpsa.chunk_palimpsa -> ctypes -> C ABI.
+The chunked kernels contract in bf16 on the matrix cores whatever the input
+dtype, so their bar is the bf16 one: max|o - ref| <= 2e-2 with the oracle fed
+the same rounded rows.  Final states accumulate bf16-rounded products in fp32:
+max|x-ref|/max|ref| <= 1e-2.
+"""
+import pytest
+import torch
+
+from oracle import palimpsa_oracle as po
+from tests import helpers as hp
+
+pytestmark = pytest.mark.gpu
+STATE_REL_TOL = 1e-2
+
+
+def _ops():
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa, fused_recurrent_palimpsa
+    return chunk_palimpsa, fused_recurrent_palimpsa
+
+
+def _call(fn, d, **kw):
+    return fn(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"], **kw)
+
+
+@pytest.mark.parametrize("T", [1, 63, 64, 65, 200])
+def test_bf16_forward_lengths(gpu_device, T):
+    ck, _ = _ops()
+    inp = hp.rounded(po.make_inputs(2, T, 3, 64, 64, seed=T), torch.bfloat16)
+    inp["g"] = torch.tensor([1.0, 4.0, 0.25])
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, want_var=True)
+    d = hp.to_device(inp, gpu_device)
+    (o, ov), mu, I = _call(ck, d, output_final_state=True, output_uncertainty=True, chunk_size=64)
+    assert o.dtype == torch.bfloat16 and ov.dtype == torch.bfloat16
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_abs(ov, ov_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL
+    assert hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
+@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 32), (48, 96), (96, 96), (128, 128), (64, 192), (256, 32), (31, 65)])
+def test_bf16_forward_head_dims_with_initial_state(gpu_device, dk, dv):
+    ck, _ = _ops()
+    B, T, H = 2, 130, 2
+    inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=dk * 3 + dv), torch.bfloat16)
+    inp["Ip"] = torch.tensor([0.5, 2.0])
+    gen = torch.Generator().manual_seed(2)
+    mu0 = torch.randn(B, H, dv, dk, generator=gen) * 0.1
+    I0 = inp["Ip"].view(1, H, 1, 1) + torch.nn.functional.softplus(torch.randn(B, H, dv, dk, generator=gen))
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, scale=0.5, mu0=mu0, I0=I0)
+    d = hp.to_device(inp, gpu_device)
+    o, mu, I = _call(ck, d, scale=0.5, initial_mu_state=mu0.to(gpu_device), initial_I_state=I0.to(gpu_device),
+                     output_final_state=True)
+    assert o.shape == (B, T, H, dv) and mu.shape == (B, H, dv, dk)
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL
+    assert hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
+def test_fp32_inputs_run_at_bf16_contraction_accuracy(gpu_device):
+    ck, _ = _ops()
+    inp = po.make_inputs(2, 100, 2, 32, 48, seed=4)
+    o_ref, _, _, _ = hp.oracle_forward(inp)
+    d = hp.to_device(inp, gpu_device)
+    o = _call(ck, d)
+    assert o.dtype == torch.float32
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+
+
+def test_varlen_equals_per_document_oracle(gpu_device):
+    ck, _ = _ops()
+    H, dk, dv = 2, 64, 64
+    cu = [0, 1, 65, 129, 130, 330, 400]
+    T, N = cu[-1], len(cu) - 1
+    inp = hp.rounded(po.make_inputs(1, T, H, dk, dv, seed=7), torch.bfloat16)
+    gen = torch.Generator().manual_seed(3)
+    mu0 = torch.randn(N, H, dv, dk, generator=gen) * 0.1
+    I0 = 1.0 + torch.rand(N, H, dv, dk, generator=gen)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0, I0=I0, cu=cu)
+    d = hp.to_device(inp, gpu_device)
+    o, mu, I = _call(ck, d, initial_mu_state=mu0.to(gpu_device), initial_I_state=I0.to(gpu_device),
+                     output_final_state=True, cu_seqlens=torch.tensor(cu, device=gpu_device))
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL
+    assert hp.max_rel(I, I_ref) <= STATE_REL_TOL
+    # no initial state: every document restarts from (0, Ip)
+    o_ref2, _, _, _ = hp.oracle_forward(inp, cu=cu)
+    o2 = _call(ck, d, cu_seqlens=torch.tensor(cu, device=gpu_device))
+    assert hp.max_abs(o2, o_ref2) <= hp.BF16_OUT_ABS_TOL
+
+
+def test_c1_shape_subset_against_oracle_and_full_against_recurrent(gpu_device):
+    """Config 1 (B=8,T=2048,H=12,d=64,bf16): the oracle checks a (batch, head) subset at full T
+    (entries are independent); the whole tensor is checked against the fp32-state recurrent kernel."""
+    ck, fr = _ops()
+    inp = hp.rounded(po.make_inputs(8, 2048, 12, 64, 64, seed=0), torch.bfloat16)
+    d = hp.to_device(inp, gpu_device)
+    o, mu, I = _call(ck, d, output_final_state=True, chunk_size=64)
+    o_r, mu_r, I_r = _call(fr, d, output_final_state=True)
+    assert hp.max_abs(o.float(), o_r.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_r) <= STATE_REL_TOL
+    assert hp.max_rel(I, I_r) <= STATE_REL_TOL
+    bs, hs = [0, 5], [1, 7, 11]
+    sub = {n: inp[n][bs][:, :, hs] for n in ("q", "k", "v", "b", "gt")}
+    sub["g"], sub["Ip"] = inp["g"][hs], inp["Ip"][hs]
+    o_ref, _, _, _ = hp.oracle_forward(sub)
+    assert hp.max_abs(o[bs][:, :, hs], o_ref) <= hp.BF16_OUT_ABS_TOL
+
+
+def test_error_paths_match_reference(gpu_device):
+    ck, _ = _ops()
+    inp = hp.to_device(po.make_inputs(2, 8, 2, 16, 16, seed=0), gpu_device)
+    with pytest.raises(ValueError):
+        _call(ck, inp, cu_seqlens=torch.tensor([0, 8], device=gpu_device))
