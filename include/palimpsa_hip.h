@@ -159,6 +159,18 @@ size_t pal_chunk_bwd_workspace_bytes(const PalDims *dims);
 int pal_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------------------ measurement */
+
+/* Per-kernel timing aid; no counterpart in the reference.  While enabled, every
+ * kernel launch of the library is bracketed by two HIP events on the launch
+ * stream; pal_profile_read waits for the outstanding ones and returns the
+ * accumulated time and launch count of one kernel.  Process-global, for
+ * benchmarks only (not thread-safe while enabled). */
+int pal_profile_enable(int on);               /* also resets the counters */
+int pal_profile_kernel_count(void);
+const char *pal_profile_kernel_name(int kernel_id);
+int pal_profile_read(int kernel_id, double *total_ms, int64_t *launches);
+
 #ifdef __cplusplus
 }
 #endif

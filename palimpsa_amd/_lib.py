@@ -84,6 +84,14 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_size_t
         fn.argtypes = [P(PalDims)]
+    lib.pal_profile_enable.restype = C.c_int
+    lib.pal_profile_enable.argtypes = [C.c_int]
+    lib.pal_profile_kernel_count.restype = C.c_int
+    lib.pal_profile_kernel_count.argtypes = []
+    lib.pal_profile_kernel_name.restype = C.c_char_p
+    lib.pal_profile_kernel_name.argtypes = [C.c_int]
+    lib.pal_profile_read.restype = C.c_int
+    lib.pal_profile_read.argtypes = [C.c_int, P(C.c_double), P(C.c_int64)]
     if lib.pal_abi_version() != PAL_ABI_VERSION:
         raise ImportError(f"{LIB_PATH}: ABI version {lib.pal_abi_version()} != expected {PAL_ABI_VERSION}; rebuild")
     _lib = lib
@@ -122,3 +130,20 @@ def build_chunk_table(cu_seqlens_host):
     if rc < 0:
         check(rc, "pal_build_chunk_table")
     return table[:total], offsets
+
+
+def profile_enable(on: bool) -> None:
+    """Switch the library's per-kernel HIP-event timing on or off (resets the counters)."""
+    load().pal_profile_enable(1 if on else 0)
+
+
+def profile_read():
+    """{kernel name: (total_ms, launches)} for every kernel launched since profile_enable(True)."""
+    lib = load()
+    out = {}
+    for i in range(lib.pal_profile_kernel_count()):
+        ms, n = C.c_double(0.0), C.c_int64(0)
+        lib.pal_profile_read(i, C.byref(ms), C.byref(n))
+        if n.value:
+            out[lib.pal_profile_kernel_name(i).decode()] = (ms.value, n.value)
+    return out

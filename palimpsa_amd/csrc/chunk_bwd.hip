@@ -1,0 +1,825 @@
+// Chunked Palimpsa backward.
+//
+// Replaces chunk_palimpsa_bwd_kernel and the host-side reductions of
+// ChunkPalimpsa.backward (chunk_palimpsa_forgetting_scalar.py:239-434, :519-620).
+//
+// With G_t = scale do_t q_t^T, the per-token local gradients are
+//   dMloc_t = G_t / I_t,  dJloc_t = -G_t M_t / I_t^2 (- scale dovar_t (q_t*q_t)^T / I_t^2)
+// and the state gradients obey the reverse recurrence dM_s = dMloc_s + f_{s+1} dM_{s+1}
+// (:360-384).  All tiles of 64 tokens are processed in parallel; what crosses a
+// tile boundary is handled by two small extra passes:
+//
+//  local   per (tile, head): recompute M_t, I_t from the tile-start state (as the
+//          forward does), form dMloc/dJloc, dq; feed them straight from the MFMA
+//          accumulators into the reverse contraction dM^loc = L^T dMloc (k index =
+//          token, so accumulator registers are already in operand layout); from it
+//          the tile-local parts of dv, db, dk and the carry the tile hands to its
+//          predecessor, R_loc = f_first * dM^loc_first.
+//  scan    per state entry: R_{c-1} = R_loc,c + F_C,c R_c backwards over the tiles
+//          of a sequence (the role of curr_dM/curr_dI, :429-430); also yields the
+//          gradients of the initial state.
+//  apply   per (tile, head): adds the carry terms a_s R k_s etc. to dv, db, dk
+//          with four small MFMA products.
+//  gate    d log f_s = <dM_s, f_s M_{s-1}> + <dJ_s, f_s J_{s-1}>, evaluated without any
+//          cancellation (the reference un-shifts the state by dividing by f, :409-412):
+//            local part   gamma_s = <dM^loc_s, S_s> + <dJ^loc_s, S^J_s>, S_s = f_s M_{s-1} from a
+//                         strictly-lower-triangular MFMA product in the layout of dM^loc;
+//            carry part   sum_{r<s, r in tile} beta_r + F_C (<R_M, M_0> + <R_J, J_0>), with
+//                         beta_r = <v_r, dv^carry_r> + <b_r, db^carry_r> from the apply pass and
+//                         (M_0, J_0) the state at the start of the tile.
+//          dgt = -g dlogf, dg = -sum gt dlogf, dIp = sum dJloc (- sum dJ_0 with an initial state).
+#include "chunk_common.h"
+#include "pal_host.h"
+#include "pal_profile.h"
+
+namespace pal {
+
+void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t);
+
+struct BwdArgs {
+  ChunkArgs c;
+  const void *d_o, *d_o_var;
+  void *dq, *dk, *dv, *db;
+  float *dgt, *dg, *dIp, *d_init_mu, *d_init_I;
+  float *wDM, *wDJ;       // [total_chunks,H,dv,dk] local carries, then incoming carries
+  float* wFtot;           // [total_chunks,H] log2 of the total decay of a tile
+  float* wSig;            // [total_chunks,H] sum over the tile of dJloc
+  float* wBnd;            // [total_chunks,H] F_C <carry, state at the start of the tile>
+  float* wE;              // [H, tokens]  local part of d log f
+  float* wBc;             // [H, tokens]  beta_r of the carry terms
+  float* wInitPart;       // [n_seqs,H,dv*dk/256] partial sums of dJ_0
+  double *wDgPart, *wDIpPart;  // [n_seqs,H]
+  int32_t tokens;
+};
+
+constexpr int kVS2 = 68;
+constexpr int kDG2 = 16;
+
+__device__ __forceinline__ constexpr int lidx2(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
+__device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2 * sb + p : 4 + (sb - 2); }
+
+// ---------------------------------------------------------------- local pass
+template <typename TIn, int NB, bool HAS_VAR>
+__global__ __launch_bounds__(NB * 64) void chunk_bwd_local_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  extern __shared__ float smem[];
+  constexpr int NST = HAS_VAR ? 4 : 3;  // staged tensors: v, b, do, (dovar)
+  constexpr int NT = NB * 64;
+  constexpr int STG = kDG2 * kVS2;
+  constexpr int NITEM = (kC * kDG2 / 4 + NT - 1) / NT;
+  float* sC = smem;                      // [64] running log2 decay
+  float* sF = sC + kC;                   // [64] 2^c
+  float* sSt = sF + kC;                  // [2][NST][16][kVS2]
+  float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
+  float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
+  float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [NB] sums of dJloc
+  const int tid = threadIdx.x, lane = tid & 63, nb = tid >> 6, i = lane & 15, g = lane >> 4;
+  const int H = a.H, dk = a.dk, dv = a.dv;
+  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  const float Ip = a.Ip[h];
+  const float gh = a.g[h] * kLog2e;
+  const float scale = a.scale;
+
+  if (nb == 0) {
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    const float c = wave_inclusive_scan(-gt * gh, lane);
+    sC[lane] = c;
+    sF[lane] = fast_exp2(c);
+    if (lane == 63) A.wFtot[(int64_t)cidx * H + h] = c;
+  }
+  const int64_t row0 = ((int64_t)t0 * H + h) * dv;
+  const TIn* vp = (const TIn*)a.v + row0;
+  const TIn* bp = (const TIn*)a.b + row0;
+  const TIn* dop = (const TIn*)A.d_o + row0;
+  float st[NST][NITEM][4];
+  auto stage_load = [&](int dg) {
+#pragma unroll
+    for (int it = 0; it < NITEM; ++it) {
+      const int idx = tid + it * NT;
+      const int s = idx >> 2, dq4 = idx & 3;
+      if (idx < kC * kDG2 / 4 && s < clen) {
+        const int64_t off = (int64_t)s * H * dv + dg * kDG2 + 4 * dq4;
+        load_vec<4>(vp + off, st[0][it]);
+        load_vec<4>(bp + off, st[1][it]);
+        load_vec<4>(dop + off, st[2][it]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st[2][it][e] *= scale;
+        if (HAS_VAR) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) st[NST - 1][it][e] = scale * load_rt(A.d_o_var, row0 + off + e, a.var_bf16);
+        }
+      } else {
+#pragma unroll
+        for (int x = 0; x < NST; ++x)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) st[x][it][e] = 0.f;
+      }
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int it = 0; it < NITEM; ++it) {
+      const int idx = tid + it * NT;
+      const int s = idx >> 2, dq4 = idx & 3;
+      if (idx < kC * kDG2 / 4) {
+#pragma unroll
+        for (int x = 0; x < NST; ++x)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * dq4 + e) * kVS2 + s] = st[x][it][e];
+      }
+    }
+  };
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+
+  // ---- per-wave constants of this tile
+  bf16x8 Lr[6], Lrev[6], Ls[6];
+  float kA[2][8], kk[2][8];
+  {
+    float ct[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) ct[tb] = sC[16 * tb + i];
+    const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      float cs[8];
+      *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
+      *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int s = 8 * g + j + 32 * ks;
+        const bool ok = s < clen;
+        const float kv = to_f32(kp[(int64_t)(ok ? s : 0) * H * dk]);
+        kA[ks][j] = ok ? kv : 0.f;
+        kk[ks][j] = kA[ks][j] * kA[ks][j];
+#pragma unroll
+        for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
+          const int t = 16 * tb + i;
+          const float lv = fast_exp2(ct[tb] - cs[j]);
+          Lr[lidx2(tb, ks)][j] = (bf16_t)((s <= t) ? lv : 0.f);
+          Ls[lidx2(tb, ks)][j] = (bf16_t)((s < t) ? lv : 0.f);   // same (i,g,j) roles with s,t swapped in name
+        }
+      }
+    }
+    // reverse operand: column s = 16sb + i, k index (g,j) <-> token t = 16(2p + j/4) + 4g + j%4
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      float ctt[8];
+      *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * p + 4 * g];
+      *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * p + 16 + 4 * g];
+#pragma unroll
+      for (int sb = 0; sb < (p ? 4 : 2); ++sb) {
+        const int s = 16 * sb + i;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int t = 16 * (2 * p + (j >> 2)) + 4 * g + (j & 3);
+          Lrev[ridx(sb, p)][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sb]) : 0.f);
+        }
+      }
+    }
+  }
+  float qP[4][4], kB[4][4];
+  {
+    const TIn* qp = (const TIn*)a.q + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
+    const TIn* kp4 = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + 4 * g;
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 16 * tb + 4 * g + r;
+        const bool ok = t < clen;
+        const float qv = to_f32(qp[(int64_t)(ok ? t : 0) * H * dk]);
+        qP[tb][r] = ok ? qv : 0.f;
+      }
+      const int s = 16 * tb + i;
+      if (s < clen) {
+        load_vec<4>(kp4 + (int64_t)s * H * dk, kB[tb]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) kB[tb][r] = 0.f;
+      }
+    }
+  }
+  float dqa[4][4], dkM[4][4], dkJ[4][4], gam[4], FsB[4];
+  float sigacc = 0.f;
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    gam[x] = 0.f;
+    FsB[x] = sF[16 * x + i];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { dqa[x][r] = 0.f; dkM[x][r] = 0.f; dkJ[x][r] = 0.f; }
+  }
+
+  const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
+  const float* cmu = a.chunk_mu + tile_off + 16 * nb + i;
+  const float* cI = a.chunk_I + tile_off + 16 * nb + i;
+  const float* cmuT = a.chunk_mu + tile_off + 16 * nb + 4 * g;   // same state, 4 key columns per lane group
+  const float* cIT = a.chunk_I + tile_off + 16 * nb + 4 * g;
+  float* wDM = A.wDM + tile_off + 16 * nb + 4 * g;
+  float* wDJ = A.wDJ + tile_off + 16 * nb + 4 * g;
+  const float f_first = fast_exp2(sC[0]);
+
+  const int n_groups = dv / kDG2;
+  for (int dg = 0; dg < n_groups; ++dg) {
+    const int buf = dg & 1;
+    const float* sV = sSt + (buf * NST + 0) * STG;
+    const float* sB = sSt + (buf * NST + 1) * STG;
+    const float* sDo = sSt + (buf * NST + 2) * STG;
+    const float* sDov = sSt + (buf * NST + NST - 1) * STG;
+    if (dg + 1 < n_groups) stage_load(dg + 1);
+    for (int dd = 0; dd < kDG2; ++dd) {
+      const int d = dg * kDG2 + dd;
+      const float mu0 = cmu[(int64_t)d * dk];
+      const float I0 = cI[(int64_t)d * dk];
+      const float M0 = mu0 * I0, J0 = I0 - Ip;
+      const f32x4 muT = *(const f32x4*)(cmuT + (int64_t)d * dk);
+      const f32x4 IT = *(const f32x4*)(cIT + (int64_t)d * dk);
+      bf16x8 XM[2], XJ[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const f32x4 v0 = *(const f32x4*)&sV[dd * kVS2 + 8 * g + 32 * ks];
+        const f32x4 v1 = *(const f32x4*)&sV[dd * kVS2 + 8 * g + 32 * ks + 4];
+        const f32x4 b0 = *(const f32x4*)&sB[dd * kVS2 + 8 * g + 32 * ks];
+        const f32x4 b1 = *(const f32x4*)&sB[dd * kVS2 + 8 * g + 32 * ks + 4];
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
+          const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
+          const bf16x2 pm = pack2(kA[ks][j] * va, kA[ks][j + 1] * vb);
+          const bf16x2 pj = pack2(kk[ks][j] * ba, kk[ks][j + 1] * bb);
+          XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
+          XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
+        }
+      }
+      // ---- phase A: states of this value row for all 64 tokens, local gradients
+      bf16x8 PM[2], PJ[2];
+#pragma unroll
+      for (int tb = 0; tb < 4; ++tb) {
+        f32x4 accM = {0.f, 0.f, 0.f, 0.f};
+        f32x4 accI = {Ip, Ip, Ip, Ip};
+        accM = mfma16(Lr[lidx2(tb, 0)], XM[0], accM);
+        accI = mfma16(Lr[lidx2(tb, 0)], XJ[0], accI);
+        if (tb >= 2) {
+          accM = mfma16(Lr[lidx2(tb, 1)], XM[1], accM);
+          accI = mfma16(Lr[lidx2(tb, 1)], XJ[1], accI);
+        }
+        const f32x4 Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
+        const f32x4 dov = *(const f32x4*)&sDo[dd * kVS2 + 16 * tb + 4 * g];
+        f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
+        if (HAS_VAR) dvv = *(const f32x4*)&sDov[dd * kVS2 + 16 * tb + 4 * g];
+        float dMl[4], dJl[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float Mf = fmaf(Fv[r], M0, accM[r]);
+          const float If = fmaf(Fv[r], J0, accI[r]);
+          const float rI = fast_rcp(If);
+          const float mu = Mf * rI;
+          const float q = qP[tb][r];
+          dMl[r] = (dov[r] * q) * rI;
+          dJl[r] = -(dMl[r] * mu);
+          dqa[tb][r] = fmaf(mu, dov[r], dqa[tb][r]);
+          if (HAS_VAR) {
+            const float wq = dvv[r] * q;          // scale*dovar*q
+            const float w = wq * q * rI;          // scale*dovar*q^2/I
+            dJl[r] = fmaf(-w, rI, dJl[r]);
+            dqa[tb][r] = fmaf(2.f * wq, rI, dqa[tb][r]);
+          }
+          sigacc += dJl[r];
+        }
+        const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
+        const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
+        const int o4 = (tb & 1) * 4;
+        PM[tb >> 1][o4 + 0] = m0[0]; PM[tb >> 1][o4 + 1] = m0[1]; PM[tb >> 1][o4 + 2] = m1[0]; PM[tb >> 1][o4 + 3] = m1[1];
+        PJ[tb >> 1][o4 + 0] = j0[0]; PJ[tb >> 1][o4 + 1] = j0[1]; PJ[tb >> 1][o4 + 2] = j1[0]; PJ[tb >> 1][o4 + 3] = j1[1];
+      }
+      // ---- phase B: dM^loc[n, s] = sum_t dMloc[t, n] L[t, s], accumulators -> operands directly
+#pragma unroll
+      for (int sb = 0; sb < 4; ++sb) {
+        f32x4 aM = {0.f, 0.f, 0.f, 0.f}, aJ = {0.f, 0.f, 0.f, 0.f};
+        if (sb < 2) {
+          aM = mfma16(PM[0], Lrev[ridx(sb, 0)], aM);
+          aJ = mfma16(PJ[0], Lrev[ridx(sb, 0)], aJ);
+        }
+        aM = mfma16(PM[1], Lrev[ridx(sb, 1)], aM);
+        aJ = mfma16(PJ[1], Lrev[ridx(sb, 1)], aJ);
+        // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
+        f32x4 sM = {0.f, 0.f, 0.f, 0.f}, sJ = {0.f, 0.f, 0.f, 0.f};
+        sM = mfma16(XM[0], Ls[lidx2(sb, 0)], sM);
+        sJ = mfma16(XJ[0], Ls[lidx2(sb, 0)], sJ);
+        if (sb >= 2) {
+          sM = mfma16(XM[1], Ls[lidx2(sb, 1)], sM);
+          sJ = mfma16(XJ[1], Ls[lidx2(sb, 1)], sJ);
+        }
+        const float vS = sV[dd * kVS2 + 16 * sb + i];
+        const float bS = sB[dd * kVS2 + 16 * sb + i];
+        float dvp = 0.f, dbp = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float kv = kB[sb][r];
+          dvp = fmaf(aM[r], kv, dvp);
+          dbp = fmaf(aJ[r] * kv, kv, dbp);
+          dkM[sb][r] = fmaf(aM[r], vS, dkM[sb][r]);
+          dkJ[sb][r] = fmaf(aJ[r], bS, dkJ[sb][r]);
+          const float Ss = fmaf(FsB[sb], muT[r] * IT[r], sM[r]);
+          const float SJ = fmaf(FsB[sb], IT[r] - Ip, sJ[r]);
+          gam[sb] = fmaf(aM[r], Ss, gam[sb]);
+          gam[sb] = fmaf(aJ[r], SJ, gam[sb]);
+        }
+        dvp = rows4_sum(dvp);
+        dbp = rows4_sum(dbp);
+        if (g == 0) {
+          sPv[(nb * kDG2 + dd) * kC + 16 * sb + i] = dvp;
+          sPb[(nb * kDG2 + dd) * kC + 16 * sb + i] = dbp;
+        }
+        if (sb == 0 && i == 0) {
+          // carry handed to the previous tile: f_first * dM^loc at the first token
+          const f32x4 rm = {f_first * aM[0], f_first * aM[1], f_first * aM[2], f_first * aM[3]};
+          const f32x4 rj = {f_first * aJ[0], f_first * aJ[1], f_first * aJ[2], f_first * aJ[3]};
+          *(f32x4*)(wDM + (int64_t)d * dk) = rm;
+          *(f32x4*)(wDJ + (int64_t)d * dk) = rj;
+        }
+      }
+    }
+    __syncthreads();
+    // flush the tile-local dv, db of this group; work item = (token s, 4 value rows)
+#pragma unroll
+    for (int it = 0; it < NITEM; ++it) {
+      const int idx = tid + it * NT;
+      const int s = idx >> 2, dq4 = idx & 3;
+      if (idx < kC * kDG2 / 4 && s < clen) {
+        const int64_t off = row0 + (int64_t)s * H * dv + dg * kDG2 + 4 * dq4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float sv = 0.f, sb_ = 0.f;
+#pragma unroll
+          for (int w = 0; w < NB; ++w) {
+            sv += sPv[(w * kDG2 + 4 * dq4 + e) * kC + s];
+            sb_ += sPb[(w * kDG2 + 4 * dq4 + e) * kC + s];
+          }
+          ((TIn*)A.dv)[off + e] = from_f32<TIn>(sv);
+          ((TIn*)A.db)[off + e] = from_f32<TIn>(sb_);
+        }
+      }
+    }
+    if (dg + 1 < n_groups) stage_store((dg + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- tile end: dq (final), tile-local dk
+  {
+    TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
+    TIn* dkp = (TIn*)A.dk + ((int64_t)t0 * H + h) * dk + 16 * nb + 4 * g;
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 16 * tb + 4 * g + r;
+        if (t < clen) dqp[(int64_t)t * H * dk] = from_f32<TIn>(dqa[tb][r]);
+      }
+      const int s = 16 * tb + i;
+      if (s < clen) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          dkp[(int64_t)s * H * dk + r] = from_f32<TIn>(fmaf(2.f * kB[tb][r], dkJ[tb][r], dkM[tb][r]));
+      }
+    }
+  }
+  // ---- local part of d log f per token, tile sum of dJloc
+#pragma unroll
+  for (int sb = 0; sb < 4; ++sb) {
+    const float x = rows4_sum(gam[sb]);
+    if (g == 0) sRed[nb * kC + 16 * sb + i] = x;
+  }
+  {
+    const float x = wave_sum(sigacc);
+    if (lane == 0) sRed[NB * kC + nb] = x;
+  }
+  __syncthreads();
+  if (tid < kC) {
+    float gm = 0.f;
+#pragma unroll
+    for (int w = 0; w < NB; ++w) gm += sRed[w * kC + tid];
+    if (tid < clen) A.wE[(int64_t)h * A.tokens + t0 + tid] = gm;
+    if (tid == 0) {
+      float sg = 0.f;
+#pragma unroll
+      for (int w = 0; w < NB; ++w) sg += sRed[NB * kC + w];
+      A.wSig[(int64_t)cidx * H + h] = sg;
+    }
+  }
+}
+
+// ----------------------------------------------------------------- carry scan
+// one thread per (sequence, head, state entry); 256 consecutive entries per block
+__global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  __shared__ float sW[4];
+  const int64_t E = (int64_t)a.dv * a.dk;
+  const int nblk = (int)(E / 256);
+  const int blk = blockIdx.x % nblk;
+  const int nh = blockIdx.x / nblk;
+  const int h = nh % a.H, n = nh / a.H;
+  const int64_t e = (int64_t)blk * 256 + threadIdx.x;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const int nchunks = (len + kC - 1) / kC;
+  float RM = 0.f, RJ = 0.f;
+  for (int c = nchunks - 1; c >= 0; --c) {
+    const int64_t off = ((int64_t)(cbase + c) * a.H + h) * E + e;
+    const float DM = A.wDM[off], DJ = A.wDJ[off];
+    const float Ft = fast_exp2(A.wFtot[(int64_t)(cbase + c) * a.H + h]);
+    A.wDM[off] = RM;
+    A.wDJ[off] = RJ;
+    RM = fmaf(Ft, RM, DM);
+    RJ = fmaf(Ft, RJ, DJ);
+  }
+  if (a.init_mu) {
+    const int64_t so = (int64_t)nh * E + e;
+    if (A.d_init_mu) {
+      const float mu0 = a.init_mu[so], I0 = a.init_I[so];
+      A.d_init_mu[so] = RM * I0;
+      A.d_init_I[so] = fmaf(RM, mu0, RJ);
+    }
+    // J_0 = I_0 - Ip: the prior also receives -sum dJ_0
+    float s = wave_sum(RJ);
+    if ((threadIdx.x & 63) == 0) sW[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) A.wInitPart[(int64_t)nh * nblk + blk] = sW[0] + sW[1] + sW[2] + sW[3];
+  }
+}
+
+// ---------------------------------------------------------------- carry apply
+// dv_s += a_s R_M k_s ; db_s += a_s R_J k_s^2 ; dk_s += a_s (R_M^T v_s + 2 k_s * R_J^T b_s)
+template <typename TIn>
+__global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  __shared__ float sAs[kC];
+  __shared__ float sBt[kC];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
+  const int H = a.H, dk = a.dk, dv = a.dv;
+  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  int bos, len, cbase;
+  seq_lookup(a, seq, bos, len, cbase);
+  const bool last = cis == (len + kC - 1) / kC - 1;
+  if (last) {  // nothing flows in from beyond the end of the sequence (uniform for the block)
+    if (tid == 0) A.wBnd[(int64_t)cidx * H + h] = 0.f;
+    if (tid < clen) A.wBc[(int64_t)h * A.tokens + t0 + tid] = 0.f;
+    return;
+  }
+  const float gh = a.g[h] * kLog2e;
+  __shared__ float sW4[5];
+  if (w == 0) {
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    const float c = wave_inclusive_scan(-gt * gh, lane);
+    const float tot = __shfl(c, 63);
+    sAs[lane] = fast_exp2(tot - c);
+    if (lane == 0) sW4[4] = fast_exp2(tot);
+  }
+  {
+    // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile
+    const int64_t E = (int64_t)dv * dk;
+    const float* rm = A.wDM + ((int64_t)cidx * H + h) * E;
+    const float* rj = A.wDJ + ((int64_t)cidx * H + h) * E;
+    const float* smu = a.chunk_mu + ((int64_t)cidx * H + h) * E;
+    const float* sI = a.chunk_I + ((int64_t)cidx * H + h) * E;
+    const float Ipb = a.Ip[h];
+    float acc = 0.f;
+    for (int64_t e = tid; e < E; e += 256) {
+      const float I = sI[e];
+      acc = fmaf(rm[e], smu[e] * I, acc);
+      acc = fmaf(rj[e], I - Ipb, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) sW4[w] = acc;
+  }
+  __syncthreads();
+  if (tid == 0) A.wBnd[(int64_t)cidx * H + h] = sW4[4] * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);
+  const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
+  const float* RM = A.wDM + tile_off;
+  const float* RJ = A.wDJ + tile_off;
+  const int srow = 16 * w + i;            // operand row (token) of this lane
+  const bool row_ok = srow < clen;
+  const float as = sAs[srow];
+  const int64_t tokA = ((int64_t)(t0 + (row_ok ? srow : 0)) * H + h);
+  float beta4[4] = {0.f, 0.f, 0.f, 0.f};
+
+  // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
+  {
+    const int KS = (dk + 31) / 32;
+    bf16x8 A1[8], A2[8];
+    const TIn* kp = (const TIn*)a.k + tokA * dk;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks < KS) {
+        const int n0 = 8 * g + 32 * ks;
+        float kv[8];
+        if (row_ok && n0 < dk) {
+          load_vec<4>(kp + n0, kv);
+          load_vec<4>(kp + n0 + 4, kv + 4);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) kv[j] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          A1[ks][j] = (bf16_t)(as * kv[j]);
+          A2[ks][j] = (bf16_t)(as * kv[j] * kv[j]);
+        }
+      }
+    }
+    TIn* dvo = (TIn*)A.dv;
+    TIn* dbo = (TIn*)A.db;
+    const TIn* vin = (const TIn*)a.v;
+    const TIn* bin = (const TIn*)a.b;
+    for (int db_ = 0; db_ < dv / 16; ++db_) {
+      f32x4 accV = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks < KS) {
+          const int n0 = 8 * g + 32 * ks;
+          bf16x8 B1, B2;
+          if (n0 < dk) {
+            const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
+            const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
+            const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
+            const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
+              B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { B1[j] = (bf16_t)0.f; B2[j] = (bf16_t)0.f; }
+          }
+          accV = mfma16(A1[ks], B1, accV);
+          accB = mfma16(A2[ks], B2, accB);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int s = 16 * w + 4 * g + r;
+        if (s < clen) {
+          const int64_t off = ((int64_t)(t0 + s) * H + h) * dv + 16 * db_ + i;
+          dvo[off] = from_f32<TIn>(to_f32(dvo[off]) + accV[r]);
+          dbo[off] = from_f32<TIn>(to_f32(dbo[off]) + accB[r]);
+          beta4[r] = fmaf(to_f32(vin[off]), accV[r], beta4[r]);
+          beta4[r] = fmaf(to_f32(bin[off]), accB[r], beta4[r]);
+        }
+      }
+    }
+  }
+  // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
+  {
+    const int KS = (dv + 31) / 32;
+    bf16x8 A3[8], A4[8];
+    const TIn* vp = (const TIn*)a.v + tokA * dv;
+    const TIn* bp = (const TIn*)a.b + tokA * dv;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks < KS) {
+        const int d0 = 8 * g + 32 * ks;
+        float vv[8], bb[8];
+        if (row_ok && d0 < dv) {
+          load_vec<4>(vp + d0, vv); load_vec<4>(vp + d0 + 4, vv + 4);
+          load_vec<4>(bp + d0, bb); load_vec<4>(bp + d0 + 4, bb + 4);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { vv[j] = 0.f; bb[j] = 0.f; }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          A3[ks][j] = (bf16_t)(as * vv[j]);
+          A4[ks][j] = (bf16_t)(as * bb[j]);
+        }
+      }
+    }
+    TIn* dko = (TIn*)A.dk;
+    const TIn* kin = (const TIn*)a.k;
+    for (int nbk = 0; nbk < dk / 16; ++nbk) {
+      f32x4 accM = {0.f, 0.f, 0.f, 0.f}, accJ = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks < KS) {
+          const int d0 = 8 * g + 32 * ks;
+          bf16x8 B3, B4;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const bool ok = d0 + j < dv;
+            const int64_t ro = (int64_t)(ok ? d0 + j : 0) * dk + 16 * nbk + i;
+            const float x = RM[ro], y = RJ[ro];
+            B3[j] = (bf16_t)(ok ? x : 0.f);
+            B4[j] = (bf16_t)(ok ? y : 0.f);
+          }
+          accM = mfma16(A3[ks], B3, accM);
+          accJ = mfma16(A4[ks], B4, accJ);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int s = 16 * w + 4 * g + r;
+        if (s < clen) {
+          const int64_t off = ((int64_t)(t0 + s) * H + h) * dk + 16 * nbk + i;
+          const float kv = to_f32(kin[off]);
+          dko[off] = from_f32<TIn>(to_f32(dko[off]) + accM[r] + 2.f * kv * accJ[r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float x = row16_sum(beta4[r]);
+    if (i == 0) sBt[16 * w + 4 * g + r] = x;
+  }
+  __syncthreads();
+  if (tid < clen) A.wBc[(int64_t)h * A.tokens + t0 + tid] = sBt[tid];
+}
+
+// ----------------------------------------------------------------- gate pass
+// one block per (sequence, head); a wave per tile: local part + prefix of the carry terms + boundary term
+__global__ __launch_bounds__(256) void chunk_bwd_gate_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  __shared__ double sG[4];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int h = blockIdx.x % a.H, n = blockIdx.x / a.H;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const float gh = a.g[h];
+  double dg_acc = 0.0;
+  const int nchunks = (len + kC - 1) / kC;
+  const int nseg = (len + 255) / 256;
+  for (int seg = 0; seg < nseg; ++seg) {
+    const int t = seg * 256 + tid;
+    const bool ok = t < len;
+    const float bc = ok ? A.wBc[(int64_t)h * A.tokens + bos + t] : 0.f;
+    const float pre = wave_inclusive_scan(bc, lane) - bc;   // carry terms of the earlier tokens of the tile
+    if (ok) {
+      const int tile = seg * 4 + w;
+      const float dlogf = A.wE[(int64_t)h * A.tokens + bos + t] + pre + A.wBnd[(int64_t)(cbase + tile) * a.H + h];
+      const float gt = load_gate(a.gt, (int64_t)(bos + t) * a.H + h, a.gate_bf16);
+      A.dgt[(int64_t)(bos + t) * a.H + h] = -gh * dlogf;
+      dg_acc -= (double)gt * (double)dlogf;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) dg_acc += __shfl_xor(dg_acc, off);
+  if (lane == 0) sG[w] = dg_acc;
+  __syncthreads();
+  if (tid == 0) {
+    A.wDgPart[(int64_t)n * a.H + h] = sG[0] + sG[1] + sG[2] + sG[3];
+    double s = 0.0;
+    for (int c = 0; c < nchunks; ++c) s += (double)A.wSig[(int64_t)(cbase + c) * a.H + h];
+    if (a.init_mu) {
+      const int nblk = (int)(((int64_t)a.dv * a.dk) / 256);
+      for (int b2 = 0; b2 < nblk; ++b2) s -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
+    }
+    A.wDIpPart[(int64_t)n * a.H + h] = s;
+  }
+}
+
+__global__ void chunk_bwd_head_reduce_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  const int h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= a.H) return;
+  double sg = 0.0, si = 0.0;
+  for (int n = 0; n < a.n_seqs; ++n) {
+    sg += A.wDgPart[(int64_t)n * a.H + h];
+    si += A.wDIpPart[(int64_t)n * a.H + h];
+  }
+  A.dg[h] = (float)sg;
+  A.dIp[h] = (float)si;
+}
+
+// ------------------------------------------------------------------- host
+struct BwdLayout {
+  size_t oDM, oDJ, oFtot, oSig, oBnd, oE, oBc, oInit, oDg, oDIp, total;
+};
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static BwdLayout bwd_layout(const PalDims* d) {
+  BwdLayout L;
+  const size_t E = (size_t)d->dv * d->dk;
+  const size_t tiles = (size_t)d->total_chunks * d->n_heads;
+  const size_t tokens = (size_t)d->batch * d->seq_len;
+  size_t o = 0;
+  L.oDM = o; o = align256(o + tiles * E * 4);
+  L.oDJ = o; o = align256(o + tiles * E * 4);
+  L.oFtot = o; o = align256(o + tiles * 4);
+  L.oSig = o; o = align256(o + tiles * 4);
+  L.oBnd = o; o = align256(o + tiles * 4);
+  L.oE = o; o = align256(o + tokens * d->n_heads * 4);
+  L.oBc = o; o = align256(o + tokens * d->n_heads * 4);
+  L.oInit = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * (E / 256) * 4);
+  L.oDg = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * 8);
+  L.oDIp = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * 8);
+  L.total = o;
+  return L;
+}
+
+template <typename TIn, int NB>
+static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
+  const bool var = A.c.flags & PAL_FLAG_HAS_VAR;
+  const int NT = NB * 64;
+  const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + NB);
+  const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
+  if (blocks > 0x7fffffff) return PAL_E_DIM;
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  if (var) {
+    if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, true>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+  } else {
+    if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, false>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+  }
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+template <typename TIn>
+static int launch_local(const BwdArgs& A, hipStream_t s) {
+  switch (A.c.dk / 16) {
+    case 1: return launch_local_nb<TIn, 1>(A, s);
+    case 2: return launch_local_nb<TIn, 2>(A, s);
+    case 3: return launch_local_nb<TIn, 3>(A, s);
+    case 4: return launch_local_nb<TIn, 4>(A, s);
+    case 5: return launch_local_nb<TIn, 5>(A, s);
+    case 6: return launch_local_nb<TIn, 6>(A, s);
+    case 7: return launch_local_nb<TIn, 7>(A, s);
+    case 8: return launch_local_nb<TIn, 8>(A, s);
+    case 9: return launch_local_nb<TIn, 9>(A, s);
+    case 10: return launch_local_nb<TIn, 10>(A, s);
+    case 11: return launch_local_nb<TIn, 11>(A, s);
+    case 12: return launch_local_nb<TIn, 12>(A, s);
+    case 13: return launch_local_nb<TIn, 13>(A, s);
+    case 14: return launch_local_nb<TIn, 14>(A, s);
+    case 15: return launch_local_nb<TIn, 15>(A, s);
+    case 16: return launch_local_nb<TIn, 16>(A, s);
+    default: return PAL_E_HEADDIM;
+  }
+}
+
+}  // namespace pal
+
+extern "C" size_t pal_chunk_bwd_workspace_bytes(const PalDims* d) {
+  if (pal_validate_dims(d) != PAL_OK || d->total_chunks <= 0) return 0;
+  return pal::bwd_layout(d).total;
+}
+
+extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const PalBwdTensors* gr, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  using namespace pal;
+  if (!d || !t) return PAL_E_NULL;
+  // the forward-side struct is reused with o pointing at any valid buffer; final states are not needed
+  PalDims dd = *d;
+  dd.flags &= ~PAL_FLAG_STORE_FINAL;
+  PalFwdTensors tt = *t;
+  tt.final_mu = tt.final_I = nullptr;
+  if (!tt.o) tt.o = gr ? (void*)gr->d_o : nullptr;
+  if ((dd.flags & PAL_FLAG_HAS_VAR) && !tt.o_var) tt.o_var = gr ? (void*)gr->d_o_var : nullptr;
+  int rc = check_chunk_common(&dd, &tt);
+  if (rc) return rc;
+  rc = check_bwd_common(&dd, gr);
+  if (rc) return rc;
+  const BwdLayout L = bwd_layout(&dd);
+  if (!workspace || workspace_bytes < L.total || !is_aligned16(workspace)) return PAL_E_WORKSPACE;
+  BwdArgs A;
+  fill_chunk_args(A.c, &dd, &tt);
+  A.d_o = gr->d_o;
+  A.d_o_var = (dd.flags & PAL_FLAG_HAS_VAR) ? gr->d_o_var : nullptr;
+  A.dq = gr->dq; A.dk = gr->dk; A.dv = gr->dv; A.db = gr->db;
+  A.dgt = gr->dgt; A.dg = gr->dg; A.dIp = gr->dIp;
+  A.d_init_mu = gr->d_init_mu; A.d_init_I = gr->d_init_I;
+  char* ws = (char*)workspace;
+  A.wDM = (float*)(ws + L.oDM); A.wDJ = (float*)(ws + L.oDJ);
+  A.wFtot = (float*)(ws + L.oFtot); A.wSig = (float*)(ws + L.oSig); A.wBnd = (float*)(ws + L.oBnd);
+  A.wE = (float*)(ws + L.oE); A.wBc = (float*)(ws + L.oBc); A.wInitPart = (float*)(ws + L.oInit);
+  A.wDgPart = (double*)(ws + L.oDg); A.wDIpPart = (double*)(ws + L.oDIp);
+  A.tokens = dd.batch * dd.seq_len;
+  hipStream_t s = (hipStream_t)stream;
+  const bool bf = dd.dtype == PAL_DTYPE_BF16;
+  rc = bf ? launch_local<bf16_t>(A, s) : launch_local<float>(A, s);
+  if (rc) return rc;
+  {
+    const int64_t blocks = (int64_t)dd.n_seqs * dd.n_heads * (((int64_t)dd.dv * dd.dk) / 256);
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    PAL_TIMED_LAUNCH(kKernBwdCarryScan, s, chunk_bwd_carry_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, A);
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  {
+    const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
+    if (bf) PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<bf16_t>), dim3(blocks), dim3(256), 0, s, A);
+    else PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<float>), dim3(blocks), dim3(256), 0, s, A);
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads)), dim3(256), 0, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((dd.n_heads + 63) / 64), dim3(64), 0, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}

@@ -17,6 +17,7 @@
 //      sum over n stays inside a lane.
 #include "chunk_common.h"
 #include "pal_host.h"
+#include "pal_profile.h"
 
 namespace pal {
 
@@ -348,8 +349,14 @@ static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
   const size_t lds = sizeof(float) * (kC + 2 * kDG * kVS + (var ? 2 : 1) * NB * kDG * kC);
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
-  if (var) hipLaunchKernelGGL((chunk_out_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
-  else hipLaunchKernelGGL((chunk_out_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  if (var) {
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
+  } else {
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
+  }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
@@ -406,8 +413,8 @@ extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* str
   hipStream_t s = (hipStream_t)stream;
   const int64_t waves = (int64_t)d->n_seqs * d->n_heads * (d->dv / 16) * (d->dk / 16);
   if (waves > 0x7fffffff) return PAL_E_DIM;
-  if (d->dtype == PAL_DTYPE_BF16) hipLaunchKernelGGL((chunk_state_kernel<bf16_t>), dim3((unsigned)waves), dim3(64), 0, s, a);
-  else hipLaunchKernelGGL((chunk_state_kernel<float>), dim3((unsigned)waves), dim3(64), 0, s, a);
+  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_state_kernel<bf16_t>), dim3((unsigned)waves), dim3(64), 0, s, a);
+  else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_state_kernel<float>), dim3((unsigned)waves), dim3(64), 0, s, a);
   PAL_HIP_LAUNCH_CHECK();
   if (d->dtype == PAL_DTYPE_BF16) return launch_out<bf16_t>(a, s);
   return launch_out<float>(a, s);

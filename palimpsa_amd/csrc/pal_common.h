@@ -127,6 +127,15 @@ __device__ __forceinline__ bf16x2 pack2(float lo, float hi) {
     if (e__ != hipSuccess) return (int)e__;    \
   } while (0)
 
+// LDS of one gfx950 compute unit; a launch asking for more than 64 KiB of dynamic
+// LDS has to raise the kernel's limit first.
+constexpr size_t kMaxLds = 160 * 1024;
+inline int allow_lds(const void* kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  return e == hipSuccess ? 0 : (int)e;
+}
+
 inline bool is_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
 }  // namespace pal

@@ -1,0 +1,77 @@
+// Per-kernel timing aid: when enabled, every kernel launch of the library is
+// bracketed by two HIP events on the launch stream.  Meant for benchmarks; it
+// keeps process-global state and is not thread-safe while enabled.
+#include <mutex>
+#include <vector>
+
+#include "pal_common.h"
+#include "pal_profile.h"
+
+namespace pal {
+
+static bool g_on = false;
+static std::mutex g_mu;
+struct Pair { int id; hipEvent_t a, b; };
+static std::vector<Pair> g_pending;
+static double g_ms[kKernCount];
+static long long g_n[kKernCount];
+
+ProfScope::ProfScope(int id_, hipStream_t s_) : id(id_), s(s_), e0(nullptr), on(g_on) {
+  if (!on) return;
+  if (hipEventCreate(&e0) != hipSuccess) { on = false; return; }
+  (void)hipEventRecord(e0, s);
+}
+ProfScope::~ProfScope() {
+  if (!on) return;
+  hipEvent_t e1;
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return; }
+  (void)hipEventRecord(e1, s);
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_pending.push_back({id, e0, e1});
+}
+
+static void drain() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  for (auto& p : g_pending) {
+    float ms = 0.f;
+    if (hipEventSynchronize(p.b) == hipSuccess && hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+      g_ms[p.id] += ms;
+      g_n[p.id] += 1;
+    }
+    (void)hipEventDestroy(p.a);
+    (void)hipEventDestroy(p.b);
+  }
+  g_pending.clear();
+}
+
+static const char* kNames[kKernCount] = {
+    "recurrent_fwd_kernel", "chunk_state_kernel", "chunk_out_kernel", "chunk_bwd_local_kernel",
+    "chunk_bwd_carry_scan_kernel", "chunk_bwd_carry_apply_kernel", "chunk_bwd_gate_kernel",
+    "chunk_bwd_head_reduce_kernel", "recurrent_bwd_state_kernel", "recurrent_bwd_kernel"};
+
+}  // namespace pal
+
+extern "C" {
+
+int pal_profile_enable(int on) {
+  pal::drain();
+  for (int i = 0; i < pal::kKernCount; ++i) { pal::g_ms[i] = 0.0; pal::g_n[i] = 0; }
+  pal::g_on = on != 0;
+  return PAL_OK;
+}
+
+int pal_profile_kernel_count(void) { return pal::kKernCount; }
+
+const char* pal_profile_kernel_name(int id) {
+  return (id >= 0 && id < pal::kKernCount) ? pal::kNames[id] : "";
+}
+
+int pal_profile_read(int id, double* total_ms, int64_t* launches) {
+  if (id < 0 || id >= pal::kKernCount || !total_ms || !launches) return PAL_E_DIM;
+  pal::drain();
+  *total_ms = pal::g_ms[id];
+  *launches = pal::g_n[id];
+  return PAL_OK;
+}
+
+}  // extern "C"

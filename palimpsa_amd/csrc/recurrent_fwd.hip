@@ -15,6 +15,7 @@
 // up front as 16-byte vectors that are contiguous across the row.
 #include "pal_common.h"
 #include "pal_host.h"
+#include "pal_profile.h"
 
 namespace pal {
 
@@ -181,8 +182,8 @@ template <typename TIn, int NPL>
 static int launch_npl(const RecArgs& a, int rd, hipStream_t s) {
   const int64_t blocks = (int64_t)a.n_seqs * a.H * (a.dv / (4 * rd));
   if (blocks > 0x7fffffff) return PAL_E_DIM;
-  if (rd == 4) hipLaunchKernelGGL((recurrent_fwd_kernel<TIn, NPL, 4>), dim3((unsigned)blocks), dim3(64), 0, s, a);
-  else hipLaunchKernelGGL((recurrent_fwd_kernel<TIn, NPL, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+  if (rd == 4) PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 4>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+  else PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }

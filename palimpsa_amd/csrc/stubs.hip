@@ -3,6 +3,4 @@
 extern "C" {
 size_t pal_recurrent_bwd_workspace_bytes(const PalDims*) { return 0; }
 int pal_recurrent_bwd(const PalDims*, const PalFwdTensors*, const PalBwdTensors*, void*, size_t, void*) { return PAL_E_WORKSPACE; }
-size_t pal_chunk_bwd_workspace_bytes(const PalDims*) { return 0; }
-int pal_chunk_bwd(const PalDims*, const PalFwdTensors*, const PalBwdTensors*, void*, size_t, void*) { return PAL_E_WORKSPACE; }
 }
