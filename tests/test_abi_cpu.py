@@ -1,0 +1,165 @@
+"""CPU-only checks of the C-ABI shared library: it loads, exports every symbol the header declares,
+rejects bad arguments before any HIP call, and the host-side chunk bookkeeping matches the oracle.
+No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import palimpsa_oracle as po
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "palimpsa_hip.h")
+
+
+@pytest.fixture(scope="module")
+def L():
+    from palimpsa_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from palimpsa_amd import build
+
+        build.build()
+    _lib.load()
+    return _lib
+
+
+def _declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(pal_[a-z_0-9]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol(L):
+    lib = L.load()
+    names = _declared_functions()
+    assert {"pal_recurrent_fwd", "pal_recurrent_bwd", "pal_chunk_fwd", "pal_chunk_bwd", "pal_build_chunk_table",
+            "pal_strerror", "pal_abi_version", "pal_validate_dims"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in palimpsa_hip.h but not exported"
+
+
+def test_abi_version_and_strerror(L):
+    lib = L.load()
+    assert lib.pal_abi_version() == L.PAL_ABI_VERSION
+    assert L.strerror(0) == "ok"
+    for code in range(-11, 0):
+        assert "unknown" not in L.strerror(code)
+    assert "unknown" in L.strerror(-99)
+
+
+def _dims(L, **kw):
+    d = dict(batch=2, seq_len=16, n_seqs=2, n_heads=2, dk=32, dv=32, total_chunks=2, dtype=L.PAL_DTYPE_BF16,
+             gate_dtype=L.PAL_DTYPE_F32, var_dtype=L.PAL_DTYPE_F32, flags=0, scale=1.0)
+    d.update(kw)
+    return L.PalDims(**d)
+
+
+def test_validate_dims_codes(L):
+    v = L.load().pal_validate_dims
+    assert v(_dims(L)) == 0
+    assert v(None) == L.PAL_E_NULL
+    assert v(_dims(L, batch=0)) == L.PAL_E_DIM
+    assert v(_dims(L, seq_len=-1)) == L.PAL_E_DIM
+    assert v(_dims(L, n_heads=0)) == L.PAL_E_DIM
+    assert v(_dims(L, dk=31)) == L.PAL_E_HEADDIM
+    assert v(_dims(L, dv=272)) == L.PAL_E_HEADDIM
+    assert v(_dims(L, dk=8)) == L.PAL_E_HEADDIM
+    assert v(_dims(L, dtype=7)) == L.PAL_E_DTYPE
+    assert v(_dims(L, gate_dtype=-1)) == L.PAL_E_DTYPE
+    assert v(_dims(L, flags=L.PAL_FLAG_VARLEN)) == L.PAL_E_VARLEN_BATCH      # B != 1 with cu_seqlens
+    assert v(_dims(L, n_seqs=3)) == L.PAL_E_DIM                               # fixed length: N must equal B
+    assert v(_dims(L, batch=1, n_seqs=40, flags=L.PAL_FLAG_VARLEN)) == L.PAL_E_CU_SEQLENS  # more docs than tokens
+    assert v(_dims(L, scale=float("nan"))) == L.PAL_E_DIM
+    assert v(_dims(L, batch=1, n_seqs=3, flags=L.PAL_FLAG_VARLEN)) == 0
+
+
+def _fake(addr=0x1000):
+    return C.c_void_p(addr)
+
+
+def _fwd_tensors(L, **kw):
+    names = ("q", "k", "v", "b", "gt", "g", "Ip", "o")
+    t = {n: _fake(0x1000 * (i + 1)) for i, n in enumerate(names)}
+    t.update(kw)
+    return L.PalFwdTensors(**t)
+
+
+def test_entry_points_reject_bad_arguments_without_touching_a_gpu(L):
+    """Every error below is detected by the host-side checks, so no HIP call is made (this test runs
+    on machines without a GPU; the pointers are fake and never dereferenced)."""
+    lib = L.load()
+    assert lib.pal_recurrent_fwd(None, None, None) == L.PAL_E_NULL
+    assert lib.pal_recurrent_fwd(_dims(L), None, None) == L.PAL_E_NULL
+    assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, q=None), None) == L.PAL_E_NULL
+    assert lib.pal_recurrent_fwd(_dims(L, dk=24), _fwd_tensors(L), None) == L.PAL_E_HEADDIM
+    assert lib.pal_recurrent_fwd(_dims(L, dk=80), _fwd_tensors(L), None) == L.PAL_E_HEADDIM   # chunk-only size
+    assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, q=_fake(0x1004)), None) == L.PAL_E_ALIGN
+    # state flags and pointers must agree
+    assert lib.pal_recurrent_fwd(_dims(L, flags=L.PAL_FLAG_HAS_INIT), _fwd_tensors(L), None) == L.PAL_E_STATE
+    assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, init_mu=_fake(), init_I=_fake()), None) == L.PAL_E_STATE
+    assert lib.pal_recurrent_fwd(_dims(L, flags=L.PAL_FLAG_STORE_FINAL), _fwd_tensors(L, final_mu=_fake()),
+                                 None) == L.PAL_E_STATE
+    assert lib.pal_recurrent_fwd(_dims(L, flags=L.PAL_FLAG_HAS_VAR), _fwd_tensors(L), None) == L.PAL_E_NULL
+    # varlen flag without cu_seqlens, and the other way round
+    assert lib.pal_recurrent_fwd(_dims(L, batch=1, n_seqs=2, flags=L.PAL_FLAG_VARLEN), _fwd_tensors(L),
+                                 None) == L.PAL_E_CU_SEQLENS
+    assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, cu_seqlens=_fake()), None) == L.PAL_E_CU_SEQLENS
+    # chunk path
+    assert lib.pal_chunk_fwd(_dims(L, flags=L.PAL_FLAG_STORE_FINAL), _fwd_tensors(L, final_mu=_fake(), final_I=_fake()),
+                             None) == L.PAL_E_NULL                               # chunk_mu / chunk_I missing
+    ok_chunk = dict(final_mu=_fake(), final_I=_fake(), chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000))
+    assert lib.pal_chunk_fwd(_dims(L, flags=L.PAL_FLAG_STORE_FINAL, total_chunks=5), _fwd_tensors(L, **ok_chunk),
+                             None) == L.PAL_E_CHUNK                              # 2 sequences of 16 tokens = 2 tiles
+    assert lib.pal_chunk_bwd(_dims(L), _fwd_tensors(L, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)), None, None, 0,
+                             None) == L.PAL_E_NULL
+    gr = L.PalBwdTensors(**{n: _fake(0x1000 * (i + 20)) for i, n in enumerate(
+        ("d_o", "dq", "dk", "dv", "db", "dgt", "dg", "dIp"))})
+    assert lib.pal_chunk_bwd(_dims(L), _fwd_tensors(L, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)), gr, None, 0,
+                             None) == L.PAL_E_WORKSPACE
+    assert lib.pal_chunk_bwd_workspace_bytes(_dims(L)) > 0
+    assert lib.pal_chunk_bwd_workspace_bytes(_dims(L, dk=5)) == 0
+
+
+def test_error_codes_map_to_python_exceptions(L):
+    with pytest.raises(ValueError):
+        L.check(L.PAL_E_VARLEN_BATCH, "x")
+    with pytest.raises(ValueError):
+        L.check(L.PAL_E_HEADDIM, "x")
+    with pytest.raises(L.PalimpsaHipError):
+        L.check(L.PAL_E_WORKSPACE, "x")
+    with pytest.raises(L.PalimpsaHipError):
+        L.check(1, "x")          # a hipError_t
+    L.check(0, "x")
+
+
+def test_chunk_table_matches_oracle(L):
+    rng = np.random.RandomState(0)
+    for _ in range(20):
+        lens = rng.randint(0, 300, size=rng.randint(1, 9))
+        lens[rng.randint(len(lens))] += 1            # at least one token overall
+        cu = np.concatenate([[0], np.cumsum(lens)])
+        table, offsets = L.build_chunk_table(cu)
+        ref = po.build_chunk_table(cu.tolist(), 64)
+        assert [tuple(r[:3]) for r in table.tolist()] == ref
+        assert offsets.tolist() == po.chunk_offsets(cu.tolist(), 64)
+        # index inside the sequence restarts at every document
+        for row in table.tolist():
+            assert row[1] == cu[row[0]] + 64 * row[3]
+    cu = po.make_varlen_lengths(32768, seed=0)
+    table, offsets = L.build_chunk_table(cu)
+    assert table[:, 2].sum() == 32768 and table[:, 2].max() <= 64 and table[:, 2].min() >= 1
+
+
+def test_chunk_table_rejects_bad_cu_seqlens(L):
+    with pytest.raises(ValueError):
+        L.build_chunk_table([1, 5])            # does not start at 0
+    with pytest.raises(ValueError):
+        L.build_chunk_table([0, 9, 5])         # decreasing
+    lib = L.load()
+    cu = (C.c_int64 * 3)(0, 100, 200)
+    out = (C.c_int32 * 8)()
+    assert lib.pal_build_chunk_table(cu, 2, out, 2, None) == L.PAL_E_CAPACITY
+    assert lib.pal_build_chunk_table(None, 2, None, 0, None) == L.PAL_E_NULL
