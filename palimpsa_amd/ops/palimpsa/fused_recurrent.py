@@ -57,21 +57,73 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
         p, dims, o, o_var, final_mu, final_I = _recurrent_forward(
             q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I_state,
             output_final_state, output_uncertainty, cu_seqlens)
-        ctx.prepared = p
-        ctx.scale = float(scale)
-        ctx.output_uncertainty = bool(output_uncertainty)
-        ctx.in_dtypes = (q.dtype, k.dtype, v.dtype, b.dtype, gt.dtype, g.dtype, Ip.dtype)
-        ctx.in_shapes = (g.shape, Ip.shape)
-        ctx.has_init = initial_mu_state is not None
+        ctx.save_for_backward(p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens)
+        ctx.meta = dict(dk=p.dk, dv=p.dv, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype, scale=float(scale),
+                        in_dtypes=(q.dtype, k.dtype, v.dtype, b.dtype, gt.dtype, g.dtype, Ip.dtype),
+                        g_shape=tuple(g.shape), Ip_shape=tuple(Ip.shape), has_init=p.init_mu is not None,
+                        output_uncertainty=bool(output_uncertainty))
         o = cm.unpad_last(o, p.dv).to(v.dtype)
         o_var = cm.unpad_last(o_var, p.dv)
         return o, o_var, cm.unpad_state(final_mu, p), cm.unpad_state(final_I, p)
 
     @staticmethod
     def backward(ctx, do, do_var, d_final_mu, d_final_I):
-        from .recurrent_backward import recurrent_backward
+        # gradients arriving at the final states are ignored, as in the chunked path (chunk...py:522)
+        q, k, v, b, gt, g, Ip, init_mu, init_I, cu = ctx.saved_tensors
+        m = ctx.meta
+        dev = q.device
+        B, T, H, dk_p = q.shape
+        dv_p = v.shape[-1]
+        cd = m["compute_dtype"]
+        has_var = m["output_uncertainty"] and do_var is not None
 
-        return recurrent_backward(ctx, do, do_var)
+        def prep(x, dt):
+            x = x.to(dt)
+            if dv_p != m["dv"]:
+                x = torch.nn.functional.pad(x, (0, dv_p - m["dv"]))
+            return x.contiguous()
+
+        do_p = prep(do, cd)
+        dovar_p = prep(do_var, torch.float32) if has_var else None
+        dq, dk_, dv_, db = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(b)
+        dgt = torch.empty(B, T, H, dtype=torch.float32, device=dev)
+        dg = torch.empty(H, dtype=torch.float32, device=dev)
+        dIp = torch.empty(H, dtype=torch.float32, device=dev)
+        d_init_mu = torch.empty_like(init_mu) if m["has_init"] else None
+        d_init_I = torch.empty_like(init_I) if m["has_init"] else None
+        flags = 0
+        if cu is not None:
+            flags |= L.PAL_FLAG_VARLEN
+        if m["has_init"]:
+            flags |= L.PAL_FLAG_HAS_INIT
+        if has_var:
+            flags |= L.PAL_FLAG_HAS_VAR
+        dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
+                         dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
+                         flags=flags, scale=m["scale"])
+        pt = cm._ptr
+        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
+                               init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))
+        grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk_), dv=pt(dv_), db=pt(db),
+                                dgt=pt(dgt), dg=pt(dg), dIp=pt(dIp), d_init_mu=pt(d_init_mu), d_init_I=pt(d_init_I))
+        lib = L.load()
+        ws_bytes = int(lib.pal_recurrent_bwd_workspace_bytes(dims))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        import ctypes as C
+        with torch.cuda.device(dev):
+            rc = lib.pal_recurrent_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes,
+                                       cm.current_stream_ptr(dev))
+        L.check(rc, "pal_recurrent_bwd")
+        dts = m["in_dtypes"]
+        dq = cm.unpad_last(dq, m["dk"]).to(dts[0])
+        dk_ = cm.unpad_last(dk_, m["dk"]).to(dts[1])
+        dv_ = cm.unpad_last(dv_, m["dv"]).to(dts[2])
+        db = cm.unpad_last(db, m["dv"]).to(dts[3])
+        if d_init_mu is not None and (dk_p != m["dk"] or dv_p != m["dv"]):
+            d_init_mu = d_init_mu[:, :, :m["dv"], :m["dk"]].contiguous()
+            d_init_I = d_init_I[:, :, :m["dv"], :m["dk"]].contiguous()
+        return (dq, dk_, dv_, db, dgt.to(dts[4]), dg.reshape(m["g_shape"]).to(dts[5]),
+                dIp.reshape(m["Ip_shape"]).to(dts[6]), None, d_init_mu, d_init_I, None, None, None)
 
 
 def fused_recurrent_palimpsa(

@@ -148,3 +148,74 @@ def test_error_paths_match_reference(gpu_device):
     cu = torch.tensor([0, 8], device=gpu_device)
     with pytest.raises(ValueError):
         fr(inp["q"], inp["k"], inp["v"], inp["b"], inp["gt"], inp["g"], inp["Ip"], cu_seqlens=cu)
+
+
+# ------------------------------------------------------------------ backward (fp32 end to end)
+def _rec_grads(inp, dev, do, dovar=None, mu0=None, I0=None, cu=None, scale=None):
+    fr = _ops()
+    names = ["q", "k", "v", "b", "gt", "g", "Ip"]
+    leaves = {n: inp[n].to(dev).clone().requires_grad_(True) for n in names}
+    kw = {}
+    if mu0 is not None:
+        leaves["mu0"] = mu0.to(dev).clone().requires_grad_(True)
+        leaves["I0"] = I0.to(dev).clone().requires_grad_(True)
+        kw.update(initial_mu_state=leaves["mu0"], initial_I_state=leaves["I0"])
+    if cu is not None:
+        kw["cu_seqlens"] = torch.tensor(cu, device=dev)
+    out = fr(*[leaves[n] for n in names], scale=scale, output_uncertainty=dovar is not None, **kw)
+    if dovar is not None:
+        loss = (out[0].float() * do.to(dev)).sum() + (out[1].float() * dovar.to(dev)).sum()
+    else:
+        loss = (out.float() * do.to(dev)).sum()
+    loss.backward()
+    return {n: x.grad for n, x in leaves.items()}
+
+
+# fp32 gradients against float64 autograd of the oracle: same bar as the fp32 forward
+GRAD_TOL = 1e-4
+
+
+@pytest.mark.parametrize("dk,dv,T", [(16, 16, 1), (32, 32, 37), (64, 64, 70), (128, 128, 20), (192, 48, 33), (256, 32, 19),
+                                     (31, 65, 45)])
+def test_fp32_backward_matches_oracle(gpu_device, dk, dv, T):
+    B, H = 2, 2
+    inp = po.make_inputs(B, T, H, dk, dv, seed=dk + dv + T)
+    inp["g"] = torch.tensor([1.0, 6.0])
+    inp["Ip"] = torch.tensor([0.6, 1.7])
+    gen = torch.Generator().manual_seed(3)
+    mu0 = torch.randn(B, H, dv, dk, generator=gen) * 0.1
+    I0 = inp["Ip"].view(1, H, 1, 1) + torch.rand(B, H, dv, dk, generator=gen)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    dovar = torch.randn(B, T, H, dv, generator=gen) * 0.3
+    ref = hp.oracle_grads(inp, do, dovar, scale=0.6, mu0=mu0, I0=I0)
+    got = _rec_grads(inp, gpu_device, do, dovar, mu0=mu0, I0=I0, scale=0.6)
+    for n in ["q", "k", "v", "b", "gt", "g", "Ip", "mu0", "I0"]:
+        assert hp.max_rel(got[n], ref[n]) <= GRAD_TOL, (n, hp.max_rel(got[n], ref[n]))
+
+
+def test_fp32_backward_varlen_and_no_state(gpu_device):
+    H, d = 3, 32
+    cu = [0, 1, 18, 19, 83, 130]
+    T = cu[-1]
+    inp = po.make_inputs(1, T, H, d, d, seed=13)
+    do = torch.randn(1, T, H, d, generator=torch.Generator().manual_seed(14))
+    ref = hp.oracle_grads(inp, do, cu=cu)
+    got = _rec_grads(inp, gpu_device, do, cu=cu)
+    for n in ["q", "k", "v", "b", "gt", "g", "Ip"]:
+        assert hp.max_rel(got[n], ref[n]) <= GRAD_TOL, (n, hp.max_rel(got[n], ref[n]))
+
+
+def test_bf16_rows_backward(gpu_device):
+    B, T, H, d = 2, 50, 2, 64
+    inp = hp.rounded(po.make_inputs(B, T, H, d, d, seed=17), torch.bfloat16)
+    do = torch.randn(B, T, H, d, generator=torch.Generator().manual_seed(18))
+    ref = hp.oracle_grads(inp, do)
+    got = _rec_grads(inp, gpu_device, do)
+    assert got["q"].dtype == torch.bfloat16
+    # arithmetic is fp32, but o is a bf16 tensor, so autograd hands the kernel dO rounded to bf16
+    # (2^-9 relative) and the row gradients are stored in bf16: every gradient carries that rounding
+    for n in ["q", "k", "v", "b", "gt"]:
+        assert hp.max_rel(got[n], ref[n]) <= 5e-3, n
+    # per-head reductions over all tokens of those rounded terms: the bf16 gradient bar
+    for n in ["g", "Ip"]:
+        assert hp.max_rel(got[n], ref[n]) <= hp.BF16_GRAD_NORM_TOL, n
