@@ -24,6 +24,9 @@ ARCH = "gfx950"
 CXXFLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results are consumed by VALU epilogues: keep them in arch VGPRs instead of
+    # AccVGPRs that would need a v_accvgpr_read per element
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

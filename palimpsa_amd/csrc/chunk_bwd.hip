@@ -222,6 +222,10 @@ __global__ __launch_bounds__(NB * 64) void chunk_bwd_local_kernel(BwdArgs A) {
   float* wDJ = A.wDJ + tile_off + 16 * nb + 4 * g;
   const float f_first = fast_exp2(sC[0]);
 
+  // tile-start state of the next value row is fetched one iteration ahead
+  float mu0_n = cmu[0], I0_n = cI[0];
+  f32x4 muT_n = *(const f32x4*)cmuT, IT_n = *(const f32x4*)cIT;
+
   const int n_groups = dv / kDG2;
   for (int dg = 0; dg < n_groups; ++dg) {
     const int buf = dg & 1;
@@ -232,11 +236,16 @@ __global__ __launch_bounds__(NB * 64) void chunk_bwd_local_kernel(BwdArgs A) {
     if (dg + 1 < n_groups) stage_load(dg + 1);
     for (int dd = 0; dd < kDG2; ++dd) {
       const int d = dg * kDG2 + dd;
-      const float mu0 = cmu[(int64_t)d * dk];
-      const float I0 = cI[(int64_t)d * dk];
+      const float mu0 = mu0_n, I0 = I0_n;
+      const f32x4 muT = muT_n, IT = IT_n;
+      {
+        const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
+        mu0_n = cmu[dn];
+        I0_n = cI[dn];
+        muT_n = *(const f32x4*)(cmuT + dn);
+        IT_n = *(const f32x4*)(cIT + dn);
+      }
       const float M0 = mu0 * I0, J0 = I0 - Ip;
-      const f32x4 muT = *(const f32x4*)(cmuT + (int64_t)d * dk);
-      const f32x4 IT = *(const f32x4*)(cIT + (int64_t)d * dk);
       bf16x8 XM[2], XJ[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {

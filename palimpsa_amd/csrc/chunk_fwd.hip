@@ -1,13 +1,12 @@
-// Chunked Palimpsa forward: two kernels.
+// Chunked Palimpsa forward: three kernels.
 //
-//  (1) chunk_state_kernel — one wave per (sequence, head, 16x16 tile of the
-//      dv x dk state) walks the tiles of its sequence in order and applies
-//        S <- F_C * S + (a o V)^T K          (a_s = decay from token s to tile end)
-//      with bf16 MFMA contractions, fp32 state in registers.  It writes the
-//      state at the START of every tile (what the reference stores as
-//      intermediate_mu_state / intermediate_I_state,
-//      chunk_palimpsa_forgetting_scalar.py:187-188) and the final state
-//      (:214-218).  This is the only serial part of the forward.
+//  (1) chunk_delta_kernel + chunk_scan_kernel — the state at the START of every
+//      tile.  The first computes every tile's own contribution
+//        Delta = (a o V)^T K                 (a_s = decay from token s to tile end)
+//      with bf16 MFMA contractions, all tiles in parallel; the second runs the
+//      recurrence S_c = F_C S_{c-1} + Delta_c over the tiles of a sequence as an
+//      fp32 streaming scan (the only serial part of the forward) and leaves the
+//      tile-start states and the final state in (mu, I) form.
 //  (2) chunk_out_kernel — one workgroup per (tile, head), all tiles in
 //      parallel.  Wave w owns key columns [16w, 16w+16).  For every value row d
 //      it builds the operand X^T[n,s] = k_s[n] v_s[d] (and k_s[n]^2 b_s[d]),
@@ -21,117 +20,182 @@
 
 namespace pal {
 
-// ------------------------------------------------------------------ kernel 1
+// ------------------------------------------------------------------ kernel 1a
+// Local contribution of one tile to the state: Delta = (a o V)^T K, with a_s the decay from token s
+// to the end of the tile.  One workgroup of 4 waves per (tile, head), all tiles in parallel: the
+// K, V, B rows of the tile are staged once through LDS (16-byte loads, stored transposed so that an
+// MFMA operand is one contiguous run of tokens), then wave w produces the 16x16 blocks of the state
+// whose key columns are [16w, 16w+16) (+64, ...).  The result is parked in the tile's slot of
+// chunk_mu / chunk_I until the scan below replaces it.
+constexpr int kTS = 68;  // row stride (floats) of the transposed staging tiles
+
 template <typename TIn>
-__global__ __launch_bounds__(64) void chunk_state_kernel(ChunkArgs a) {
-  __shared__ float sA[kC];
-  const int lane = threadIdx.x, i = lane & 15, g = lane >> 4;
-  const int NB = a.dk >> 4, ND = a.dv >> 4;
-  int bid = blockIdx.x;
-  const int nb = bid % NB; bid /= NB;
-  const int dt = bid % ND; bid /= ND;
-  const int h = bid % a.H;
-  const int n = bid / a.H;
-  const int H = a.H, dk = a.dk, dv = a.dv;
-  int bos, len, cbase;
-  seq_lookup(a, n, bos, len, cbase);
-  const float Ip = a.Ip[h];
-  const float gh = a.g[h] * kLog2e;
-
-  // state tile in MFMA accumulator layout: rows d = 16dt + 4g + r, column n = 16nb + i
-  f32x4 M = {0.f, 0.f, 0.f, 0.f}, J = {0.f, 0.f, 0.f, 0.f};
-  const int64_t st_off = (((int64_t)n * H + h) * dv + 16 * dt + 4 * g) * dk + 16 * nb + i;
-  if (a.init_mu) {
+__device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_stride, int width, int clen, float* dst,
+                                                 int tid) {
+  // src: [64 tokens][width] rows -> dst[width][kTS] (token index fastest), rows >= clen are zero
+  const int groups = width >> 3;
+  for (int idx = tid; idx < kC * groups; idx += 256) {
+    const int s = idx & (kC - 1), c8 = idx >> 6;
+    float x[8];
+    if (s < clen) {
+      load_vec<4>(src + (int64_t)s * row_stride + 8 * c8, x);
+      load_vec<4>(src + (int64_t)s * row_stride + 8 * c8 + 4, x + 4);
+    } else {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float mu = a.init_mu[st_off + (int64_t)r * dk];
-      const float I = a.init_I[st_off + (int64_t)r * dk];
-      M[r] = mu * I;
-      J[r] = I - Ip;
+      for (int e = 0; e < 8; ++e) x[e] = 0.f;
     }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[(8 * c8 + e) * kTS + s] = x[e];
   }
+}
 
-  const TIn* kp = (const TIn*)a.k + (int64_t)h * dk + 16 * nb + i;
-  const TIn* vp = (const TIn*)a.v + (int64_t)h * dv + 16 * dt + i;
-  const TIn* bp = (const TIn*)a.b + (int64_t)h * dv + 16 * dt + i;
-
-  const int nchunks = (len + kC - 1) / kC;
-  float kr[2][8], vr[2][8], br[2][8], gtr;
-  auto load_tile = [&](int c, float (&kx)[2][8], float (&vx)[2][8], float (&bx)[2][8], float& gx) {
-    const int t0 = bos + c * kC;
-    const int clen = min(kC, len - c * kC);
+template <typename TIn>
+__global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
+  extern __shared__ float smem[];
+  const int H = a.H, dk = a.dk, dv = a.dv;
+  float* sA = smem;                 // [64] decay from token s to the end of the tile
+  float* sKT = sA + kC;             // [dk][kTS]
+  float* sVT = sKT + dk * kTS;      // [dv][kTS]
+  float* sBT = sVT + dv * kTS;      // [dv][kTS]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
+  const int NB = dk >> 4, ND = dv >> 4;
+  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  if (w == 0) {
+    const float gh = a.g[h] * kLog2e;
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    const float cs = wave_inclusive_scan(-gt * gh, lane);
+    sA[lane] = fast_exp2(__shfl(cs, 63) - cs);
+  }
+  stage_transposed((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, (int64_t)H * dk, dk, clen, sKT, tid);
+  stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sVT, tid);
+  stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sBT, tid);
+  __syncthreads();
+  float as[2][8];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int s = 8 * g + j + 32 * ks;
-        const bool ok = s < clen;
-        const int64_t tok = (int64_t)(t0 + (ok ? s : 0)) * H;
-        const float kv = to_f32(kp[tok * dk]), vv = to_f32(vp[tok * dv]), bv = to_f32(bp[tok * dv]);
-        kx[ks][j] = ok ? kv : 0.f;
-        vx[ks][j] = ok ? vv : 0.f;
-        bx[ks][j] = ok ? bv : 0.f;
-      }
-    gx = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
-  };
-
-  if (nchunks > 0) load_tile(0, kr, vr, br, gtr);
-  for (int c = 0; c < nchunks; ++c) {
-    // state at the start of this tile, in (mu, I) form
-    {
-      const int64_t co = (((int64_t)(cbase + c) * H + h) * dv + 16 * dt + 4 * g) * dk + 16 * nb + i;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float I = J[r] + Ip;
-        a.chunk_mu[co + (int64_t)r * dk] = M[r] * fast_rcp(I);
-        a.chunk_I[co + (int64_t)r * dk] = I;
-      }
-    }
-    float kn[2][8], vn[2][8], bn[2][8], gtn = 0.f;
-    const bool more = c + 1 < nchunks;
-    if (more) load_tile(c + 1, kn, vn, bn, gtn);
-
-    const float cs = wave_inclusive_scan(-gtr * gh, lane);
-    const float tot = __shfl(cs, 63);
-    __syncthreads();
-    sA[lane] = fast_exp2(tot - cs);
-    __syncthreads();
-    const float FC = fast_exp2(tot);
-    bf16x8 AM[2], AJ[2], BK[2], BKK[2];
+  for (int ks = 0; ks < 2; ++ks) {
+    *(f32x4*)&as[ks][0] = *(const f32x4*)&sA[8 * g + 32 * ks];
+    *(f32x4*)&as[ks][4] = *(const f32x4*)&sA[8 * g + 32 * ks + 4];
+  }
+  for (int nb = w; nb < NB; nb += 4) {
+    bf16x8 BK[2], BKK[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const f32x4 a0 = *(const f32x4*)&sA[8 * g + 32 * ks];
-      const f32x4 a1 = *(const f32x4*)&sA[8 * g + 32 * ks + 4];
+      float kv[8];
+      *(f32x4*)&kv[0] = *(const f32x4*)&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks];
+      *(f32x4*)&kv[4] = *(const f32x4*)&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks + 4];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float as = j < 4 ? a0[j & 3] : a1[j & 3];
-        AM[ks][j] = (bf16_t)(as * vr[ks][j]);
-        AJ[ks][j] = (bf16_t)(as * br[ks][j]);
-        BK[ks][j] = (bf16_t)kr[ks][j];
-        BKK[ks][j] = (bf16_t)(kr[ks][j] * kr[ks][j]);
+        BK[ks][j] = (bf16_t)kv[j];
+        BKK[ks][j] = (bf16_t)(kv[j] * kv[j]);
       }
     }
+    for (int dt = 0; dt < ND; ++dt) {
+      bf16x8 AM[2], AJ[2];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) { M[r] *= FC; J[r] *= FC; }
-    M = mfma16(AM[0], BK[0], M);
-    J = mfma16(AJ[0], BKK[0], J);
-    M = mfma16(AM[1], BK[1], M);
-    J = mfma16(AJ[1], BKK[1], J);
-    if (more) {
+      for (int ks = 0; ks < 2; ++ks) {
+        float vv[8], bb[8];
+        *(f32x4*)&vv[0] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
+        *(f32x4*)&vv[4] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
+        *(f32x4*)&bb[0] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
+        *(f32x4*)&bb[4] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+        for (int j = 0; j < 8; ++j) {
+          AM[ks][j] = (bf16_t)(as[ks][j] * vv[j]);
+          AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
+        }
+      }
+      f32x4 M = {0.f, 0.f, 0.f, 0.f}, J = {0.f, 0.f, 0.f, 0.f};
+      M = mfma16(AM[0], BK[0], M);
+      J = mfma16(AJ[0], BKK[0], J);
+      M = mfma16(AM[1], BK[1], M);
+      J = mfma16(AJ[1], BKK[1], J);
+      // accumulator layout: rows d = 16dt + 4g + r, column n = 16nb + i
+      const int64_t co = (((int64_t)cidx * H + h) * dv + 16 * dt + 4 * g) * dk + 16 * nb + i;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { kr[ks][j] = kn[ks][j]; vr[ks][j] = vn[ks][j]; br[ks][j] = bn[ks][j]; }
-      gtr = gtn;
+      for (int r = 0; r < 4; ++r) {
+        a.chunk_mu[co + (int64_t)r * dk] = M[r];
+        a.chunk_I[co + (int64_t)r * dk] = J[r];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ kernel 1b
+// Serial part of the forward: S_c = F_c S_{c-1} + Delta_c per state entry, fp32, pure streaming.
+// One thread per (sequence, head, state entry), 256 consecutive entries per block.  Each slot of
+// chunk_mu / chunk_I is overwritten with the state at the START of its tile in (mu, I) form
+// (what the reference stores as intermediate_*_state, chunk_palimpsa_forgetting_scalar.py:187-188);
+// the state after the last tile goes to final_mu / final_I (:214-218).
+constexpr int kScanTiles = 1024;   // per-tile decays kept in LDS at a time
+
+__global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
+  __shared__ float sF[kScanTiles];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int64_t E = (int64_t)a.dv * a.dk;
+  const int nblk = (int)(E / 256);
+  const int blk = blockIdx.x % nblk;
+  const int nh = blockIdx.x / nblk;
+  const int h = nh % a.H, n = nh / a.H;
+  const int64_t e = (int64_t)blk * 256 + tid;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const int nchunks = (len + kC - 1) / kC;
+  const float Ip = a.Ip[h];
+  const float gh = a.g[h] * kLog2e;
+  float SM = 0.f, SJ = 0.f;
+  const int64_t so = (int64_t)nh * E + e;
+  if (a.init_mu) {
+    const float mu = a.init_mu[so], I = a.init_I[so];
+    SM = mu * I;
+    SJ = I - Ip;
+  }
+  for (int c0 = 0; c0 < nchunks; c0 += kScanTiles) {
+    const int cn = min(kScanTiles, nchunks - c0);
+    __syncthreads();
+    for (int c = w; c < cn; c += 4) {
+      const int t = (c0 + c) * kC + lane;
+      const float gt = (t < len) ? load_gate(a.gt, (int64_t)(bos + t) * a.H + h, a.gate_bf16) : 0.f;
+      const float tot = wave_sum(-gt * gh);
+      if (lane == 0) sF[c] = fast_exp2(tot);
+    }
+    __syncthreads();
+    int c = 0;
+    for (; c + 4 <= cn; c += 4) {
+      float dM[4], dJ[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t off = ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e;
+        dM[u] = a.chunk_mu[off];
+        dJ[u] = a.chunk_I[off];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t off = ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e;
+        const float I = SJ + Ip;
+        a.chunk_mu[off] = SM * fast_rcp(I);
+        a.chunk_I[off] = I;
+        const float F = sF[c + u];
+        SM = fmaf(F, SM, dM[u]);
+        SJ = fmaf(F, SJ, dJ[u]);
+      }
+    }
+    for (; c < cn; ++c) {
+      const int64_t off = ((int64_t)(cbase + c0 + c) * a.H + h) * E + e;
+      const float dM = a.chunk_mu[off], dJ = a.chunk_I[off];
+      const float I = SJ + Ip;
+      a.chunk_mu[off] = SM * fast_rcp(I);
+      a.chunk_I[off] = I;
+      const float F = sF[c];
+      SM = fmaf(F, SM, dM);
+      SJ = fmaf(F, SJ, dJ);
     }
   }
   if (a.final_mu) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float I = J[r] + Ip;
-      a.final_mu[st_off + (int64_t)r * dk] = M[r] * fast_rcp(I);
-      a.final_I[st_off + (int64_t)r * dk] = I;
-    }
+    const float I = SJ + Ip;
+    a.final_mu[so] = SM * fast_rcp(I);
+    a.final_I[so] = I;
   }
 }
 
@@ -251,14 +315,19 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
   const float* cmu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
   const float* cI = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
 
+  // tile-start state of the next value row is fetched one iteration ahead
+  f32x4 mu0_n = *(const f32x4*)cmu, I0_n = *(const f32x4*)cI;
   const int n_groups = dv / kDG;
   for (int dg = 0; dg < n_groups; ++dg) {
     if (dg + 1 < n_groups) stage_load(dg + 1);
-#pragma unroll 2
     for (int dd = 0; dd < kDG; ++dd) {
       const int d = dg * kDG + dd;
-      const f32x4 mu0 = *(const f32x4*)(cmu + (int64_t)d * dk);
-      const f32x4 I0 = *(const f32x4*)(cI + (int64_t)d * dk);
+      const f32x4 mu0 = mu0_n, I0 = I0_n;
+      {
+        const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
+        mu0_n = *(const f32x4*)(cmu + dn);
+        I0_n = *(const f32x4*)(cI + dn);
+      }
       float M0[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) M0[r] = mu0[r] * I0[r];
@@ -411,11 +480,26 @@ extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* str
   ChunkArgs a;
   fill_chunk_args(a, d, t);
   hipStream_t s = (hipStream_t)stream;
-  const int64_t waves = (int64_t)d->n_seqs * d->n_heads * (d->dv / 16) * (d->dk / 16);
-  if (waves > 0x7fffffff) return PAL_E_DIM;
-  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_state_kernel<bf16_t>), dim3((unsigned)waves), dim3(64), 0, s, a);
-  else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_state_kernel<float>), dim3((unsigned)waves), dim3(64), 0, s, a);
-  PAL_HIP_LAUNCH_CHECK();
+  {
+    const int64_t blocks = (int64_t)d->total_chunks * d->n_heads;
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    const size_t lds = sizeof(float) * (kC + (size_t)(d->dk + 2 * d->dv) * kTS);
+    if (lds > kMaxLds) return PAL_E_HEADDIM;
+    if (d->dtype == PAL_DTYPE_BF16) {
+      if (int rc2 = allow_lds((const void*)&chunk_delta_kernel<bf16_t>, lds)) return rc2;
+      PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+    } else {
+      if (int rc2 = allow_lds((const void*)&chunk_delta_kernel<float>, lds)) return rc2;
+      PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+    }
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  {
+    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk) / 256);
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    PAL_TIMED_LAUNCH(kKernChunkScan, s, chunk_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    PAL_HIP_LAUNCH_CHECK();
+  }
   if (d->dtype == PAL_DTYPE_BF16) return launch_out<bf16_t>(a, s);
   return launch_out<float>(a, s);
 }

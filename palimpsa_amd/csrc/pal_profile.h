@@ -7,6 +7,7 @@ namespace pal {
 enum KernelId {
   kKernRecurrentFwd = 0,
   kKernChunkState,
+  kKernChunkScan,
   kKernChunkOut,
   kKernBwdLocal,
   kKernBwdCarryScan,
