@@ -462,13 +462,24 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
 
 // ---------------------------------------------------------------- carry apply
 // dv_s += a_s R_M k_s ; db_s += a_s R_J k_s^2 ; dk_s += a_s (R_M^T v_s + 2 k_s * R_J^T b_s)
+// One workgroup of 4 waves per (tile, head); wave w owns tokens [16w, 16w+16).  The four products
+// run on the matrix cores (bf16 operands, fp32 accumulate); their results are parked in LDS and then
+// added to the tile-local gradients with 16-byte loads/stores that are contiguous along the head dim.
 template <typename TIn>
 __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
-  __shared__ float sAs[kC];
-  __shared__ float sBt[kC];
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
+  extern __shared__ float smem[];
   const int H = a.H, dk = a.dk, dv = a.dv;
+  const int dmax = dk > dv ? dk : dv;
+  float* sAs = smem;                       // [64] decay from token s to the end of the tile
+  float* sW4 = sAs + kC;                   // [8]
+  float* sBt = sW4 + 8;                    // [64][32] beta of the carry terms, one slot per work item
+  float* sO1 = sBt + kC * 32;                   // [64][kOS..] dv^carry, later dk^carry
+  float* sO2 = sO1 + kC * (dmax + 4);      // [64][..]   db^carry
+  bf16_t* sRT = (bf16_t*)(sO2 + kC * (dmax + 4));   // [2][dk][dv + 8] R_M^T, R_J^T in bf16
+  const int RS = dv + 8;
+  const int OS = dmax + 4;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
   chunk_lookup(a, cidx, seq, t0, clen, cis);
@@ -481,7 +492,6 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     return;
   }
   const float gh = a.g[h] * kLog2e;
-  __shared__ float sW4[5];
   if (w == 0) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     const float c = wave_inclusive_scan(-gt * gh, lane);
@@ -489,33 +499,41 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     sAs[lane] = fast_exp2(tot - c);
     if (lane == 0) sW4[4] = fast_exp2(tot);
   }
+  const int64_t E = (int64_t)dv * dk;
+  const float* RM = A.wDM + ((int64_t)cidx * H + h) * E;
+  const float* RJ = A.wDJ + ((int64_t)cidx * H + h) * E;
   {
-    // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile
-    const int64_t E = (int64_t)dv * dk;
-    const float* rm = A.wDM + ((int64_t)cidx * H + h) * E;
-    const float* rj = A.wDJ + ((int64_t)cidx * H + h) * E;
+    // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile; the same
+    // pass leaves R^T in LDS for the products that contract over the value rows
     const float* smu = a.chunk_mu + ((int64_t)cidx * H + h) * E;
     const float* sI = a.chunk_I + ((int64_t)cidx * H + h) * E;
     const float Ipb = a.Ip[h];
     float acc = 0.f;
-    for (int64_t e = tid; e < E; e += 256) {
-      const float I = sI[e];
-      acc = fmaf(rm[e], smu[e] * I, acc);
-      acc = fmaf(rj[e], I - Ipb, acc);
+    const int ngrp = dk >> 2;
+    for (int idx = tid; idx < dv * ngrp; idx += 256) {
+      const int d = idx % dv, c4 = idx / dv;
+      const int64_t e = (int64_t)d * dk + 4 * c4;
+      const f32x4 rm = *(const f32x4*)(RM + e), rj = *(const f32x4*)(RJ + e);
+      const f32x4 mu = *(const f32x4*)(smu + e), I = *(const f32x4*)(sI + e);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        acc = fmaf(rm[x], mu[x] * I[x], acc);
+        acc = fmaf(rj[x], I[x] - Ipb, acc);
+        sRT[(4 * c4 + x) * RS + d] = (bf16_t)rm[x];
+        sRT[(dk + 4 * c4 + x) * RS + d] = (bf16_t)rj[x];
+      }
     }
     acc = wave_sum(acc);
     if (lane == 0) sW4[w] = acc;
   }
   __syncthreads();
   if (tid == 0) A.wBnd[(int64_t)cidx * H + h] = sW4[4] * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);
-  const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
-  const float* RM = A.wDM + tile_off;
-  const float* RJ = A.wDJ + tile_off;
+
   const int srow = 16 * w + i;            // operand row (token) of this lane
   const bool row_ok = srow < clen;
   const float as = sAs[srow];
   const int64_t tokA = ((int64_t)(t0 + (row_ok ? srow : 0)) * H + h);
-  float beta4[4] = {0.f, 0.f, 0.f, 0.f};
+  const int64_t tok0 = ((int64_t)t0 * H + h);
 
   // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
   {
@@ -541,10 +559,6 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         }
       }
     }
-    TIn* dvo = (TIn*)A.dv;
-    TIn* dbo = (TIn*)A.db;
-    const TIn* vin = (const TIn*)a.v;
-    const TIn* bin = (const TIn*)a.b;
     for (int db_ = 0; db_ < dv / 16; ++db_) {
       f32x4 accV = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -570,19 +584,51 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
           accB = mfma16(A2[ks], B2, accB);
         }
       }
+      // accumulator layout: rows s = 16w + 4g + r, column d = 16db_ + i
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int s = 16 * w + 4 * g + r;
-        if (s < clen) {
-          const int64_t off = ((int64_t)(t0 + s) * H + h) * dv + 16 * db_ + i;
-          dvo[off] = from_f32<TIn>(to_f32(dvo[off]) + accV[r]);
-          dbo[off] = from_f32<TIn>(to_f32(dbo[off]) + accB[r]);
-          beta4[r] = fmaf(to_f32(vin[off]), accV[r], beta4[r]);
-          beta4[r] = fmaf(to_f32(bin[off]), accB[r], beta4[r]);
-        }
+        sO1[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accV[r];
+        sO2[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accB[r];
       }
     }
   }
+  __syncthreads();
+  {
+    // add to the tile-local dv, db; beta_s = <v_s, dv^carry_s> + <b_s, db^carry_s>
+    const int groups = dv >> 3;   // work item = (token, 8 value rows); the items of a token sit in adjacent lanes
+    const TIn* vin = (const TIn*)a.v + tok0 * dv;
+    const TIn* bin = (const TIn*)a.b + tok0 * dv;
+    TIn* dvo = (TIn*)A.dv + tok0 * dv;
+    TIn* dbo = (TIn*)A.db + tok0 * dv;
+    for (int idx = tid; idx < kC * groups; idx += 256) {
+      const int c8 = idx % groups, s = idx / groups;
+      float beta = 0.f;
+      if (s < clen) {
+        const int64_t off = (int64_t)s * H * dv + 8 * c8;
+        float xv[8], xb[8], gv[8], gb[8];
+        load_vec<4>(vin + off, xv); load_vec<4>(vin + off + 4, xv + 4);
+        load_vec<4>(bin + off, xb); load_vec<4>(bin + off + 4, xb + 4);
+        load_vec<4>(dvo + off, gv); load_vec<4>(dvo + off + 4, gv + 4);
+        load_vec<4>(dbo + off, gb); load_vec<4>(dbo + off + 4, gb + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float cv = sO1[s * OS + 8 * c8 + e], cb = sO2[s * OS + 8 * c8 + e];
+          beta = fmaf(xv[e], cv, beta);
+          beta = fmaf(xb[e], cb, beta);
+          dvo[off + e] = from_f32<TIn>(gv[e] + cv);
+          dbo[off + e] = from_f32<TIn>(gb[e] + cb);
+        }
+      }
+      sBt[idx] = beta;
+    }
+    __syncthreads();
+    if (tid < clen) {
+      float bsum = 0.f;
+      for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[tid * groups + c8];   // fixed order
+      A.wBc[(int64_t)h * A.tokens + t0 + tid] = bsum;
+    }
+  }
+
   // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
   {
     const int KS = (dv + 31) / 32;
@@ -608,8 +654,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         }
       }
     }
-    TIn* dko = (TIn*)A.dk;
-    const TIn* kin = (const TIn*)a.k;
+    const TIn* kin = (const TIn*)a.k + tok0 * dk;
     for (int nbk = 0; nbk < dk / 16; ++nbk) {
       f32x4 accM = {0.f, 0.f, 0.f, 0.f}, accJ = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -617,36 +662,41 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         if (ks < KS) {
           const int d0 = 8 * g + 32 * ks;
           bf16x8 B3, B4;
+          if (d0 < dv) {
+            B3 = *(const bf16x8*)&sRT[(16 * nbk + i) * RS + d0];
+            B4 = *(const bf16x8*)&sRT[(dk + 16 * nbk + i) * RS + d0];
+          } else {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const bool ok = d0 + j < dv;
-            const int64_t ro = (int64_t)(ok ? d0 + j : 0) * dk + 16 * nbk + i;
-            const float x = RM[ro], y = RJ[ro];
-            B3[j] = (bf16_t)(ok ? x : 0.f);
-            B4[j] = (bf16_t)(ok ? y : 0.f);
+            for (int j = 0; j < 8; ++j) { B3[j] = (bf16_t)0.f; B4[j] = (bf16_t)0.f; }
           }
           accM = mfma16(A3[ks], B3, accM);
           accJ = mfma16(A4[ks], B4, accJ);
         }
       }
+      // rows s = 16w + 4g + r, column n = 16nbk + i
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int s = 16 * w + 4 * g + r;
-        if (s < clen) {
-          const int64_t off = ((int64_t)(t0 + s) * H + h) * dk + 16 * nbk + i;
-          const float kv = to_f32(kin[off]);
-          dko[off] = from_f32<TIn>(to_f32(dko[off]) + accM[r] + 2.f * kv * accJ[r]);
-        }
+        const float kv = (s < clen) ? to_f32(kin[(int64_t)s * H * dk + 16 * nbk + i]) : 0.f;
+        sO1[s * OS + 16 * nbk + i] = fmaf(2.f * kv, accJ[r], accM[r]);
       }
     }
   }
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float x = row16_sum(beta4[r]);
-    if (i == 0) sBt[16 * w + 4 * g + r] = x;
-  }
   __syncthreads();
-  if (tid < clen) A.wBc[(int64_t)h * A.tokens + t0 + tid] = sBt[tid];
+  {
+    const int groups = dk >> 3;
+    TIn* dko = (TIn*)A.dk + tok0 * dk;
+    for (int idx = tid; idx < kC * groups; idx += 256) {
+      const int c8 = idx % groups, s = idx / groups;
+      if (s < clen) {
+        const int64_t off = (int64_t)s * H * dk + 8 * c8;
+        float gk[8];
+        load_vec<4>(dko + off, gk); load_vec<4>(dko + off + 4, gk + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dko[off + e] = from_f32<TIn>(gk[e] + sO1[s * OS + 8 * c8 + e]);
+      }
+    }
+  }
 }
 
 // ----------------------------------------------------------------- gate pass
@@ -822,8 +872,16 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   }
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
-    if (bf) PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<bf16_t>), dim3(blocks), dim3(256), 0, s, A);
-    else PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<float>), dim3(blocks), dim3(256), 0, s, A);
+    const int dmax = dd.dk > dd.dv ? dd.dk : dd.dv;
+    const size_t lds = sizeof(float) * (kC + 8 + kC * 32 + 2 * (size_t)kC * (dmax + 4)) + 2 * (size_t)2 * dd.dk * (dd.dv + 8);
+    if (lds > kMaxLds) return PAL_E_HEADDIM;
+    if (bf) {
+      if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<bf16_t>, lds)) return rc2;
+      PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<bf16_t>), dim3(blocks), dim3(256), lds, s, A);
+    } else {
+      if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<float>, lds)) return rc2;
+      PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<float>), dim3(blocks), dim3(256), lds, s, A);
+    }
     PAL_HIP_LAUNCH_CHECK();
   }
   PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads)), dim3(256), 0, s, A);
