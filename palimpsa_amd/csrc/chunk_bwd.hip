@@ -28,6 +28,8 @@
 //                         beta_r = <v_r, dv^carry_r> + <b_r, db^carry_r> from the apply pass and
 //                         (M_0, J_0) the state at the start of the tile.
 //          dgt = -g dlogf, dg = -sum gt dlogf, dIp = sum dJloc (- sum dJ_0 with an initial state).
+#include <type_traits>
+
 #include "chunk_common.h"
 #include "pal_host.h"
 #include "pal_profile.h"
@@ -421,6 +423,424 @@ __global__ __launch_bounds__(NB * 64) void chunk_bwd_local_kernel(BwdArgs A) {
   }
 }
 
+// ------------------------------------------------- local pass, four wave roles
+// Same arithmetic as chunk_bwd_local_kernel, organised for four waves per SIMD: one wave issues a
+// VALU instruction every 5-9 cycles at best while the SIMD can start one every 2-3, so the tile's
+// work is cut into roles small enough for 128 registers.  A workgroup has 4*NB waves; wave = role*NB + nb.
+//   roles 0/1 ("producers", token blocks 0-1 / 2-3): recompute the states of one value row for 16 key
+//     columns, form dMloc/dJloc and dq, and leave packed bf16 operands in an LDS slot:
+//     role 0 writes P^M_0, P^J_0, X^M_0, X^J_0 (tokens 0..31), role 1 the halves for tokens 32..63;
+//   roles 2/3 ("consumers", token blocks 0-1 / 2-3 of the column token s): pick the slot up one iteration
+//     later and do the reverse contraction, the strictly-lower product and the dv/db/dk/gate epilogue.
+// The roles keep their per-tile constants and accumulators in the same register arrays (Lop, R0..R3)
+// with role-specific meaning, so that the allocator does not reserve space for all of them at once.
+template <typename TIn, int NB, bool HAS_VAR>
+__global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(4)))
+void chunk_bwd_local_roles_kernel(BwdArgs A) {
+  const ChunkArgs& a = A.c;
+  extern __shared__ float smem[];
+  constexpr int NST = HAS_VAR ? 4 : 3;  // staged tensors: v, b, do, (dovar)
+  constexpr int STG = kDG2 * kVS2;
+  float* sC = smem;                      // [64] running log2 decay
+  float* sF = sC + kC;                   // [64] 2^c
+  float* sSt = sF + kC;                  // [2][NST][16][kVS2]
+  float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
+  float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
+  float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [2*NB] sums of dJloc (padded to 16 floats)
+  float* sMJ = sRed + NB * kC + 16;      // [NB][2 slots][2][16] tile-start M_0, J_0 of the row in flight
+  bf16x8* sX = (bf16x8*)(sMJ + NB * 64);   // [NB][2 slots][8 operands][64 lanes]
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: role branches are scalar
+  const int role = wave / NB, nb = wave - role * NB;
+  const int H = a.H, dk = a.dk, dv = a.dv;
+  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  const float Ip = a.Ip[h];
+  const float gh = a.g[h] * kLog2e;
+  const float scale = a.scale;
+
+  if (wave == 0) {
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    const float c = wave_inclusive_scan(-gt * gh, lane);
+    sC[lane] = c;
+    sF[lane] = fast_exp2(c);
+    if (lane == 63) A.wFtot[(int64_t)cidx * H + h] = c;
+  }
+  // Global addresses are kept as a wave-uniform base plus a 32-bit lane offset, so that the
+  // loop-invariant parts live in scalar registers.
+  // Staging of 16 value rows x 64 tokens (v, b, do, dovar) and the dv/db flush: threads 0..255,
+  // thread = (token s, quad of rows q4).
+  const int64_t row0 = ((int64_t)t0 * H + h) * dv;
+  const TIn* vp = (const TIn*)a.v + row0;
+  const TIn* bp = (const TIn*)a.b + row0;
+  const TIn* dop = (const TIn*)A.d_o + row0;
+  const int st_s = tid >> 2, st_q = tid & 3;
+  const bool st_on = tid < kC * kDG2 / 4;
+  const unsigned st_off = (unsigned)(st_s * H * dv + 4 * st_q);
+  auto stage = [&](int dg) {
+    if (!st_on) return;
+    float st[NST][4];
+    if (st_s < clen) {
+      load_vec<4>(vp + dg * kDG2 + st_off, st[0]);
+      load_vec<4>(bp + dg * kDG2 + st_off, st[1]);
+      load_vec<4>(dop + dg * kDG2 + st_off, st[2]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) st[2][e] *= scale;
+      if (HAS_VAR) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st[NST - 1][e] = scale * load_rt(A.d_o_var, row0 + dg * kDG2 + st_off + e, a.var_bf16);
+      }
+    } else {
+#pragma unroll
+      for (int x = 0; x < NST; ++x)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st[x][e] = 0.f;
+    }
+    const int buf = dg & 1;
+#pragma unroll
+    for (int x = 0; x < NST; ++x)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * st_q + e) * kVS2 + st_s] = st[x][e];
+  };
+  stage(0);
+  __syncthreads();
+
+  const int64_t rs = (int64_t)H * dk;   // token stride of q, k
+  const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
+  const int n_groups = dv / kDG2;
+  const float f_first = fast_exp2(sC[0]);
+
+  // end of one iteration, identical for every role: stage the next group of 16 value rows mid-group
+  // into the other buffer, synchronise, and flush dv/db once the consumers have finished a group
+  auto iter_tail = [&](int it) {
+    if ((it & 15) == 8 && (it >> 4) + 1 < n_groups) stage((it >> 4) + 1);
+    __syncthreads();
+    if (it >= 1 && ((it - 1) & 15) == 15) {
+      const int dg = (it - 1) >> 4;
+      if (st_on && st_s < clen) {
+        TIn* dvo = (TIn*)A.dv + row0 + dg * kDG2;
+        TIn* dbo = (TIn*)A.db + row0 + dg * kDG2;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float sv = 0.f, sb_ = 0.f;
+#pragma unroll
+          for (int w = 0; w < NB; ++w) {
+            sv += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+            sb_ += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+          }
+          dvo[st_off + e] = from_f32<TIn>(sv);
+          dbo[st_off + e] = from_f32<TIn>(sb_);
+        }
+      }
+      __syncthreads();
+    }
+  };
+
+  // ------------------------------------------------------------------ producers
+  auto producer = [&](auto hfc) {
+    constexpr int HF = decltype(hfc)::value;   // token blocks 2HF, 2HF+1 (index tl)
+    bf16x8 Lop[HF ? 4 : 2];   // forward operand L[t,s], s <= t: HF=0 [tl], HF=1 [2tl+ks]
+    float kk[HF ? 16 : 8];    // k in operand layout (n = i, s = 8g+j+32ks)
+    float qq[8];              // q in result layout (t = 16tb+4g+r, n = i)
+    float dq[8];
+    float sigacc = 0.f;
+    {
+      const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb;
+      const TIn* qp = (const TIn*)a.q + ((int64_t)t0 * H + h) * dk + 16 * nb;
+      float ct[2];
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl) ct[tl] = sC[16 * (2 * HF + tl) + i];
+#pragma unroll
+      for (int ks = 0; ks <= HF; ++ks) {
+        float cs[8];
+        *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
+        *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int s = 8 * g + j + 32 * ks;
+          const bool ok = s < clen;
+          const float kv = to_f32((kp + (int64_t)(ok ? s : 0) * rs)[i]);
+          kk[ks * 8 + j] = ok ? kv : 0.f;
+#pragma unroll
+          for (int tl = 0; tl < 2; ++tl) {
+            const int t = 16 * (2 * HF + tl) + i;
+            Lop[HF ? 2 * tl + ks : tl][j] = (bf16_t)((s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f);
+          }
+        }
+      }
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = 16 * (2 * HF + tl) + 4 * g + r;
+          const bool ok = t < clen;
+          const float qv = to_f32((qp + (int64_t)(ok ? t : 0) * rs)[i]);
+          qq[tl * 4 + r] = ok ? qv : 0.f;
+          dq[tl * 4 + r] = 0.f;
+        }
+    }
+    // tile-start state of the next value row (entry of the own key column n = i), fetched one iteration ahead
+    const float* cmu = a.chunk_mu + tile_off + 16 * nb;
+    const float* cI = a.chunk_I + tile_off + 16 * nb;
+    float mu_n = cmu[i], I_n = cI[i];
+
+    for (int it = 0; it <= dv; ++it) {
+      if (it < dv) {
+        const int d = it, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
+        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
+        const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
+        const float* sDov = sSt + (buf * NST + NST - 1) * STG + dd * kVS2;
+        const float mu0 = mu_n, I0 = I_n;
+        {
+          const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
+          mu_n = (cmu + dn)[i];
+          I_n = (cI + dn)[i];
+        }
+        const float M0 = mu0 * I0, J0 = I0 - Ip;
+        if (!HF && g == 0) {
+          sMJ[(nb * 2 + (d & 1)) * 32 + i] = M0;
+          sMJ[(nb * 2 + (d & 1)) * 32 + 16 + i] = J0;
+        }
+        bf16x8 XM[HF + 1], XJ[HF + 1];
+#pragma unroll
+        for (int ks = 0; ks <= HF; ++ks) {
+          const f32x4 v0 = *(const f32x4*)&sV[8 * g + 32 * ks];
+          const f32x4 v1 = *(const f32x4*)&sV[8 * g + 32 * ks + 4];
+          const f32x4 b0 = *(const f32x4*)&sB[8 * g + 32 * ks];
+          const f32x4 b1 = *(const f32x4*)&sB[8 * g + 32 * ks + 4];
+#pragma unroll
+          for (int j = 0; j < 8; j += 2) {
+            const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
+            const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
+            const float ka = kk[ks * 8 + j], kb = kk[ks * 8 + j + 1];
+            const bf16x2 pm = pack2(ka * va, kb * vb);
+            const bf16x2 pj = pack2((ka * ba) * ka, (kb * bb) * kb);
+            XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
+            XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
+          }
+        }
+        bf16x8 PM, PJ;
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+          const int tb = 2 * HF + tl;
+          f32x4 accM = {0.f, 0.f, 0.f, 0.f};
+          f32x4 accI = {Ip, Ip, Ip, Ip};
+          accM = mfma16(Lop[HF ? 2 * tl : tl], XM[0], accM);
+          accI = mfma16(Lop[HF ? 2 * tl : tl], XJ[0], accI);
+          if (HF) {
+            accM = mfma16(Lop[2 * tl + HF], XM[HF], accM);
+            accI = mfma16(Lop[2 * tl + HF], XJ[HF], accI);
+          }
+          const f32x4 Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
+          const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
+          f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
+          if (HAS_VAR) dvv = *(const f32x4*)&sDov[16 * tb + 4 * g];
+          float dMl[4], dJl[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float Mf = fmaf(Fv[r], M0, accM[r]);
+            const float If = fmaf(Fv[r], J0, accI[r]);
+            const float rI = fast_rcp(If);
+            const float mu = Mf * rI;
+            const float q = qq[tl * 4 + r];
+            dMl[r] = (dov[r] * q) * rI;
+            dJl[r] = -(dMl[r] * mu);
+            dq[tl * 4 + r] = fmaf(mu, dov[r], dq[tl * 4 + r]);
+            if (HAS_VAR) {
+              const float wq = dvv[r] * q;          // scale*dovar*q
+              const float w = wq * q * rI;          // scale*dovar*q^2/I
+              dJl[r] = fmaf(-w, rI, dJl[r]);
+              dq[tl * 4 + r] = fmaf(2.f * wq, rI, dq[tl * 4 + r]);
+            }
+            sigacc += dJl[r];
+          }
+          const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
+          const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
+          const int o4 = tl * 4;
+          PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
+          PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
+        }
+        bf16x8* slot = sX + ((nb * 2 + (d & 1)) * 8) * 64 + lane;
+        slot[(0 + HF) * 64] = PM; slot[(2 + HF) * 64] = PJ;
+        slot[(4 + HF) * 64] = XM[HF]; slot[(6 + HF) * 64] = XJ[HF];
+      }
+      iter_tail(it);
+    }
+
+    TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb;
+#pragma unroll
+    for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 16 * (2 * HF + tl) + 4 * g + r;
+        if (t < clen) (dqp + (int64_t)t * rs)[i] = from_f32<TIn>(dq[tl * 4 + r]);
+      }
+    const float x = wave_sum(sigacc);
+    if (lane == 0) sRed[NB * kC + HF * NB + nb] = x;
+  };
+
+  // ------------------------------------------------------------------ consumers
+  auto consumer = [&](auto hfc) {
+    constexpr int HF = decltype(hfc)::value;   // column-token blocks 2HF, 2HF+1 (index sl)
+    bf16x8 Lop[6];    // reverse operand, HF=0 [2sl+p], HF=1 [sl] (p=1); strictly-lower operand, HF=0 [4+sl], HF=1 [2+2sl+ks]
+    float kr[8];      // k in result layout (s = 16sb+i, n = 4g+r)
+    float dkM[8], dkJ[8];
+    float gate[2], Fs[2];
+    {
+      const TIn* kp4 = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb;
+      float ct[2];
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) ct[sl] = sC[16 * (2 * HF + sl) + i];
+      // strictly-lower operand: column token t = 16sb + i, contraction token s = 8g + j + 32ks < t
+#pragma unroll
+      for (int ks = 0; ks <= HF; ++ks) {
+        float cs[8];
+        *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
+        *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int s = 8 * g + j + 32 * ks;
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl) {
+            const int t = 16 * (2 * HF + sl) + i;
+            Lop[HF ? 2 + 2 * sl + ks : 4 + sl][j] = (bf16_t)((s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f);
+          }
+        }
+      }
+      // reverse operand: column s = 16sb + i, contraction index (g,j) <-> token t = 16(2p + j/4) + 4g + j%4 >= s
+#pragma unroll
+      for (int p = HF; p < 2; ++p) {
+        float ctt[8];
+        *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * p + 4 * g];
+        *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * p + 16 + 4 * g];
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl) {
+          const int s = 16 * (2 * HF + sl) + i;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int t = 16 * (2 * p + (j >> 2)) + 4 * g + (j & 3);
+            Lop[HF ? sl : 2 * sl + p][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f);
+          }
+        }
+      }
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const int s = 16 * (2 * HF + sl) + i;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { kr[sl * 4 + r] = 0.f; dkM[sl * 4 + r] = 0.f; dkJ[sl * 4 + r] = 0.f; }
+        if (s < clen) load_vec<4>(kp4 + (int64_t)s * rs + 4 * g, &kr[sl * 4]);
+        gate[sl] = 0.f;
+        Fs[sl] = sF[16 * (2 * HF + sl) + i];
+      }
+    }
+    float* wDM = A.wDM + tile_off + 16 * nb;
+    float* wDJ = A.wDJ + tile_off + 16 * nb;
+    // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
+    float* pw = ((g < 2) ? sPv : sPb) + nb * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
+
+    for (int it = 0; it <= dv; ++it) {
+      if (it >= 1) {
+        const int d = it - 1, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
+        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
+        const bf16x8* slot = sX + ((nb * 2 + (d & 1)) * 8) * 64 + lane;
+        // HF=0 (column tokens 0..31): reverse needs both P halves, strictly-lower only X_0;
+        // HF=1 (column tokens 32..63): reverse needs P_1 only, strictly-lower both X halves
+        const bf16x8 PM1 = slot[1 * 64], PJ1 = slot[3 * 64], XM0 = slot[4 * 64], XJ0 = slot[6 * 64];
+        const bf16x8 Ma = slot[(HF ? 5 : 0) * 64];   // HF=0: P^M_0, HF=1: X^M_1
+        const bf16x8 Ja = slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
+        const f32x4 M0T = *(const f32x4*)&sMJ[(nb * 2 + (d & 1)) * 32 + 4 * g];
+        const f32x4 J0T = *(const f32x4*)&sMJ[(nb * 2 + (d & 1)) * 32 + 16 + 4 * g];
+        float dvp[2], dbp[2];
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl) {
+          const int sb = 2 * HF + sl;
+          f32x4 aM = {0.f, 0.f, 0.f, 0.f}, aJ = {0.f, 0.f, 0.f, 0.f};
+          f32x4 sM = {0.f, 0.f, 0.f, 0.f}, sJ = {0.f, 0.f, 0.f, 0.f};
+          if (!HF) {
+            aM = mfma16(Ma, Lop[2 * sl], aM);
+            aJ = mfma16(Ja, Lop[2 * sl], aJ);
+            aM = mfma16(PM1, Lop[2 * sl + 1], aM);
+            aJ = mfma16(PJ1, Lop[2 * sl + 1], aJ);
+            // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
+            sM = mfma16(XM0, Lop[4 + sl], sM);
+            sJ = mfma16(XJ0, Lop[4 + sl], sJ);
+          } else {
+            aM = mfma16(PM1, Lop[sl], aM);
+            aJ = mfma16(PJ1, Lop[sl], aJ);
+            sM = mfma16(XM0, Lop[2 + 2 * sl], sM);
+            sJ = mfma16(XJ0, Lop[2 + 2 * sl], sJ);
+            sM = mfma16(Ma, Lop[2 + 2 * sl + 1], sM);
+            sJ = mfma16(Ja, Lop[2 + 2 * sl + 1], sJ);
+          }
+          const float vS = sV[16 * sb + i];
+          const float bS = sB[16 * sb + i];
+          float dvs = 0.f, dbs = 0.f, gm = gate[sl];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float kv = kr[sl * 4 + r];
+            dvs = fmaf(aM[r], kv, dvs);
+            dbs = fmaf(aJ[r] * kv, kv, dbs);
+            dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
+            dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
+            const float Ss = fmaf(Fs[sl], M0T[r], sM[r]);
+            const float SJ = fmaf(Fs[sl], J0T[r], sJ[r]);
+            gm = fmaf(aM[r], Ss, gm);
+            gm = fmaf(aJ[r], SJ, gm);
+          }
+          gate[sl] = gm;
+          dvp[sl] = dvs;
+          dbp[sl] = dbs;
+          if (!HF && sl == 0 && i == 0) {
+            // carry handed to the previous tile: f_first * dM^loc at the first token
+            const f32x4 rm = {f_first * aM[0], f_first * aM[1], f_first * aM[2], f_first * aM[3]};
+            const f32x4 rj = {f_first * aJ[0], f_first * aJ[1], f_first * aJ[2], f_first * aJ[3]};
+            *(f32x4*)&(wDM + (int64_t)d * dk)[4 * g] = rm;
+            *(f32x4*)&(wDJ + (int64_t)d * dk)[4 * g] = rj;
+          }
+        }
+        pw[dd * kC] = rows4_sum_x4(dvp[0], dvp[1], dbp[0], dbp[1]);
+      }
+      iter_tail(it);
+    }
+
+    TIn* dkp = (TIn*)A.dk + ((int64_t)t0 * H + h) * dk + 16 * nb;
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl) {
+      const int s = 16 * (2 * HF + sl) + i;
+      if (s < clen) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          (dkp + (int64_t)s * rs)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
+      }
+      const float x = rows4_sum(gate[sl]);
+      if (g == 0) sRed[nb * kC + 16 * (2 * HF + sl) + i] = x;
+    }
+  };
+
+  // every role runs dv+1 iterations with the same barriers
+  if (role == 0) producer(std::integral_constant<int, 0>{});
+  else if (role == 1) producer(std::integral_constant<int, 1>{});
+  else if (role == 2) consumer(std::integral_constant<int, 0>{});
+  else consumer(std::integral_constant<int, 1>{});
+
+  __syncthreads();
+  if (tid < kC) {
+    float gm = 0.f;
+#pragma unroll
+    for (int w = 0; w < NB; ++w) gm += sRed[w * kC + tid];
+    if (tid < clen) A.wE[(int64_t)h * A.tokens + t0 + tid] = gm;
+    if (tid == 0) {
+      float sg = 0.f;
+#pragma unroll
+      for (int w = 0; w < 2 * NB; ++w) sg += sRed[NB * kC + w];
+      A.wSig[(int64_t)cidx * H + h] = sg;
+    }
+  }
+}
+
 // ----------------------------------------------------------------- carry scan
 // one thread per (sequence, head, state entry); 256 consecutive entries per block
 __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
@@ -784,17 +1204,32 @@ static BwdLayout bwd_layout(const PalDims* d) {
 template <typename TIn, int NB>
 static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   const bool var = A.c.flags & PAL_FLAG_HAS_VAR;
-  const int NT = NB * 64;
-  const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + NB);
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
-  if (lds > kMaxLds) return PAL_E_HEADDIM;
-  if (var) {
-    if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, true>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+  if constexpr (NB <= 4) {
+    // four wave roles per workgroup (see chunk_bwd_local_roles_kernel)
+    const int NT = 4 * NB * 64;
+    const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
+                       (size_t)NB * 2 * 8 * 64 * 16;
+    if (lds > kMaxLds) return PAL_E_HEADDIM;
+    if (var) {
+      if (int rc = allow_lds((const void*)&chunk_bwd_local_roles_kernel<TIn, NB, true>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_roles_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    } else {
+      if (int rc = allow_lds((const void*)&chunk_bwd_local_roles_kernel<TIn, NB, false>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_roles_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    }
   } else {
-    if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, false>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    const int NT = NB * 64;
+    const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + NB);
+    if (lds > kMaxLds) return PAL_E_HEADDIM;
+    if (var) {
+      if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, true>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    } else {
+      if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, false>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    }
   }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;

@@ -84,6 +84,33 @@ __device__ __forceinline__ void store_vec(float* p, const float* in) {
   }
 }
 
+// streaming variants for data that is touched exactly once (decode state): no reuse, so hint the
+// caches not to keep it
+template <int VW>
+__device__ __forceinline__ void load_vec_stream(const float* p, float* out) {
+  if constexpr (VW == 4) {
+    f32x4 x = __builtin_nontemporal_load((const f32x4*)p);
+    out[0] = x[0]; out[1] = x[1]; out[2] = x[2]; out[3] = x[3];
+  } else if constexpr (VW == 2) {
+    f32x2 x = __builtin_nontemporal_load((const f32x2*)p);
+    out[0] = x[0]; out[1] = x[1];
+  } else {
+    out[0] = __builtin_nontemporal_load(p);
+  }
+}
+template <int VW>
+__device__ __forceinline__ void store_vec_stream(float* p, const float* in) {
+  if constexpr (VW == 4) {
+    f32x4 x = {in[0], in[1], in[2], in[3]};
+    __builtin_nontemporal_store(x, (f32x4*)p);
+  } else if constexpr (VW == 2) {
+    f32x2 x = {in[0], in[1]};
+    __builtin_nontemporal_store(x, (f32x2*)p);
+  } else {
+    __builtin_nontemporal_store(in[0], p);
+  }
+}
+
 // ------------------------------------------------------- cross-lane helpers
 // rotate within each row of 16 lanes (DPP row_ror:N)
 template <int N>
@@ -99,11 +126,34 @@ __device__ __forceinline__ float row16_sum(float x) {
   x += row_ror<1>(x);
   return x;
 }
+// gfx950 lane swaps run in the VALU; the LDS-routed shuffles they replace cost ~64 cycles of latency each.
+// Written as inline assembly: with hipcc 7.2 the two results of the __builtin_amdgcn_permlane*_swap
+// builtins are merged into one register when both feed the same arithmetic instruction.  The s_nop
+// covers the two wait states the instruction needs after a VALU write of its operands.
+// a <- {a lanes 0-31, b lanes 0-31}, b <- {a lanes 32-63, b lanes 32-63}
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// rows of 16 lanes: a <- {a0, b0, a2, b2}, b <- {a1, b1, a3, b3}
+__device__ __forceinline__ void swap_rows(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
 // sum over the four 16-lane rows of a wave (same lane-in-row); all lanes get it
 __device__ __forceinline__ float rows4_sum(float x) {
-  x += __shfl_xor(x, 16);
-  x += __shfl_xor(x, 32);
-  return x;
+  float a = x, b = x;
+  swap_halves(a, b);
+  a += b;
+  b = a;
+  swap_rows(a, b);
+  return a + b;
+}
+// four partials, each to be summed over the four rows: the lanes of row g get the total of p_g
+__device__ __forceinline__ float rows4_sum_x4(float p0, float p1, float p2, float p3) {
+  swap_halves(p0, p2);   // rows 0,1: p0 summed over row pairs; rows 2,3: p2
+  swap_halves(p1, p3);
+  float s0 = p0 + p2, s1 = p1 + p3;
+  swap_rows(s0, s1);
+  return s0 + s1;
 }
 __device__ __forceinline__ float wave_sum(float x) { return rows4_sum(row16_sum(x)); }
 

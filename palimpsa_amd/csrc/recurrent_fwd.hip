@@ -81,8 +81,8 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
 #pragma unroll
       for (int iv = 0; iv < NV; ++iv) {
         float mu[VW], I[VW];
-        load_vec<VW>(a.init_mu + base + Map::vec_start(j, iv), mu);
-        load_vec<VW>(a.init_I + base + Map::vec_start(j, iv), I);
+        load_vec_stream<VW>(a.init_mu + base + Map::vec_start(j, iv), mu);
+        load_vec_stream<VW>(a.init_I + base + Map::vec_start(j, iv), I);
 #pragma unroll
         for (int e = 0; e < VW; ++e) {
           M[rr][iv * VW + e] = mu[e] * I[e];
@@ -171,8 +171,8 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
           I[e] = J[rr][iv * VW + e] + Ip;
           mu[e] = M[rr][iv * VW + e] * fast_rcp(I[e]);
         }
-        store_vec<VW>(a.final_mu + base + Map::vec_start(j, iv), mu);
-        store_vec<VW>(a.final_I + base + Map::vec_start(j, iv), I);
+        store_vec_stream<VW>(a.final_mu + base + Map::vec_start(j, iv), mu);
+        store_vec_stream<VW>(a.final_I + base + Map::vec_start(j, iv), I);
       }
     }
   }
@@ -229,9 +229,10 @@ extern "C" int pal_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, void*
   a.var_bf16 = d->var_dtype == PAL_DTYPE_BF16;
   a.flags = d->flags;
   a.scale = d->scale;
-  // 16 value rows per wave once that still gives every SIMD of the chip two waves
+  // long scans: 16 value rows per wave once that still gives every SIMD of the chip two waves
   const int64_t waves16 = (int64_t)d->n_seqs * d->n_heads * (d->dv / 16);
-  const int rd = (waves16 >= 2048) ? 4 : 1;
+  // decode (a handful of tokens) is pure state streaming: many small waves keep more loads in flight
+  const int rd = (d->seq_len > 4 && waves16 >= 2048) ? 4 : 1;
   hipStream_t s = (hipStream_t)stream;
   if (d->dtype == PAL_DTYPE_BF16) return launch_dtype<bf16_t>(a, rd, s);
   return launch_dtype<float>(a, rd, s);
