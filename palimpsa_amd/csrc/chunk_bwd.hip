@@ -481,15 +481,18 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   auto stage = [&](int dg) {
     if (!st_on) return;
     float st[NST][4];
+    // the lane offset is made opaque here so that no per-lane 64-bit address is kept across the loop
+    unsigned off = st_off;
+    asm volatile("" : "+v"(off));
     if (st_s < clen) {
-      load_vec<4>(vp + dg * kDG2 + st_off, st[0]);
-      load_vec<4>(bp + dg * kDG2 + st_off, st[1]);
-      load_vec<4>(dop + dg * kDG2 + st_off, st[2]);
+      load_vec<4>(vp + dg * kDG2 + off, st[0]);
+      load_vec<4>(bp + dg * kDG2 + off, st[1]);
+      load_vec<4>(dop + dg * kDG2 + off, st[2]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) st[2][e] *= scale;
       if (HAS_VAR) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) st[NST - 1][e] = scale * load_rt(A.d_o_var, row0 + dg * kDG2 + st_off + e, a.var_bf16);
+        for (int e = 0; e < 4; ++e) st[NST - 1][e] = scale * load_rt(A.d_o_var, row0 + dg * kDG2 + off + e, a.var_bf16);
       }
     } else {
 #pragma unroll
@@ -519,19 +522,22 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     if (it >= 1 && ((it - 1) & 15) == 15) {
       const int dg = (it - 1) >> 4;
       if (st_on && st_s < clen) {
-        TIn* dvo = (TIn*)A.dv + row0 + dg * kDG2;
-        TIn* dbo = (TIn*)A.db + row0 + dg * kDG2;
+        unsigned off = st_off;
+        asm volatile("" : "+v"(off));
+        TIn* dvo = (TIn*)A.dv + row0 + dg * kDG2 + off;
+        TIn* dbo = (TIn*)A.db + row0 + dg * kDG2 + off;
+        float sv[4], sb_[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float sv = 0.f, sb_ = 0.f;
+          sv[e] = 0.f; sb_[e] = 0.f;
 #pragma unroll
           for (int w = 0; w < NB; ++w) {
-            sv += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
-            sb_ += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+            sv[e] += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+            sb_[e] += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
           }
-          dvo[st_off + e] = from_f32<TIn>(sv);
-          dbo[st_off + e] = from_f32<TIn>(sb_);
         }
+        store_vec<4>(dvo, sv);
+        store_vec<4>(dbo, sb_);
       }
       __syncthreads();
     }

@@ -169,6 +169,18 @@ __device__ __forceinline__ bf16x2 pack2(float lo, float hi) {
   f32x2 x = {lo, hi};
   return __builtin_convertvector(x, bf16x2);
 }
+template <int VW>
+__device__ __forceinline__ void store_vec(bf16_t* p, const float* in) {
+  if constexpr (VW == 4) {
+    const bf16x2 a = pack2(in[0], in[1]), b = pack2(in[2], in[3]);
+    const bf16x4 x = {a[0], a[1], b[0], b[1]};
+    *(bf16x4*)p = x;
+  } else if constexpr (VW == 2) {
+    *(bf16x2*)p = pack2(in[0], in[1]);
+  } else {
+    *p = (bf16_t)in[0];
+  }
+}
 
 // ------------------------------------------------------------------ host
 #define PAL_HIP_LAUNCH_CHECK()                 \
