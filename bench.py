@@ -28,6 +28,10 @@ if ROOT not in sys.path:
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E peak
 CHUNK = 64
+# HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
+# from inside this process, so the figures are carried here and are stale once those kernels change.
+MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 479.7e6, "recurrent_fwd_kernel": 1111.9e6}
 
 
 def make_inputs(torch, B, T, H, dk, dv, seed, dtype):
@@ -93,7 +97,7 @@ def bench_chunk(torch, dev, steps, warmup):
         "bound": "mfma", "kernel": "chunk_bwd_local_kernel",
         "achieved": achieved, "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_MFMA_TFLOPS,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES["chunk_bwd_local_kernel"],
         "algorithmic_flops_per_launch": flops_local,
         "avg_launch_ms": avg_local_ms,
         "step_frac": flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
@@ -148,7 +152,8 @@ def bench_decode(torch, dev, steps):
         "steps": steps, "tokens_per_s": B * steps / elapsed, "ms_per_step": elapsed * 1e3 / steps,
         "hbm_gbs_wall": bytes_step * steps / elapsed / 1e9,
         "roofline": {"bound": "hbm", "kernel": "recurrent_fwd_kernel", "achieved": gbs_kernel, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": gbs_kernel / PEAK_HBM_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": gbs_kernel / PEAK_HBM_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES["recurrent_fwd_kernel"],
                      "algorithmic_bytes_per_launch": bytes_step, "avg_launch_ms": avg_ms},
     }
 
@@ -183,6 +188,8 @@ def main():
     ap.add_argument("--decode-steps", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the operator shards over batch/heads without any "
@@ -195,6 +202,14 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        # a copy kernel of known size: 1 GiB read + 1 GiB written per launch
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     res = bench_chunk(torch, dev, args.steps, args.warmup)
     extra = {"kernels": res["kernels"], "ms_per_step_no_events": res["ms_per_step_no_events"]}
     if not args.no_decode:
