@@ -899,10 +899,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const int dmax = dk > dv ? dk : dv;
   float* sAs = smem;                       // [64] decay from token s to the end of the tile
   float* sW4 = sAs + kC;                   // [8]
-  float* sBt = sW4 + 8;                    // [64][32] beta of the carry terms, one slot per work item
-  float* sO1 = sBt + kC * 32;                   // [64][kOS..] dv^carry, later dk^carry
-  float* sO2 = sO1 + kC * (dmax + 4);      // [64][..]   db^carry
-  bf16_t* sRT = (bf16_t*)(sO2 + kC * (dmax + 4));   // [2][dk][dv + 8] R_M^T, R_J^T in bf16
+  float* sBt = sW4 + 8;                    // [64][dv/8] beta of the carry terms, one slot per work item
+  float* sO1 = sBt + kC * (dv >> 3);       // [64][OS] dk^carry, later dv^carry
+  // R_M^T, R_J^T in bf16 [2][dk][dv + 8] for the dk products; the same bytes hold db^carry [64][OS] afterwards
+  float* sO2 = sO1 + kC * (dmax + 4);
+  bf16_t* sRT = (bf16_t*)sO2;
   const int RS = dv + 8;
   const int OS = dmax + 4;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
@@ -960,6 +961,89 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const float as = sAs[srow];
   const int64_t tokA = ((int64_t)(t0 + (row_ok ? srow : 0)) * H + h);
   const int64_t tok0 = ((int64_t)t0 * H + h);
+
+  // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
+  {
+    const int KS = (dv + 31) / 32;
+    bf16x8 A3[8], A4[8];
+    const TIn* vp = (const TIn*)a.v + tokA * dv;
+    const TIn* bp = (const TIn*)a.b + tokA * dv;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks < KS) {
+        const int d0 = 8 * g + 32 * ks;
+        float vv[8], bb[8];
+        if (row_ok && d0 < dv) {
+          load_vec<4>(vp + d0, vv); load_vec<4>(vp + d0 + 4, vv + 4);
+          load_vec<4>(bp + d0, bb); load_vec<4>(bp + d0 + 4, bb + 4);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { vv[j] = 0.f; bb[j] = 0.f; }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          A3[ks][j] = (bf16_t)(as * vv[j]);
+          A4[ks][j] = (bf16_t)(as * bb[j]);
+        }
+      }
+    }
+    const TIn* kin = (const TIn*)a.k + tok0 * dk;
+    // k of the result entries (row s = 16w + 4g + r, column n = 16nbk + i), fetched one step ahead
+    auto load_k4 = [&](int nbk, float* kv) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int s = 16 * w + 4 * g + r;
+        kv[r] = (s < clen) ? to_f32(kin[(int64_t)s * H * dk + 16 * nbk + i]) : 0.f;
+      }
+    };
+    float kcur[4], knext[4] = {0.f, 0.f, 0.f, 0.f};
+    load_k4(0, kcur);
+    const int NBK = dk / 16;
+    for (int nbk = 0; nbk < NBK; ++nbk) {
+      if (nbk + 1 < NBK) load_k4(nbk + 1, knext);
+      f32x4 accM = {0.f, 0.f, 0.f, 0.f}, accJ = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks < KS) {
+          const int d0 = 8 * g + 32 * ks;
+          bf16x8 B3, B4;
+          if (d0 < dv) {
+            B3 = *(const bf16x8*)&sRT[(16 * nbk + i) * RS + d0];
+            B4 = *(const bf16x8*)&sRT[(dk + 16 * nbk + i) * RS + d0];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { B3[j] = (bf16_t)0.f; B4[j] = (bf16_t)0.f; }
+          }
+          accM = mfma16(A3[ks], B3, accM);
+          accJ = mfma16(A4[ks], B4, accJ);
+        }
+      }
+      // rows s = 16w + 4g + r, column n = 16nbk + i
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int s = 16 * w + 4 * g + r;
+        sO1[s * OS + 16 * nbk + i] = fmaf(2.f * kcur[r], accJ[r], accM[r]);
+        kcur[r] = knext[r];
+      }
+    }
+  }
+  __syncthreads();
+  {
+    const int groups = dk >> 3;
+    TIn* dko = (TIn*)A.dk + tok0 * dk;
+    for (int idx = tid; idx < kC * groups; idx += 256) {
+      const int c8 = idx % groups, s = idx / groups;
+      if (s < clen) {
+        const int64_t off = (int64_t)s * H * dk + 8 * c8;
+        float gk[8];
+        load_vec<4>(dko + off, gk); load_vec<4>(dko + off + 4, gk + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) gk[e] += sO1[s * OS + 8 * c8 + e];
+        store_vec<4>(dko + off, gk); store_vec<4>(dko + off + 4, gk + 4);
+      }
+    }
+  }
+  __syncthreads();   // sO1 and the R^T bytes are free again
 
   // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
   {
@@ -1041,9 +1125,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
           const float cv = sO1[s * OS + 8 * c8 + e], cb = sO2[s * OS + 8 * c8 + e];
           beta = fmaf(xv[e], cv, beta);
           beta = fmaf(xb[e], cb, beta);
-          dvo[off + e] = from_f32<TIn>(gv[e] + cv);
-          dbo[off + e] = from_f32<TIn>(gb[e] + cb);
+          gv[e] += cv;
+          gb[e] += cb;
         }
+        store_vec<4>(dvo + off, gv); store_vec<4>(dvo + off + 4, gv + 4);
+        store_vec<4>(dbo + off, gb); store_vec<4>(dbo + off + 4, gb + 4);
       }
       sBt[idx] = beta;
     }
@@ -1052,75 +1138,6 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       float bsum = 0.f;
       for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[tid * groups + c8];   // fixed order
       A.wBc[(int64_t)h * A.tokens + t0 + tid] = bsum;
-    }
-  }
-
-  // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
-  {
-    const int KS = (dv + 31) / 32;
-    bf16x8 A3[8], A4[8];
-    const TIn* vp = (const TIn*)a.v + tokA * dv;
-    const TIn* bp = (const TIn*)a.b + tokA * dv;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      if (ks < KS) {
-        const int d0 = 8 * g + 32 * ks;
-        float vv[8], bb[8];
-        if (row_ok && d0 < dv) {
-          load_vec<4>(vp + d0, vv); load_vec<4>(vp + d0 + 4, vv + 4);
-          load_vec<4>(bp + d0, bb); load_vec<4>(bp + d0 + 4, bb + 4);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) { vv[j] = 0.f; bb[j] = 0.f; }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          A3[ks][j] = (bf16_t)(as * vv[j]);
-          A4[ks][j] = (bf16_t)(as * bb[j]);
-        }
-      }
-    }
-    const TIn* kin = (const TIn*)a.k + tok0 * dk;
-    for (int nbk = 0; nbk < dk / 16; ++nbk) {
-      f32x4 accM = {0.f, 0.f, 0.f, 0.f}, accJ = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        if (ks < KS) {
-          const int d0 = 8 * g + 32 * ks;
-          bf16x8 B3, B4;
-          if (d0 < dv) {
-            B3 = *(const bf16x8*)&sRT[(16 * nbk + i) * RS + d0];
-            B4 = *(const bf16x8*)&sRT[(dk + 16 * nbk + i) * RS + d0];
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { B3[j] = (bf16_t)0.f; B4[j] = (bf16_t)0.f; }
-          }
-          accM = mfma16(A3[ks], B3, accM);
-          accJ = mfma16(A4[ks], B4, accJ);
-        }
-      }
-      // rows s = 16w + 4g + r, column n = 16nbk + i
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int s = 16 * w + 4 * g + r;
-        const float kv = (s < clen) ? to_f32(kin[(int64_t)s * H * dk + 16 * nbk + i]) : 0.f;
-        sO1[s * OS + 16 * nbk + i] = fmaf(2.f * kv, accJ[r], accM[r]);
-      }
-    }
-  }
-  __syncthreads();
-  {
-    const int groups = dk >> 3;
-    TIn* dko = (TIn*)A.dk + tok0 * dk;
-    for (int idx = tid; idx < kC * groups; idx += 256) {
-      const int c8 = idx % groups, s = idx / groups;
-      if (s < clen) {
-        const int64_t off = (int64_t)s * H * dk + 8 * c8;
-        float gk[8];
-        load_vec<4>(dko + off, gk); load_vec<4>(dko + off + 4, gk + 4);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dko[off + e] = from_f32<TIn>(gk[e] + sO1[s * OS + 8 * c8 + e]);
-      }
     }
   }
 }
@@ -1314,7 +1331,8 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
     const int dmax = dd.dk > dd.dv ? dd.dk : dd.dv;
-    const size_t lds = sizeof(float) * (kC + 8 + kC * 32 + 2 * (size_t)kC * (dmax + 4)) + 2 * (size_t)2 * dd.dk * (dd.dv + 8);
+    const size_t rt_bytes = 2 * (size_t)2 * dd.dk * (dd.dv + 8), o2_bytes = sizeof(float) * kC * (dmax + 4);
+    const size_t lds = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3) + (size_t)kC * (dmax + 4)) + (rt_bytes > o2_bytes ? rt_bytes : o2_bytes);
     if (lds > kMaxLds) return PAL_E_HEADDIM;
     if (bf) {
       if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<bf16_t>, lds)) return rc2;
