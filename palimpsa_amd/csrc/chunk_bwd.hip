@@ -60,381 +60,22 @@ constexpr int kDG2 = 16;
 __device__ __forceinline__ constexpr int lidx2(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
 __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2 * sb + p : 4 + (sb - 2); }
 
-// ---------------------------------------------------------------- local pass
-template <typename TIn, int NB, bool HAS_VAR>
-__global__ __launch_bounds__(NB * 64) void chunk_bwd_local_kernel(BwdArgs A) {
-  const ChunkArgs& a = A.c;
-  extern __shared__ float smem[];
-  constexpr int NST = HAS_VAR ? 4 : 3;  // staged tensors: v, b, do, (dovar)
-  constexpr int NT = NB * 64;
-  constexpr int STG = kDG2 * kVS2;
-  constexpr int NITEM = (kC * kDG2 / 4 + NT - 1) / NT;
-  float* sC = smem;                      // [64] running log2 decay
-  float* sF = sC + kC;                   // [64] 2^c
-  float* sSt = sF + kC;                  // [2][NST][16][kVS2]
-  float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
-  float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
-  float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [NB] sums of dJloc
-  const int tid = threadIdx.x, lane = tid & 63, nb = tid >> 6, i = lane & 15, g = lane >> 4;
-  const int H = a.H, dk = a.dk, dv = a.dv;
-  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
-  int seq, t0, clen, cis;
-  chunk_lookup(a, cidx, seq, t0, clen, cis);
-  const float Ip = a.Ip[h];
-  const float gh = a.g[h] * kLog2e;
-  const float scale = a.scale;
-
-  if (nb == 0) {
-    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
-    const float c = wave_inclusive_scan(-gt * gh, lane);
-    sC[lane] = c;
-    sF[lane] = fast_exp2(c);
-    if (lane == 63) A.wFtot[(int64_t)cidx * H + h] = c;
-  }
-  const int64_t row0 = ((int64_t)t0 * H + h) * dv;
-  const TIn* vp = (const TIn*)a.v + row0;
-  const TIn* bp = (const TIn*)a.b + row0;
-  const TIn* dop = (const TIn*)A.d_o + row0;
-  float st[NST][NITEM][4];
-  auto stage_load = [&](int dg) {
-#pragma unroll
-    for (int it = 0; it < NITEM; ++it) {
-      const int idx = tid + it * NT;
-      const int s = idx >> 2, dq4 = idx & 3;
-      if (idx < kC * kDG2 / 4 && s < clen) {
-        const int64_t off = (int64_t)s * H * dv + dg * kDG2 + 4 * dq4;
-        load_vec<4>(vp + off, st[0][it]);
-        load_vec<4>(bp + off, st[1][it]);
-        load_vec<4>(dop + off, st[2][it]);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) st[2][it][e] *= scale;
-        if (HAS_VAR) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) st[NST - 1][it][e] = scale * load_rt(A.d_o_var, row0 + off + e, a.var_bf16);
-        }
-      } else {
-#pragma unroll
-        for (int x = 0; x < NST; ++x)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) st[x][it][e] = 0.f;
-      }
-    }
-  };
-  auto stage_store = [&](int buf) {
-#pragma unroll
-    for (int it = 0; it < NITEM; ++it) {
-      const int idx = tid + it * NT;
-      const int s = idx >> 2, dq4 = idx & 3;
-      if (idx < kC * kDG2 / 4) {
-#pragma unroll
-        for (int x = 0; x < NST; ++x)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * dq4 + e) * kVS2 + s] = st[x][it][e];
-      }
-    }
-  };
-  stage_load(0);
-  stage_store(0);
-  __syncthreads();
-
-  // ---- per-wave constants of this tile
-  bf16x8 Lr[6], Lrev[6], Ls[6];
-  float kA[2][8], kk[2][8];
-  {
-    float ct[4];
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb) ct[tb] = sC[16 * tb + i];
-    const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      float cs[8];
-      *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
-      *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int s = 8 * g + j + 32 * ks;
-        const bool ok = s < clen;
-        const float kv = to_f32(kp[(int64_t)(ok ? s : 0) * H * dk]);
-        kA[ks][j] = ok ? kv : 0.f;
-        kk[ks][j] = kA[ks][j] * kA[ks][j];
-#pragma unroll
-        for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
-          const int t = 16 * tb + i;
-          const float lv = fast_exp2(ct[tb] - cs[j]);
-          Lr[lidx2(tb, ks)][j] = (bf16_t)((s <= t) ? lv : 0.f);
-          Ls[lidx2(tb, ks)][j] = (bf16_t)((s < t) ? lv : 0.f);   // same (i,g,j) roles with s,t swapped in name
-        }
-      }
-    }
-    // reverse operand: column s = 16sb + i, k index (g,j) <-> token t = 16(2p + j/4) + 4g + j%4
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      float ctt[8];
-      *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * p + 4 * g];
-      *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * p + 16 + 4 * g];
-#pragma unroll
-      for (int sb = 0; sb < (p ? 4 : 2); ++sb) {
-        const int s = 16 * sb + i;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int t = 16 * (2 * p + (j >> 2)) + 4 * g + (j & 3);
-          Lrev[ridx(sb, p)][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sb]) : 0.f);
-        }
-      }
-    }
-  }
-  float qP[4][4], kB[4][4];
-  {
-    const TIn* qp = (const TIn*)a.q + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
-    const TIn* kp4 = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + 4 * g;
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = 16 * tb + 4 * g + r;
-        const bool ok = t < clen;
-        const float qv = to_f32(qp[(int64_t)(ok ? t : 0) * H * dk]);
-        qP[tb][r] = ok ? qv : 0.f;
-      }
-      const int s = 16 * tb + i;
-      if (s < clen) {
-        load_vec<4>(kp4 + (int64_t)s * H * dk, kB[tb]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) kB[tb][r] = 0.f;
-      }
-    }
-  }
-  float dqa[4][4], dkM[4][4], dkJ[4][4], gam[4], FsB[4];
-  float sigacc = 0.f;
-#pragma unroll
-  for (int x = 0; x < 4; ++x) {
-    gam[x] = 0.f;
-    FsB[x] = sF[16 * x + i];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) { dqa[x][r] = 0.f; dkM[x][r] = 0.f; dkJ[x][r] = 0.f; }
-  }
-
-  const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
-  const float* cmu = a.chunk_mu + tile_off + 16 * nb + i;
-  const float* cI = a.chunk_I + tile_off + 16 * nb + i;
-  const float* cmuT = a.chunk_mu + tile_off + 16 * nb + 4 * g;   // same state, 4 key columns per lane group
-  const float* cIT = a.chunk_I + tile_off + 16 * nb + 4 * g;
-  float* wDM = A.wDM + tile_off + 16 * nb + 4 * g;
-  float* wDJ = A.wDJ + tile_off + 16 * nb + 4 * g;
-  const float f_first = fast_exp2(sC[0]);
-
-  // tile-start state of the next value row is fetched one iteration ahead
-  float mu0_n = cmu[0], I0_n = cI[0];
-  f32x4 muT_n = *(const f32x4*)cmuT, IT_n = *(const f32x4*)cIT;
-
-  const int n_groups = dv / kDG2;
-  for (int dg = 0; dg < n_groups; ++dg) {
-    const int buf = dg & 1;
-    const float* sV = sSt + (buf * NST + 0) * STG;
-    const float* sB = sSt + (buf * NST + 1) * STG;
-    const float* sDo = sSt + (buf * NST + 2) * STG;
-    const float* sDov = sSt + (buf * NST + NST - 1) * STG;
-    if (dg + 1 < n_groups) stage_load(dg + 1);
-    for (int dd = 0; dd < kDG2; ++dd) {
-      const int d = dg * kDG2 + dd;
-      const float mu0 = mu0_n, I0 = I0_n;
-      const f32x4 muT = muT_n, IT = IT_n;
-      {
-        const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
-        mu0_n = cmu[dn];
-        I0_n = cI[dn];
-        muT_n = *(const f32x4*)(cmuT + dn);
-        IT_n = *(const f32x4*)(cIT + dn);
-      }
-      const float M0 = mu0 * I0, J0 = I0 - Ip;
-      bf16x8 XM[2], XJ[2];
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const f32x4 v0 = *(const f32x4*)&sV[dd * kVS2 + 8 * g + 32 * ks];
-        const f32x4 v1 = *(const f32x4*)&sV[dd * kVS2 + 8 * g + 32 * ks + 4];
-        const f32x4 b0 = *(const f32x4*)&sB[dd * kVS2 + 8 * g + 32 * ks];
-        const f32x4 b1 = *(const f32x4*)&sB[dd * kVS2 + 8 * g + 32 * ks + 4];
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
-          const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
-          const bf16x2 pm = pack2(kA[ks][j] * va, kA[ks][j + 1] * vb);
-          const bf16x2 pj = pack2(kk[ks][j] * ba, kk[ks][j + 1] * bb);
-          XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
-          XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
-        }
-      }
-      // ---- phase A: states of this value row for all 64 tokens, local gradients
-      bf16x8 PM[2], PJ[2];
-#pragma unroll
-      for (int tb = 0; tb < 4; ++tb) {
-        f32x4 accM = {0.f, 0.f, 0.f, 0.f};
-        f32x4 accI = {Ip, Ip, Ip, Ip};
-        accM = mfma16(Lr[lidx2(tb, 0)], XM[0], accM);
-        accI = mfma16(Lr[lidx2(tb, 0)], XJ[0], accI);
-        if (tb >= 2) {
-          accM = mfma16(Lr[lidx2(tb, 1)], XM[1], accM);
-          accI = mfma16(Lr[lidx2(tb, 1)], XJ[1], accI);
-        }
-        const f32x4 Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
-        const f32x4 dov = *(const f32x4*)&sDo[dd * kVS2 + 16 * tb + 4 * g];
-        f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
-        if (HAS_VAR) dvv = *(const f32x4*)&sDov[dd * kVS2 + 16 * tb + 4 * g];
-        float dMl[4], dJl[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float Mf = fmaf(Fv[r], M0, accM[r]);
-          const float If = fmaf(Fv[r], J0, accI[r]);
-          const float rI = fast_rcp(If);
-          const float mu = Mf * rI;
-          const float q = qP[tb][r];
-          dMl[r] = (dov[r] * q) * rI;
-          dJl[r] = -(dMl[r] * mu);
-          dqa[tb][r] = fmaf(mu, dov[r], dqa[tb][r]);
-          if (HAS_VAR) {
-            const float wq = dvv[r] * q;          // scale*dovar*q
-            const float w = wq * q * rI;          // scale*dovar*q^2/I
-            dJl[r] = fmaf(-w, rI, dJl[r]);
-            dqa[tb][r] = fmaf(2.f * wq, rI, dqa[tb][r]);
-          }
-          sigacc += dJl[r];
-        }
-        const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
-        const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
-        const int o4 = (tb & 1) * 4;
-        PM[tb >> 1][o4 + 0] = m0[0]; PM[tb >> 1][o4 + 1] = m0[1]; PM[tb >> 1][o4 + 2] = m1[0]; PM[tb >> 1][o4 + 3] = m1[1];
-        PJ[tb >> 1][o4 + 0] = j0[0]; PJ[tb >> 1][o4 + 1] = j0[1]; PJ[tb >> 1][o4 + 2] = j1[0]; PJ[tb >> 1][o4 + 3] = j1[1];
-      }
-      // ---- phase B: dM^loc[n, s] = sum_t dMloc[t, n] L[t, s], accumulators -> operands directly
-#pragma unroll
-      for (int sb = 0; sb < 4; ++sb) {
-        f32x4 aM = {0.f, 0.f, 0.f, 0.f}, aJ = {0.f, 0.f, 0.f, 0.f};
-        if (sb < 2) {
-          aM = mfma16(PM[0], Lrev[ridx(sb, 0)], aM);
-          aJ = mfma16(PJ[0], Lrev[ridx(sb, 0)], aJ);
-        }
-        aM = mfma16(PM[1], Lrev[ridx(sb, 1)], aM);
-        aJ = mfma16(PJ[1], Lrev[ridx(sb, 1)], aJ);
-        // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
-        f32x4 sM = {0.f, 0.f, 0.f, 0.f}, sJ = {0.f, 0.f, 0.f, 0.f};
-        sM = mfma16(XM[0], Ls[lidx2(sb, 0)], sM);
-        sJ = mfma16(XJ[0], Ls[lidx2(sb, 0)], sJ);
-        if (sb >= 2) {
-          sM = mfma16(XM[1], Ls[lidx2(sb, 1)], sM);
-          sJ = mfma16(XJ[1], Ls[lidx2(sb, 1)], sJ);
-        }
-        const float vS = sV[dd * kVS2 + 16 * sb + i];
-        const float bS = sB[dd * kVS2 + 16 * sb + i];
-        float dvp = 0.f, dbp = 0.f;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float kv = kB[sb][r];
-          dvp = fmaf(aM[r], kv, dvp);
-          dbp = fmaf(aJ[r] * kv, kv, dbp);
-          dkM[sb][r] = fmaf(aM[r], vS, dkM[sb][r]);
-          dkJ[sb][r] = fmaf(aJ[r], bS, dkJ[sb][r]);
-          const float Ss = fmaf(FsB[sb], muT[r] * IT[r], sM[r]);
-          const float SJ = fmaf(FsB[sb], IT[r] - Ip, sJ[r]);
-          gam[sb] = fmaf(aM[r], Ss, gam[sb]);
-          gam[sb] = fmaf(aJ[r], SJ, gam[sb]);
-        }
-        dvp = rows4_sum(dvp);
-        dbp = rows4_sum(dbp);
-        if (g == 0) {
-          sPv[(nb * kDG2 + dd) * kC + 16 * sb + i] = dvp;
-          sPb[(nb * kDG2 + dd) * kC + 16 * sb + i] = dbp;
-        }
-        if (sb == 0 && i == 0) {
-          // carry handed to the previous tile: f_first * dM^loc at the first token
-          const f32x4 rm = {f_first * aM[0], f_first * aM[1], f_first * aM[2], f_first * aM[3]};
-          const f32x4 rj = {f_first * aJ[0], f_first * aJ[1], f_first * aJ[2], f_first * aJ[3]};
-          *(f32x4*)(wDM + (int64_t)d * dk) = rm;
-          *(f32x4*)(wDJ + (int64_t)d * dk) = rj;
-        }
-      }
-    }
-    __syncthreads();
-    // flush the tile-local dv, db of this group; work item = (token s, 4 value rows)
-#pragma unroll
-    for (int it = 0; it < NITEM; ++it) {
-      const int idx = tid + it * NT;
-      const int s = idx >> 2, dq4 = idx & 3;
-      if (idx < kC * kDG2 / 4 && s < clen) {
-        const int64_t off = row0 + (int64_t)s * H * dv + dg * kDG2 + 4 * dq4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float sv = 0.f, sb_ = 0.f;
-#pragma unroll
-          for (int w = 0; w < NB; ++w) {
-            sv += sPv[(w * kDG2 + 4 * dq4 + e) * kC + s];
-            sb_ += sPb[(w * kDG2 + 4 * dq4 + e) * kC + s];
-          }
-          ((TIn*)A.dv)[off + e] = from_f32<TIn>(sv);
-          ((TIn*)A.db)[off + e] = from_f32<TIn>(sb_);
-        }
-      }
-    }
-    if (dg + 1 < n_groups) stage_store((dg + 1) & 1);
-    __syncthreads();
-  }
-
-  // ---- tile end: dq (final), tile-local dk
-  {
-    TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
-    TIn* dkp = (TIn*)A.dk + ((int64_t)t0 * H + h) * dk + 16 * nb + 4 * g;
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = 16 * tb + 4 * g + r;
-        if (t < clen) dqp[(int64_t)t * H * dk] = from_f32<TIn>(dqa[tb][r]);
-      }
-      const int s = 16 * tb + i;
-      if (s < clen) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          dkp[(int64_t)s * H * dk + r] = from_f32<TIn>(fmaf(2.f * kB[tb][r], dkJ[tb][r], dkM[tb][r]));
-      }
-    }
-  }
-  // ---- local part of d log f per token, tile sum of dJloc
-#pragma unroll
-  for (int sb = 0; sb < 4; ++sb) {
-    const float x = rows4_sum(gam[sb]);
-    if (g == 0) sRed[nb * kC + 16 * sb + i] = x;
-  }
-  {
-    const float x = wave_sum(sigacc);
-    if (lane == 0) sRed[NB * kC + nb] = x;
-  }
-  __syncthreads();
-  if (tid < kC) {
-    float gm = 0.f;
-#pragma unroll
-    for (int w = 0; w < NB; ++w) gm += sRed[w * kC + tid];
-    if (tid < clen) A.wE[(int64_t)h * A.tokens + t0 + tid] = gm;
-    if (tid == 0) {
-      float sg = 0.f;
-#pragma unroll
-      for (int w = 0; w < NB; ++w) sg += sRed[NB * kC + w];
-      A.wSig[(int64_t)cidx * H + h] = sg;
-    }
-  }
-}
-
 // ------------------------------------------------- local pass, four wave roles
-// Same arithmetic as chunk_bwd_local_kernel, organised for four waves per SIMD: one wave issues a
-// VALU instruction every 5-9 cycles at best while the SIMD can start one every 2-3, so the tile's
-// work is cut into roles small enough for 128 registers.  A workgroup has 4*NB waves; wave = role*NB + nb.
+// One workgroup per (tile, head).  For every value row d the tile recomputes M_t, I_t for its 64 tokens
+// (orientation [t, n]), forms dMloc/dJloc and dq, contracts them backwards in time (dM^loc[n, s]) and
+// runs the dv/db/dk/gate epilogue on the result.
+// Organised for four waves per SIMD: one wave issues a VALU instruction every 5-9 cycles at best while
+// the SIMD can start one every 2-3, so the work on a block of 16 key columns is cut into four roles
+// small enough for 128 registers each.  A workgroup has 4*NB waves; wave = role*NB + (column block).
 //   roles 0/1 ("producers", token blocks 0-1 / 2-3): recompute the states of one value row for 16 key
 //     columns, form dMloc/dJloc and dq, and leave packed bf16 operands in an LDS slot:
 //     role 0 writes P^M_0, P^J_0, X^M_0, X^J_0 (tokens 0..31), role 1 the halves for tokens 32..63;
 //   roles 2/3 ("consumers", token blocks 0-1 / 2-3 of the column token s): pick the slot up one iteration
 //     later and do the reverse contraction, the strictly-lower product and the dv/db/dk/gate epilogue.
-// The roles keep their per-tile constants and accumulators in the same register arrays (Lop, R0..R3)
-// with role-specific meaning, so that the allocator does not reserve space for all of them at once.
-template <typename TIn, int NB, bool HAS_VAR>
+// Every role has its own loop (its own register allocation) with the same sequence of barriers.
+// NB <= 4 column blocks are in flight at a time (16 waves); a wider head dim takes several passes over
+// the tile, the later ones adding their dv/db/gate contributions to those of the earlier ones.
+template <typename TIn, int NB, bool HAS_VAR, bool MULTI>
 __global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(4)))
 void chunk_bwd_local_roles_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
@@ -449,10 +90,13 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [2*NB] sums of dJloc (padded to 16 floats)
   float* sMJ = sRed + NB * kC + 16;      // [NB][2 slots][2][16] tile-start M_0, J_0 of the row in flight
   bf16x8* sX = (bf16x8*)(sMJ + NB * 64);   // [NB][2 slots][8 operands][64 lanes]
-  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int tid = threadIdx.x;
+  int lane = tid & 63, i = lane & 15, g = lane >> 4;   // re-derived per pass from an opaque copy, see below
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: role branches are scalar
-  const int role = wave / NB, nb = wave - role * NB;
+  const int role = wave / NB, nbl = wave - role * NB;   // nbl: column block inside the current group
   const int H = a.H, dk = a.dk, dv = a.dv;
+  // NB blocks of 16 key columns are handled at a time; wider heads take several passes over the tile
+  const int nb_total = dk >> 4, n_pass = MULTI ? (nb_total + NB - 1) / NB : 1;   // MULTI = false: dk == 16*NB
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
   chunk_lookup(a, cidx, seq, t0, clen, cis);
@@ -506,13 +150,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * st_q + e) * kVS2 + st_s] = st[x][e];
   };
-  stage(0);
-  __syncthreads();
-
   const int64_t rs = (int64_t)H * dk;   // token stride of q, k
   const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
   const int n_groups = dv / kDG2;
-  const float f_first = fast_exp2(sC[0]);
+  int pass = 0, nb = nbl, n_act = NB;   // set per pass: global column block of this wave, active blocks
 
   // end of one iteration, identical for every role: stage the next group of 16 value rows mid-group
   // into the other buffer, synchronise, and flush dv/db once the consumers have finished a group
@@ -526,14 +167,19 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         asm volatile("" : "+v"(off));
         TIn* dvo = (TIn*)A.dv + row0 + dg * kDG2 + off;
         TIn* dbo = (TIn*)A.db + row0 + dg * kDG2 + off;
-        float sv[4], sb_[4];
+        float sv[4] = {0.f, 0.f, 0.f, 0.f}, sb_[4] = {0.f, 0.f, 0.f, 0.f};
+        if (MULTI && pass > 0) {   // later passes add to what the earlier column groups left
+          load_vec<4>(dvo, sv);
+          load_vec<4>(dbo, sb_);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          sv[e] = 0.f; sb_[e] = 0.f;
 #pragma unroll
           for (int w = 0; w < NB; ++w) {
-            sv[e] += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
-            sb_[e] += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+            if (!MULTI || w < n_act) {
+              sv[e] += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+              sb_[e] += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+            }
           }
         }
         store_vec<4>(dvo, sv);
@@ -606,8 +252,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         }
         const float M0 = mu0 * I0, J0 = I0 - Ip;
         if (!HF && g == 0) {
-          sMJ[(nb * 2 + (d & 1)) * 32 + i] = M0;
-          sMJ[(nb * 2 + (d & 1)) * 32 + 16 + i] = J0;
+          sMJ[(nbl * 2 + (d & 1)) * 32 + i] = M0;
+          sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + i] = J0;
         }
         bf16x8 XM[HF + 1], XJ[HF + 1];
 #pragma unroll
@@ -668,7 +314,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
           PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
         }
-        bf16x8* slot = sX + ((nb * 2 + (d & 1)) * 8) * 64 + lane;
+        bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * 8) * 64 + lane;
         slot[(0 + HF) * 64] = PM; slot[(2 + HF) * 64] = PJ;
         slot[(4 + HF) * 64] = XM[HF]; slot[(6 + HF) * 64] = XJ[HF];
       }
@@ -684,7 +330,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         if (t < clen) (dqp + (int64_t)t * rs)[i] = from_f32<TIn>(dq[tl * 4 + r]);
       }
     const float x = wave_sum(sigacc);
-    if (lane == 0) sRed[NB * kC + HF * NB + nb] = x;
+    if (lane == 0) sRed[NB * kC + HF * NB + nbl] = x;
   };
 
   // ------------------------------------------------------------------ consumers
@@ -741,24 +387,25 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         Fs[sl] = sF[16 * (2 * HF + sl) + i];
       }
     }
+    const float f_first = fast_exp2(sC[0]);
     float* wDM = A.wDM + tile_off + 16 * nb;
     float* wDJ = A.wDJ + tile_off + 16 * nb;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
-    float* pw = ((g < 2) ? sPv : sPb) + nb * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
+    float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
 
     for (int it = 0; it <= dv; ++it) {
       if (it >= 1) {
         const int d = it - 1, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
-        const bf16x8* slot = sX + ((nb * 2 + (d & 1)) * 8) * 64 + lane;
+        const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * 8) * 64 + lane;
         // HF=0 (column tokens 0..31): reverse needs both P halves, strictly-lower only X_0;
         // HF=1 (column tokens 32..63): reverse needs P_1 only, strictly-lower both X halves
         const bf16x8 PM1 = slot[1 * 64], PJ1 = slot[3 * 64], XM0 = slot[4 * 64], XJ0 = slot[6 * 64];
         const bf16x8 Ma = slot[(HF ? 5 : 0) * 64];   // HF=0: P^M_0, HF=1: X^M_1
         const bf16x8 Ja = slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
-        const f32x4 M0T = *(const f32x4*)&sMJ[(nb * 2 + (d & 1)) * 32 + 4 * g];
-        const f32x4 J0T = *(const f32x4*)&sMJ[(nb * 2 + (d & 1)) * 32 + 16 + 4 * g];
+        const f32x4 M0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 4 * g];
+        const f32x4 J0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + 4 * g];
         float dvp[2], dbp[2];
 #pragma unroll
         for (int sl = 0; sl < 2; ++sl) {
@@ -822,29 +469,45 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           (dkp + (int64_t)s * rs)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
       }
       const float x = rows4_sum(gate[sl]);
-      if (g == 0) sRed[nb * kC + 16 * (2 * HF + sl) + i] = x;
+      if (g == 0) sRed[nbl * kC + 16 * (2 * HF + sl) + i] = x;
     }
   };
 
-  // every role runs dv+1 iterations with the same barriers
-  if (role == 0) producer(std::integral_constant<int, 0>{});
-  else if (role == 1) producer(std::integral_constant<int, 1>{});
-  else if (role == 2) consumer(std::integral_constant<int, 0>{});
-  else consumer(std::integral_constant<int, 1>{});
-
-  __syncthreads();
-  if (tid < kC) {
-    float gm = 0.f;
+  // every role runs dv+1 iterations with the same barriers; a wave whose column block lies beyond dk
+  // (last pass of a head dim that is not a multiple of 16*NB) only keeps the barriers
+  float gm_tot = 0.f, sg_tot = 0.f;   // threads 0..63: gate term of token tid; thread 0: sum of dJloc
+  for (pass = 0; pass < n_pass; ++pass) {
+    nb = pass * NB + nbl;
+    n_act = MULTI ? min(NB, nb_total - pass * NB) : NB;
+    // the per-role constants that do not depend on the column block (decay operands) must be computed
+    // inside the role that uses them: hoisted above the role branches or out of this loop they would be
+    // live for all four roles at once
+    asm volatile("" : "+v"(lane));
+    i = lane & 15;
+    g = lane >> 4;
+    stage(0);
+    __syncthreads();
+    if (MULTI && nbl >= n_act) {
+      for (int it = 0; it <= dv; ++it) iter_tail(it);
+    } else if (role == 0) producer(std::integral_constant<int, 0>{});
+    else if (role == 1) producer(std::integral_constant<int, 1>{});
+    else if (role == 2) consumer(std::integral_constant<int, 0>{});
+    else consumer(std::integral_constant<int, 1>{});
+    __syncthreads();
+    if (tid < kC) {
 #pragma unroll
-    for (int w = 0; w < NB; ++w) gm += sRed[w * kC + tid];
-    if (tid < clen) A.wE[(int64_t)h * A.tokens + t0 + tid] = gm;
-    if (tid == 0) {
-      float sg = 0.f;
+      for (int w = 0; w < NB; ++w)
+        if (!MULTI || w < n_act) gm_tot += sRed[w * kC + tid];
+      if (tid == 0) {
 #pragma unroll
-      for (int w = 0; w < 2 * NB; ++w) sg += sRed[NB * kC + w];
-      A.wSig[(int64_t)cidx * H + h] = sg;
+        for (int w = 0; w < NB; ++w)
+          if (!MULTI || w < n_act) sg_tot += sRed[NB * kC + w] + sRed[NB * kC + NB + w];
+      }
     }
+    __syncthreads();
   }
+  if (tid < clen) A.wE[(int64_t)h * A.tokens + t0 + tid] = gm_tot;
+  if (tid == 0) A.wSig[(int64_t)cidx * H + h] = sg_tot;
 }
 
 // ----------------------------------------------------------------- carry scan
@@ -1229,54 +892,40 @@ static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   const bool var = A.c.flags & PAL_FLAG_HAS_VAR;
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
-  if constexpr (NB <= 4) {
-    // four wave roles per workgroup (see chunk_bwd_local_roles_kernel)
-    const int NT = 4 * NB * 64;
-    const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
-                       (size_t)NB * 2 * 8 * 64 * 16;
-    if (lds > kMaxLds) return PAL_E_HEADDIM;
-    if (var) {
-      if (int rc = allow_lds((const void*)&chunk_bwd_local_roles_kernel<TIn, NB, true>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_roles_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
-    } else {
-      if (int rc = allow_lds((const void*)&chunk_bwd_local_roles_kernel<TIn, NB, false>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_roles_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
-    }
+  // four wave roles per block of 16 key columns, NB such blocks at a time (see chunk_bwd_local_roles_kernel)
+  const int NT = 4 * NB * 64;
+  const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
+                     (size_t)NB * 2 * 8 * 64 * 16;
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  const bool multi = A.c.dk != 16 * NB;
+  auto go = [&](auto kern) -> int {
+    if (int rc = allow_lds((const void*)kern, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernBwdLocal, s, kern, dim3((unsigned)blocks), dim3(NT), lds, s, A);
+    return 0;
+  };
+  int rc;
+  if constexpr (NB >= 3) {
+    if (multi) rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, true>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, true>);
+    else rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false>);
   } else {
-    const int NT = NB * 64;
-    const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + NB);
-    if (lds > kMaxLds) return PAL_E_HEADDIM;
-    if (var) {
-      if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, true>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
-    } else {
-      if (int rc = allow_lds((const void*)&chunk_bwd_local_kernel<TIn, NB, false>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernBwdLocal, s, (chunk_bwd_local_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NT), lds, s, A);
-    }
+    rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false>);
   }
+  if (rc) return rc;
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
 
 template <typename TIn>
 static int launch_local(const BwdArgs& A, hipStream_t s) {
-  switch (A.c.dk / 16) {
+  // at most 4 column blocks (16 waves) per workgroup; wider heads are split into equal passes
+  const int nb_total = A.c.dk / 16;
+  if (nb_total < 1 || nb_total > 16) return PAL_E_HEADDIM;
+  const int n_pass = (nb_total + 3) / 4;
+  switch ((nb_total + n_pass - 1) / n_pass) {
     case 1: return launch_local_nb<TIn, 1>(A, s);
     case 2: return launch_local_nb<TIn, 2>(A, s);
     case 3: return launch_local_nb<TIn, 3>(A, s);
     case 4: return launch_local_nb<TIn, 4>(A, s);
-    case 5: return launch_local_nb<TIn, 5>(A, s);
-    case 6: return launch_local_nb<TIn, 6>(A, s);
-    case 7: return launch_local_nb<TIn, 7>(A, s);
-    case 8: return launch_local_nb<TIn, 8>(A, s);
-    case 9: return launch_local_nb<TIn, 9>(A, s);
-    case 10: return launch_local_nb<TIn, 10>(A, s);
-    case 11: return launch_local_nb<TIn, 11>(A, s);
-    case 12: return launch_local_nb<TIn, 12>(A, s);
-    case 13: return launch_local_nb<TIn, 13>(A, s);
-    case 14: return launch_local_nb<TIn, 14>(A, s);
-    case 15: return launch_local_nb<TIn, 15>(A, s);
-    case 16: return launch_local_nb<TIn, 16>(A, s);
     default: return PAL_E_HEADDIM;
   }
 }
