@@ -371,18 +371,10 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
         p[tb] = acc;
         pv[tb] = accv;
       }
-#pragma unroll
-      for (int tb = 0; tb < 4; ++tb) {
-        p[tb] = rows4_sum(p[tb]);
-        if (HAS_VAR) pv[tb] = rows4_sum(pv[tb]);
-      }
-      if (g == 0) {
-#pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-          sO[(nb * kDG + dd) * kC + 16 * tb + i] = p[tb];
-          if (HAS_VAR) sOv[(nb * kDG + dd) * kC + 16 * tb + i] = pv[tb];
-        }
-      }
+      // sum over the four rows of 16 lanes (key columns 4g..4g+3 of every row): transposing reduction,
+      // after which the lanes of row g hold the total of token block g
+      sO[(nb * kDG + dd) * kC + 16 * g + i] = rows4_sum_x4(p[0], p[1], p[2], p[3]);
+      if (HAS_VAR) sOv[(nb * kDG + dd) * kC + 16 * g + i] = rows4_sum_x4(pv[0], pv[1], pv[2], pv[3]);
     }
     __syncthreads();
     // flush the group's outputs: work item = (token t, 4 value rows)
