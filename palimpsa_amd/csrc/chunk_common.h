@@ -56,6 +56,52 @@ __device__ __forceinline__ void seq_lookup(const ChunkArgs& a, int n, int& bos, 
   }
 }
 
+// Block exponent E of a tile for the f16 operands of the prefix products.  The operands
+// X^M = k v 2^-E and X^J = k^2 b 2^-E are built with packed f16 multiplies from k, k^2 (f16) and the
+// staged rows v 2^-E, b 2^-E (f16); the decay operand carries the 2^E back (L 2^E <= 2^15), so the
+// fp32 accumulators hold the unscaled sums.  E = 0 unless max(|v|,|b|) max(1,|k|^2) over the tile
+// exceeds 2^12; supported range: |k| <= 128 and max(|v|,|b|) max(1,|k|^2) < 2^28.
+// Every thread of the workgroup calls this (it synchronises); sMax is LDS scratch of 3 floats per wave.
+template <typename TIn>
+__device__ __forceinline__ int tile_block_exponent(const TIn* kt, const TIn* vt, const TIn* bt, int H, int dk, int dv,
+                                                   int clen, int tid, int nthreads, float* sMax) {
+  float km = 0.f, vm = 0.f, bm = 0.f;
+  const int gk = dk >> 3, gv = dv >> 3;
+  for (int idx = tid; idx < kC * gk; idx += nthreads) {
+    const int s = idx / gk, c = idx - s * gk;
+    if (s < clen) {
+      float x[8];
+      load_vec<4>(kt + (int64_t)s * H * dk + 8 * c, x);
+      load_vec<4>(kt + (int64_t)s * H * dk + 8 * c + 4, x + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) km = fmaxf(km, fabsf(x[e]));
+    }
+  }
+  for (int idx = tid; idx < kC * gv; idx += nthreads) {
+    const int s = idx / gv, c = idx - s * gv;
+    if (s < clen) {
+      float x[8], y[8];
+      load_vec<4>(vt + (int64_t)s * H * dv + 8 * c, x);
+      load_vec<4>(vt + (int64_t)s * H * dv + 8 * c + 4, x + 4);
+      load_vec<4>(bt + (int64_t)s * H * dv + 8 * c, y);
+      load_vec<4>(bt + (int64_t)s * H * dv + 8 * c + 4, y + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { vm = fmaxf(vm, fabsf(x[e])); bm = fmaxf(bm, fabsf(y[e])); }
+    }
+  }
+  km = wave_max(km);
+  vm = wave_max(vm);
+  bm = wave_max(bm);
+  const int w = tid >> 6, nw = (nthreads + 63) >> 6;
+  if ((tid & 63) == 0) { sMax[3 * w] = km; sMax[3 * w + 1] = vm; sMax[3 * w + 2] = bm; }
+  __syncthreads();
+  km = 0.f; vm = 0.f; bm = 0.f;
+  for (int x = 0; x < nw; ++x) { km = fmaxf(km, sMax[3 * x]); vm = fmaxf(vm, sMax[3 * x + 1]); bm = fmaxf(bm, sMax[3 * x + 2]); }
+  __syncthreads();
+  const float m = fmaxf(vm, bm) * fmaxf(1.f, km * km);
+  return (m > 4096.f) ? min(15, ilogbf(m) - 12) : 0;
+}
+
 // inclusive prefix sum over the 64 lanes of a wave
 __device__ __forceinline__ float wave_inclusive_scan(float x, int lane) {
 #pragma unroll

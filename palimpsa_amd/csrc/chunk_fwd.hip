@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
 }
 
 // ------------------------------------------------------------------ kernel 2
-constexpr int kVS = 68;  // row stride (floats) of the transposed v/b staging tiles
+constexpr int kVH = 72;  // row stride (f16) of the transposed, block-scaled v/b staging tiles of chunk_out_kernel
 constexpr int kDG = 16;  // value rows per staging group
 
 // index of the L operand for (tb, ks): tb0,tb1 -> one K step; tb2,tb3 -> two
@@ -210,9 +210,9 @@ template <typename TIn, int NB, bool HAS_VAR>
 __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
   float* sC = smem;                       // [64] running log2-decay inside the tile
-  float* sV = sC + kC;                    // [16][kVS] v^T of the current value-row group
-  float* sB = sV + kDG * kVS;             // [16][kVS]
-  float* sO = sB + kDG * kVS;             // [NB][16][64] per-wave partial outputs
+  f16_t* sV = (f16_t*)(sC + kC);          // [2][16][kVH] v^T 2^-E of the current and the next value-row group, f16
+  f16_t* sB = sV + 2 * kDG * kVH;         // [2][16][kVH] b^T 2^-E
+  float* sO = (float*)(sB + 2 * kDG * kVH);   // [NB][16][64] per-wave partial outputs
   float* sOv = sO + NB * kDG * kC;        // same for o_var
   constexpr int NT = NB * 64;
   const int tid = threadIdx.x, lane = tid & 63, nb = tid >> 6, i = lane & 15, g = lane >> 4;
@@ -246,56 +246,19 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
       }
     }
   };
-  auto stage_store = [&]() {
-#pragma unroll
-    for (int it = 0; it < NITEM; ++it) {
-      const int idx = tid + it * NT;
-      const int s = idx >> 2, dq = idx & 3;
-      if (idx < kC * kDG / 4) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          sV[(4 * dq + e) * kVS + s] = vst[it][e];
-          sB[(4 * dq + e) * kVS + s] = bst[it][e];
-        }
-      }
-    }
-  };
-  stage_load(0);
-  stage_store();
-  __syncthreads();
-
-  // ---- per-wave constants of this tile
-  float F[4], Gi[4], ct[4];
-#pragma unroll
-  for (int tb = 0; tb < 4; ++tb) {
-    ct[tb] = sC[16 * tb + i];
-    F[tb] = fast_exp2(ct[tb]);
-    Gi[tb] = (1.f - F[tb]) * Ip;
-  }
-  bf16x8 Lr[6];
-  float kA[2][8], kk[2][8];
+  // the wave's k column and q rows are requested first so that their latency overlaps the block-exponent pass
+  float kraw[2][8];
   {
     const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      float cs[8];
-      *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
-      *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int s = 8 * g + j + 32 * ks;
         const bool ok = s < clen;
         const float kv = to_f32(kp[(int64_t)(ok ? s : 0) * H * dk]);
-        kA[ks][j] = ok ? kv : 0.f;
-        kk[ks][j] = kA[ks][j] * kA[ks][j];
-#pragma unroll
-        for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
-          const int t = 16 * tb + i;
-          const float lv = (s <= t) ? fast_exp2(ct[tb] - cs[j]) : 0.f;
-          Lr[lidx(tb, ks)][j] = (bf16_t)lv;
-        }
+        kraw[ks][j] = ok ? kv : 0.f;
       }
-    }
   }
   float qD[4][4];
   {
@@ -311,6 +274,57 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
       }
     }
   }
+  stage_load(0);
+  // block exponent of the f16 operands (see tile_block_exponent); sO doubles as its scratch
+  const int bexp = tile_block_exponent((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
+  const float down = __builtin_amdgcn_exp2f(-(float)bexp);
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int it = 0; it < NITEM; ++it) {
+      const int idx = tid + it * NT;
+      const int s = idx >> 2, dq = idx & 3;
+      if (idx < kC * kDG / 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          sV[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(vst[it][e] * down);
+          sB[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(bst[it][e] * down);
+        }
+      }
+    }
+  };
+  stage_store(0);
+  __syncthreads();
+
+  // ---- per-wave constants of this tile
+  float F[4], Gi[4], ct[4];
+#pragma unroll
+  for (int tb = 0; tb < 4; ++tb) {
+    ct[tb] = sC[16 * tb + i];
+    F[tb] = fast_exp2(ct[tb]);
+    Gi[tb] = (1.f - F[tb]) * Ip;
+  }
+  f16x8 Lr[6];            // decay operand times 2^E
+  f16x8 kA[2], kk[2];     // k and k*k of the wave's key column for the 64 tokens, operand layout
+  {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      float cs[8];
+      *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
+      *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int s = 8 * g + j + 32 * ks;
+        kA[ks][j] = (f16_t)kraw[ks][j];
+        kk[ks][j] = (f16_t)(kraw[ks][j] * kraw[ks][j]);
+#pragma unroll
+        for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
+          const int t = 16 * tb + i;
+          const float lv = (s <= t) ? fast_exp2(ct[tb] - cs[j] + (float)bexp) : 0.f;
+          Lr[lidx(tb, ks)][j] = (f16_t)lv;
+        }
+      }
+    }
+  }
   const float scale = a.scale;
   const float* cmu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
   const float* cI = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
@@ -319,9 +333,14 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
   f32x4 mu0_n = *(const f32x4*)cmu, I0_n = *(const f32x4*)cI;
   const int n_groups = dv / kDG;
   for (int dg = 0; dg < n_groups; ++dg) {
-    if (dg + 1 < n_groups) stage_load(dg + 1);
+    const int buf = dg & 1;
     for (int dd = 0; dd < kDG; ++dd) {
       const int d = dg * kDG + dd;
+      if (dd == kDG / 2 && dg + 1 < n_groups) {
+        // rows of the next group go to the other buffer mid-group (read only after the barriers below)
+        stage_load(dg + 1);
+        stage_store(buf ^ 1);
+      }
       const f32x4 mu0 = mu0_n, I0 = I0_n;
       {
         const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
@@ -331,33 +350,23 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
       float M0[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) M0[r] = mu0[r] * I0[r];
-      bf16x8 XM[2], XJ[2];
+      f16x8 XM[2], XJ[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        const f32x4 v0 = *(const f32x4*)&sV[dd * kVS + 8 * g + 32 * ks];
-        const f32x4 v1 = *(const f32x4*)&sV[dd * kVS + 8 * g + 32 * ks + 4];
-        const f32x4 b0 = *(const f32x4*)&sB[dd * kVS + 8 * g + 32 * ks];
-        const f32x4 b1 = *(const f32x4*)&sB[dd * kVS + 8 * g + 32 * ks + 4];
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
-          const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
-          const bf16x2 pm = pack2(kA[ks][j] * va, kA[ks][j + 1] * vb);
-          const bf16x2 pj = pack2(kk[ks][j] * ba, kk[ks][j + 1] * bb);
-          XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
-          XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
-        }
+        // 8 consecutive tokens of the row: one 16-byte LDS read each; packed f16 products are the operands
+        XM[ks] = kA[ks] * *(const f16x8*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+        XJ[ks] = kk[ks] * *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
       }
       float p[4], pv[4];
 #pragma unroll
       for (int tb = 0; tb < 4; ++tb) {
         f32x4 accM = {0.f, 0.f, 0.f, 0.f};
         f32x4 accI = {Gi[tb], Gi[tb], Gi[tb], Gi[tb]};
-        accM = mfma16(XM[0], Lr[lidx(tb, 0)], accM);
-        accI = mfma16(XJ[0], Lr[lidx(tb, 0)], accI);
+        accM = mfma16h(XM[0], Lr[lidx(tb, 0)], accM);
+        accI = mfma16h(XJ[0], Lr[lidx(tb, 0)], accI);
         if (tb >= 2) {
-          accM = mfma16(XM[1], Lr[lidx(tb, 1)], accM);
-          accI = mfma16(XJ[1], Lr[lidx(tb, 1)], accI);
+          accM = mfma16h(XM[1], Lr[lidx(tb, 1)], accM);
+          accI = mfma16h(XJ[1], Lr[lidx(tb, 1)], accI);
         }
         float acc = 0.f, accv = 0.f;
 #pragma unroll
@@ -399,7 +408,6 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
         }
       }
     }
-    if (dg + 1 < n_groups) stage_store();
     __syncthreads();
   }
 }
@@ -407,7 +415,7 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
 template <typename TIn, int NB>
 static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
   const bool var = a.flags & PAL_FLAG_HAS_VAR;
-  const size_t lds = sizeof(float) * (kC + 2 * kDG * kVS + (var ? 2 : 1) * NB * kDG * kC);
+  const size_t lds = sizeof(float) * (kC + (var ? 2 : 1) * NB * kDG * kC) + 4 * sizeof(f16_t) * kDG * kVH;
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;

@@ -12,6 +12,8 @@ typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
@@ -156,6 +158,19 @@ __device__ __forceinline__ float rows4_sum_x4(float p0, float p1, float p2, floa
   return s0 + s1;
 }
 __device__ __forceinline__ float wave_sum(float x) { return rows4_sum(row16_sum(x)); }
+// maximum over the 64 lanes of a wave; every lane gets it
+__device__ __forceinline__ float wave_max(float x) {
+  x = fmaxf(x, row_ror<8>(x));
+  x = fmaxf(x, row_ror<4>(x));
+  x = fmaxf(x, row_ror<2>(x));
+  x = fmaxf(x, row_ror<1>(x));
+  float a = x, b = x;
+  swap_halves(a, b);
+  a = fmaxf(a, b);
+  b = a;
+  swap_rows(a, b);
+  return fmaxf(a, b);
+}
 
 // ------------------------------------------------------------------- MFMA
 // D[16x16] += A[16x32] * B[32x16], bf16 operands, fp32 accumulate.
@@ -163,6 +178,11 @@ __device__ __forceinline__ float wave_sum(float x) { return rows4_sum(row16_sum(
 // D col (l%16), rows 4*(l/16)+r.
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// same shape with f16 operands (11-bit mantissa; range handled by the caller's block exponent)
+__device__ __forceinline__ f32x4 mfma16h(f16x8 a, f16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
 __device__ __forceinline__ bf16x2 pack2(float lo, float hi) {
