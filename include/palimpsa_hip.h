@@ -148,7 +148,9 @@ int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
 /* Chunked forward.  Replaces ChunkPalimpsa.forward + chunk_palimpsa_fwd_kernel
  * (chunk_palimpsa_forgetting_scalar.py:66-218, :441-517).  Fills chunk_mu /
  * chunk_I (the reference's intermediate_mu_state / intermediate_I_state,
- * :187-188) for the backward. */
+ * :187-188) for the backward.  The prefix products of the output kernel use f16
+ * operands with a per-tile block exponent: |k| <= 128 and
+ * max(|v|,|b|) * max(1,|k|^2) < 2^28 are required of the rows of a 64-token tile. */
 int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
 /* Chunked backward.  Replaces ChunkPalimpsa.backward + chunk_palimpsa_bwd_kernel
