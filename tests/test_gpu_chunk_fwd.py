@@ -114,3 +114,21 @@ def test_error_paths_match_reference(gpu_device):
     inp = hp.to_device(po.make_inputs(2, 8, 2, 16, 16, seed=0), gpu_device)
     with pytest.raises(ValueError):
         _call(ck, inp, cu_seqlens=torch.tensor([0, 8], device=gpu_device))
+
+
+@pytest.mark.parametrize("v_scale,k_scale", [(3.0e5, 1.0), (40.0, 30.0), (1.0e-4, 1.0)])
+def test_block_exponent_of_the_f16_operands(gpu_device, v_scale, k_scale):
+    """Rows far from O(1): the output kernel's f16 operands carry a per-tile block exponent
+    (E > 0 for the first two cases, tiny values for the third); relative error as for O(1) rows."""
+    ck, _ = _ops()
+    B, T, H, d = 1, 200, 2, 64
+    inp = po.make_inputs(B, T, H, d, d, seed=77)
+    inp["v"] = inp["v"] * v_scale
+    inp["b"] = inp["b"] * v_scale
+    inp["k"] = inp["k"] * k_scale
+    inp = hp.rounded(inp, torch.bfloat16)
+    o, mu, I = _call(ck, hp.to_device(inp, gpu_device), output_final_state=True, chunk_size=64)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp)
+    assert torch.isfinite(o.float()).all()
+    assert hp.max_rel(o, o_ref) <= 1e-2
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
