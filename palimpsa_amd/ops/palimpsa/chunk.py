@@ -41,6 +41,54 @@ def _count_chunks(T: int, B: int) -> int:
     return (T + L.PAL_CHUNK - 1) // L.PAL_CHUNK * B
 
 
+# the windowed forward keeps at most this many bytes of tile-start states alive (they then stay in the
+# 256 MB last-level cache between the kernel that writes them and the two that read them)
+_WINDOW_STATE_BYTES = 128 << 20
+
+
+def _window_tiles(H: int, dv: int, dk: int) -> int:
+    return max(16, _WINDOW_STATE_BYTES // (2 * 4 * H * dv * dk))
+
+
+def _windowed_forward(p, scale, output_uncertainty, o, o_var, final_mu, final_I, window: int) -> None:
+    """Forward of one sequence (B == 1) in segments of ``window`` tiles, each started from the final
+    state of the one before.  Same kernels and same tiles as the single call; the state crosses a
+    segment boundary as (mu, I), which costs one fp32 rounding per boundary."""
+    dev = p.q.device
+    _, T, H, _ = p.q.shape
+    seg = window * L.PAL_CHUNK
+    int_mu = torch.empty(window, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+    int_I = torch.empty_like(int_mu)
+    # state out alternates between a scratch pair and (final_mu, final_I) such that the last segment
+    # writes the final buffers; a segment never reads the buffers it writes
+    scratch = (torch.empty_like(final_mu), torch.empty_like(final_I))
+    n_seg = (T + seg - 1) // seg
+    lib = L.load()
+    pt = cm._ptr
+    cur_mu, cur_I = p.init_mu, p.init_I
+    with torch.cuda.device(dev):
+        stream = cm.current_stream_ptr(dev)
+        for j in range(n_seg):
+            s, e = j * seg, min(T, (j + 1) * seg)
+            out_mu, out_I = (final_mu, final_I) if (n_seg - 1 - j) % 2 == 0 else scratch
+            flags = L.PAL_FLAG_STORE_FINAL
+            if cur_mu is not None:
+                flags |= L.PAL_FLAG_HAS_INIT
+            if output_uncertainty:
+                flags |= L.PAL_FLAG_HAS_VAR
+            n_tiles = (e - s + L.PAL_CHUNK - 1) // L.PAL_CHUNK
+            dims = L.PalDims(batch=1, seq_len=e - s, n_seqs=1, n_heads=H, dk=p.dk_p, dv=p.dv_p, total_chunks=n_tiles,
+                             dtype=cm._pal_dtype(p.compute_dtype), gate_dtype=cm._pal_dtype(p.gt.dtype),
+                             var_dtype=cm._pal_dtype(p.compute_dtype), flags=flags, scale=float(scale))
+            tens = L.PalFwdTensors(
+                q=pt(p.q[:, s:e]), k=pt(p.k[:, s:e]), v=pt(p.v[:, s:e]), b=pt(p.b[:, s:e]), gt=pt(p.gt[:, s:e]),
+                g=pt(p.g), Ip=pt(p.Ip), o=pt(o[:, s:e]), o_var=pt(o_var[:, s:e] if o_var is not None else None),
+                init_mu=pt(cur_mu), init_I=pt(cur_I), final_mu=pt(out_mu), final_I=pt(out_I), cu_seqlens=None,
+                chunk_table=None, chunk_offsets=None, chunk_mu=pt(int_mu), chunk_I=pt(int_I))
+            L.check(lib.pal_chunk_fwd(dims, tens, stream), "pal_chunk_fwd")
+            cur_mu, cur_I = out_mu, out_I
+
+
 class ChunkPalimpsa(torch.autograd.Function):
     """forward(ctx, q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
     output_final_state, output_uncertainty, cu_seqlens, chunk_offsets, int_mu, int_I)
@@ -63,18 +111,29 @@ class ChunkPalimpsa(torch.autograd.Function):
             total_chunks = int(table.numel()) // 4
         else:
             total_chunks = _count_chunks(T, B)
-        need = (total_chunks, H, p.dv_p, p.dk_p)
-        if (int_mu is None or int_I is None or tuple(int_mu.shape) != need or tuple(int_I.shape) != need
-                or int_mu.dtype != torch.float32 or int_I.dtype != torch.float32
-                or int_mu.device != dev or not int_mu.is_contiguous() or not int_I.is_contiguous()):
-            int_mu = torch.empty(need, dtype=torch.float32, device=dev)
-            int_I = torch.empty(need, dtype=torch.float32, device=dev)
         o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
         # the reference hands o_var back in q.dtype (chunk...py:515)
         o_var = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev) if output_uncertainty else None
         # final states are always produced, as in the reference (chunk...py:475-476)
         final_mu = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
         final_I = torch.empty_like(final_mu)
+
+        window = _window_tiles(H, p.dv_p, p.dk_p)
+        if (not any(ctx.needs_input_grad[:9]) and int_mu is None and int_I is None and p.cu_seqlens is None
+                and B == 1 and total_chunks > window):
+            # nothing will ask for the tile-start states again: run the sequence in windows of tiles through the
+            # state, so that the per-tile states (2*H*dv*dk*4 bytes per tile) never exist for more than one window
+            _windowed_forward(p, scale, output_uncertainty, o, o_var, final_mu, final_I, window)
+            o = cm.unpad_last(o, p.dv).to(q.dtype)
+            o_var = cm.unpad_last(o_var, p.dv).to(q.dtype) if output_uncertainty else None
+            return o, o_var, cm.unpad_state(final_mu, p), cm.unpad_state(final_I, p)
+
+        need = (total_chunks, H, p.dv_p, p.dk_p)
+        if (int_mu is None or int_I is None or tuple(int_mu.shape) != need or tuple(int_I.shape) != need
+                or int_mu.dtype != torch.float32 or int_I.dtype != torch.float32
+                or int_mu.device != dev or not int_mu.is_contiguous() or not int_I.is_contiguous()):
+            int_mu = torch.empty(need, dtype=torch.float32, device=dev)
+            int_I = torch.empty(need, dtype=torch.float32, device=dev)
         flags = L.PAL_FLAG_STORE_FINAL
         if p.cu_seqlens is not None:
             flags |= L.PAL_FLAG_VARLEN
@@ -184,9 +243,15 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
         total_chunks = _count_chunks(q.shape[1], q.shape[0])
     H = q.shape[-2]
     dk_p, dv_p = cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1])
-    # chunk-start states, allocated outside the autograd Function as in the reference (chunk...py:652-653)
-    int_mu = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
-    int_I = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
+    # chunk-start states, allocated outside the autograd Function as in the reference (chunk...py:652-653);
+    # a long single sequence that no backward will follow is run in windows instead (see _windowed_forward)
+    needs_grad = torch.is_grad_enabled() and any(
+        isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state))
+    if not needs_grad and cu_seqlens is None and q.shape[0] == 1 and total_chunks > _window_tiles(H, dv_p, dk_p):
+        int_mu = int_I = None
+    else:
+        int_mu = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
+        int_I = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=q.device)
     o, o_var, final_mu_state, final_I_state = ChunkPalimpsa.apply(
         q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
         output_final_state, output_uncertainty, cu_seqlens, chunk_offsets, int_mu, int_I)

@@ -132,3 +132,30 @@ def test_block_exponent_of_the_f16_operands(gpu_device, v_scale, k_scale):
     assert torch.isfinite(o.float()).all()
     assert hp.max_rel(o, o_ref) <= 1e-2
     assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
+def test_windowed_no_grad_forward_equals_single_call(gpu_device, monkeypatch):
+    """A single long sequence without autograd is run in windows of tiles through the state
+    (no tile-start states for the whole sequence); same kernels, same tiles, so the results agree
+    with the single call to within the fp32 rounding of the state hand-over."""
+    from palimpsa_amd.ops.palimpsa import chunk as chunk_mod
+    ck, _ = _ops()
+    B, T, H, d = 1, 2500, 2, 32
+    inp = hp.rounded(po.make_inputs(B, T, H, d, d, seed=5), torch.bfloat16)
+    dvc = hp.to_device(inp, gpu_device)
+    gen = torch.Generator().manual_seed(6)
+    mu0 = (torch.randn(B, H, d, d, generator=gen) * 0.1).to(gpu_device)
+    I0 = (1.0 + torch.rand(B, H, d, d, generator=gen)).to(gpu_device)
+    kw = dict(initial_mu_state=mu0, initial_I_state=I0, output_final_state=True, output_uncertainty=True, chunk_size=64)
+    monkeypatch.setattr(chunk_mod, "_WINDOW_STATE_BYTES", 16 * 2 * 4 * H * d * d)   # 16 tiles per window
+    assert chunk_mod._window_tiles(H, d, d) == 16
+    with torch.no_grad():
+        (o_w, ov_w), mu_w, I_w = _call(ck, dvc, **kw)
+    dvc["v"] = dvc["v"].clone().requires_grad_(True)     # autograd path: one call, all tile-start states kept
+    (o_s, ov_s), mu_s, I_s = _call(ck, dvc, **kw)
+    assert hp.max_abs(o_w.float(), o_s.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_abs(ov_w.float(), ov_s.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu_w, mu_s) <= 1e-5 and hp.max_rel(I_w, I_s) <= 1e-5
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0.cpu(), I0=I0.cpu())
+    assert hp.max_abs(o_w.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu_w, mu_ref) <= STATE_REL_TOL
