@@ -567,9 +567,8 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   float* sW4 = sAs + kC;                   // [8]
   float* sBt = sW4 + 8;                    // [64][dv/8] beta of the carry terms, one slot per work item
   float* sO1 = sBt + kC * (dv >> 3);       // [64][OS] dk^carry, later dv^carry
-  // R_M^T, R_J^T in bf16 [2][dk][dv + 8] for the dk products; the same bytes hold db^carry [64][OS] afterwards
-  float* sO2 = sO1 + kC * (dmax + 4);
-  bf16_t* sRT = (bf16_t*)sO2;
+  float* sO2 = sO1 + kC * (dmax + 4);      // [64][OS] db^carry
+  bf16_t* sRT = (bf16_t*)(sO2 + kC * (dmax + 4));   // [2][dk][dv + 8] R_M^T, R_J^T in bf16, operand source of all four products
   const int RS = dv + 8;
   const int OS = dmax + 4;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
@@ -709,7 +708,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       }
     }
   }
-  __syncthreads();   // sO1 and the R^T bytes are free again
+  __syncthreads();   // sO1 is free again
 
   // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
   {
@@ -743,14 +742,12 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
           const int n0 = 8 * g + 32 * ks;
           bf16x8 B1, B2;
           if (n0 < dk) {
-            const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
-            const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
-            const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
-            const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
+            // 8 consecutive key columns of value row d = 16db_ + i: a column walk through the transposed
+            // bf16 copy in LDS (the fp32 carries in global memory would miss L2 on this second read)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
-              B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
+            for (int j = 0; j < 8; ++j) {
+              B1[j] = sRT[(n0 + j) * RS + 16 * db_ + i];
+              B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i];
             }
           } else {
 #pragma unroll
@@ -983,8 +980,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
     const int dmax = dd.dk > dd.dv ? dd.dk : dd.dv;
-    const size_t rt_bytes = 2 * (size_t)2 * dd.dk * (dd.dv + 8), o2_bytes = sizeof(float) * kC * (dmax + 4);
-    const size_t lds = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3) + (size_t)kC * (dmax + 4)) + (rt_bytes > o2_bytes ? rt_bytes : o2_bytes);
+    const size_t lds = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3) + 2 * (size_t)kC * (dmax + 4)) + 2 * (size_t)2 * dd.dk * (dd.dv + 8);
     if (lds > kMaxLds) return PAL_E_HEADDIM;
     if (bf) {
       if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<bf16_t>, lds)) return rc2;
