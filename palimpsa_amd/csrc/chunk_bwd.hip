@@ -194,7 +194,6 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     constexpr int HF = decltype(hfc)::value;   // token blocks 2HF, 2HF+1 (index tl)
     bf16x8 Lop[HF ? 4 : 2];   // forward operand L[t,s], s <= t: HF=0 [tl], HF=1 [2tl+ks]
     float kk[HF ? 16 : 8];    // k in operand layout (n = i, s = 8g+j+32ks)
-    float k2[HF ? 16 : 8];    // k*k, same layout
     float qq[8];              // q in result layout (t = 16tb+4g+r, n = i)
     float dq[8];
     float sigacc = 0.f;
@@ -215,7 +214,6 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           const bool ok = s < clen;
           const float kv = to_f32((kp + (int64_t)(ok ? s : 0) * rs)[i]);
           kk[ks * 8 + j] = ok ? kv : 0.f;
-          k2[ks * 8 + j] = kk[ks * 8 + j] * kk[ks * 8 + j];
 #pragma unroll
           for (int tl = 0; tl < 2; ++tl) {
             const int t = 16 * (2 * HF + tl) + i;
@@ -268,8 +266,9 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           for (int j = 0; j < 8; j += 2) {
             const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
             const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
-            const bf16x2 pm = pack2(kk[ks * 8 + j] * va, kk[ks * 8 + j + 1] * vb);
-            const bf16x2 pj = pack2(k2[ks * 8 + j] * ba, k2[ks * 8 + j + 1] * bb);
+            const float ka = kk[ks * 8 + j], kb = kk[ks * 8 + j + 1];
+            const bf16x2 pm = pack2(ka * va, kb * vb);
+            const bf16x2 pj = pack2((ka * ba) * ka, (kb * bb) * kb);
             XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
             XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
           }
@@ -339,7 +338,6 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     constexpr int HF = decltype(hfc)::value;   // column-token blocks 2HF, 2HF+1 (index sl)
     bf16x8 Lop[6];    // reverse operand, HF=0 [2sl+p], HF=1 [sl] (p=1); strictly-lower operand, HF=0 [4+sl], HF=1 [2+2sl+ks]
     float kr[8];      // k in result layout (s = 16sb+i, n = 4g+r)
-    float kr2[8];     // k*k
     float dkM[8], dkJ[8];
     float gate[2], Fs[2];
     {
@@ -385,8 +383,6 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) { kr[sl * 4 + r] = 0.f; dkM[sl * 4 + r] = 0.f; dkJ[sl * 4 + r] = 0.f; }
         if (s < clen) load_vec<4>(kp4 + (int64_t)s * rs + 4 * g, &kr[sl * 4]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) kr2[sl * 4 + r] = kr[sl * 4 + r] * kr[sl * 4 + r];
         gate[sl] = 0.f;
         Fs[sl] = sF[16 * (2 * HF + sl) + i];
       }
@@ -437,8 +433,9 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           float dvs = 0.f, dbs = 0.f, gm = gate[sl];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            dvs = fmaf(aM[r], kr[sl * 4 + r], dvs);
-            dbs = fmaf(aJ[r], kr2[sl * 4 + r], dbs);
+            const float kv = kr[sl * 4 + r];
+            dvs = fmaf(aM[r], kv, dvs);
+            dbs = fmaf(aJ[r] * kv, kv, dbs);
             dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
             dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
             const float Ss = fmaf(Fs[sl], M0T[r], sM[r]);
