@@ -147,6 +147,9 @@ class ChunkPalimpsa(torch.autograd.Function):
             rc = L.load().pal_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
         L.check(rc, "pal_chunk_fwd")
 
+        # gradients of unused outputs arrive as None instead of zero-filled tensors (the final states'
+        # gradients are ignored anyway)
+        ctx.set_materialize_grads(False)
         ctx.save_for_backward(p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens,
                               table, offsets, int_mu, int_I)
         ctx.meta = dict(dk=p.dk, dv=p.dv, dk_p=p.dk_p, dv_p=p.dv_p, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype,
@@ -168,6 +171,8 @@ class ChunkPalimpsa(torch.autograd.Function):
         dv_p = v.shape[-1]
         cd = m["compute_dtype"]
         has_var = m["output_uncertainty"] and do_var is not None
+        if do is None:   # only o_var (or nothing) was used downstream
+            do = torch.zeros(B, T, H, m["dv"], dtype=cd, device=dev)
 
         def prep_grad(x):
             x = x.to(cd)

@@ -57,6 +57,7 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
         p, dims, o, o_var, final_mu, final_I = _recurrent_forward(
             q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I_state,
             output_final_state, output_uncertainty, cu_seqlens)
+        ctx.set_materialize_grads(False)   # unused outputs (o_var, final states) send None, not zero tensors
         ctx.save_for_backward(p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens)
         ctx.meta = dict(dk=p.dk, dv=p.dv, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype, scale=float(scale),
                         in_dtypes=(q.dtype, k.dtype, v.dtype, b.dtype, gt.dtype, g.dtype, Ip.dtype),
@@ -76,6 +77,8 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
         dv_p = v.shape[-1]
         cd = m["compute_dtype"]
         has_var = m["output_uncertainty"] and do_var is not None
+        if do is None:
+            do = torch.zeros(B, T, H, m["dv"], dtype=cd, device=dev)
 
         def prep(x, dt):
             x = x.to(dt)
