@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode]
 
-Headline (BASELINE.json metric, configs[1]): chunked forward+backward at
+Headline workload (the metric's own configuration): chunked forward+backward at
 B=8, T=2048, H=12, dk=dv=64, bf16 rows, fp32 gates/states, 64-token tiles,
 synthetic seeded inputs, timed through the public entry point
 (palimpsa_amd.ops.palimpsa.chunk_palimpsa + autograd), inputs resident in HBM.

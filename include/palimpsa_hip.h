@@ -57,7 +57,7 @@ extern "C" {
 #define PAL_E_CAPACITY -10   /* output table too small                        */
 #define PAL_E_ALIGN -11      /* pointer not aligned to 16 bytes               */
 
-/* Tokens per chunk tile of the chunked kernels (BASELINE chunk size). */
+/* Tokens per chunk tile of the chunked kernels (the chunk size of the benchmark configurations). */
 #define PAL_CHUNK 64
 
 typedef struct PalDims {

@@ -19,7 +19,7 @@ from oracle import palimpsa_oracle as po  # noqa: E402
 
 
 def c0_case():
-    """BASELINE config 0: B=2, T=256, H=4, dk=dv=32, fp32, seed 0; outputs every 16th token."""
+    """Benchmark configuration 0: B=2, T=256, H=4, dk=dv=32, fp32, seed 0; outputs every 16th token."""
     inp = po.make_inputs(2, 256, 4, 32, 32, seed=0)
     o, _, mu, I = po.palimpsa_recurrence(*[inp[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")])
     return dict(o_every16=o[:, ::16].numpy(), final_mu=mu.numpy(), final_I=I.numpy(),

@@ -19,7 +19,7 @@ def _ops():
 
 
 def test_c0_fp32_forward_and_final_state(gpu_device):
-    """BASELINE config 0: B=2, T=256, H=4, dk=dv=32, fp32, seed 0, zero mean state, I0 = Ip."""
+    """Benchmark configuration 0: B=2, T=256, H=4, dk=dv=32, fp32, seed 0, zero mean state, I0 = Ip."""
     fr = _ops()
     inp = po.make_inputs(2, 256, 4, 32, 32, seed=0)
     o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp)
