@@ -169,3 +169,26 @@ def test_squared_error_loss_all_gradients_max_norm(gpu_device):
     ref = hp.oracle_grads(inp, do)
     grads = _run_bwd(inp, gpu_device, do)
     _compare(grads, ref, NAMES)
+
+
+@pytest.mark.parametrize("cu", [[0, 0, 5, 5, 70], [0, 64, 64, 128], [0, 130, 130]])
+def test_bf16_backward_varlen_with_empty_documents(gpu_device, cu):
+    """Packed batches may hold documents of length zero (they own no tile); their final state is the
+    default (0, Ip) and the other documents are unaffected."""
+    H, d = 2, 32
+    T = cu[-1]
+    inp = hp.rounded(po.make_inputs(1, T, H, d, d, seed=3), torch.bfloat16)
+    gen = torch.Generator().manual_seed(4)
+    do = torch.randn(1, T, H, d, generator=gen)
+    ref = hp.oracle_grads(inp, do, cu=cu)
+    grads = _run_bwd(inp, gpu_device, do, cu=cu)
+    _compare(grads, ref, NAMES, inp=inp, dg_l1=True)
+    ck = _ck()
+    dvc = hp.to_device(inp, gpu_device)
+    o, mu, I = ck(dvc["q"], dvc["k"], dvc["v"], dvc["b"], dvc["gt"], dvc["g"], dvc["Ip"], chunk_size=64,
+                  cu_seqlens=torch.tensor(cu, device=gpu_device), output_final_state=True)
+    assert hp.max_abs(o.float(), ref["o"]) <= hp.BF16_OUT_ABS_TOL
+    for j in range(len(cu) - 1):
+        if cu[j + 1] == cu[j]:
+            assert mu[j].abs().max().item() == 0.0
+            assert torch.equal(I[j].cpu(), inp["Ip"].view(H, 1, 1).expand(H, d, d))
