@@ -52,6 +52,7 @@ struct BwdArgs {
   float* wInitPart;       // [n_seqs,H,dv*dk/256] partial sums of dJ_0
   double *wDgPart, *wDIpPart;  // [n_seqs,H]
   int32_t tokens;
+  int32_t apply_alias;     // carry apply: db^carry shares LDS with the bf16 carries (large head dims)
 };
 
 constexpr int kVS2 = 68;
@@ -565,7 +566,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   float* sBt = sW4 + 8;                    // [64][dv/8] beta of the carry terms, one slot per work item
   float* sO1 = sBt + kC * (dv >> 3);       // [64][OS] dk^carry, later dv^carry
   float* sO2 = sO1 + kC * (dmax + 4);      // [64][OS] db^carry
-  bf16_t* sRT = (bf16_t*)(sO2 + kC * (dmax + 4));   // [2][dk][dv + 8] R_M^T, R_J^T in bf16, operand source of all four products
+  // [2][dk][dv + 8] R_M^T, R_J^T in bf16, operand source of all four products.  When both do not fit the LDS
+  // (large head dims) the bf16 copy shares its bytes with db^carry and the dv/db products read the fp32
+  // carries from global memory instead.
+  const bool alias = A.apply_alias != 0;
+  bf16_t* sRT = (bf16_t*)(alias ? sO2 : sO2 + kC * (dmax + 4));
   const int RS = dv + 8;
   const int OS = dmax + 4;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
@@ -738,13 +743,23 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         if (ks < KS) {
           const int n0 = 8 * g + 32 * ks;
           bf16x8 B1, B2;
-          if (n0 < dk) {
+          if (n0 < dk && !alias) {
             // 8 consecutive key columns of value row d = 16db_ + i: a column walk through the transposed
             // bf16 copy in LDS (the fp32 carries in global memory would miss L2 on this second read)
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               B1[j] = sRT[(n0 + j) * RS + 16 * db_ + i];
               B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i];
+            }
+          } else if (n0 < dk) {
+            const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
+            const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
+            const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
+            const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
+              B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
             }
           } else {
 #pragma unroll
@@ -977,7 +992,14 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
     const int dmax = dd.dk > dd.dv ? dd.dk : dd.dv;
-    const size_t lds = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3) + 2 * (size_t)kC * (dmax + 4)) + 2 * (size_t)2 * dd.dk * (dd.dv + 8);
+    const size_t rt_bytes = 2 * (size_t)2 * dd.dk * (dd.dv + 8), o_bytes = sizeof(float) * kC * (dmax + 4);
+    const size_t lds_fixed = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3)) + o_bytes;
+    size_t lds = lds_fixed + o_bytes + rt_bytes;
+    A.apply_alias = 0;
+    if (lds > kMaxLds) {
+      A.apply_alias = 1;
+      lds = lds_fixed + (rt_bytes > o_bytes ? rt_bytes : o_bytes);
+    }
     if (lds > kMaxLds) return PAL_E_HEADDIM;
     if (bf) {
       if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<bf16_t>, lds)) return rc2;

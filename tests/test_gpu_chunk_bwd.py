@@ -89,7 +89,8 @@ def test_bf16_backward_lengths(gpu_device, T):
 
 
 @pytest.mark.parametrize("dk,dv", [(16, 16), (32, 48), (96, 96), (128, 128), (64, 192), (31, 65),
-                                   (80, 32), (112, 16), (144, 32), (256, 16)])  # uneven / 3 / 4 column passes
+                                   (80, 32), (112, 16), (144, 32), (256, 16),  # uneven / 3 / 4 column passes
+                                   (96, 192), (192, 96)])  # largest staging buffers of the carry pass
 def test_bf16_backward_head_dims_initial_state_and_var(gpu_device, dk, dv):
     B, T, H = 2, 150, 2
     inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=dk + 7 * dv), torch.bfloat16)
