@@ -107,3 +107,21 @@ def test_head_dim_padding_rules():
     assert cm.padded_dv(65) == 80
     with pytest.raises(ValueError):
         cm.padded_dk(300, True)
+
+
+def test_simple_gla_wrappers_keep_the_layer_call_site_keywords():
+    """palimpsa/layers/palimpsa.py:296-298 calls q=, k=, v=, g=, initial_state=, output_final_state=, cu_seqlens=."""
+    import inspect
+    import pytest
+    import torch
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    for fn in (chunk_simple_gla, fused_recurrent_simple_gla):
+        names = list(inspect.signature(fn).parameters)
+        assert names[:4] == ["q", "k", "v", "g"]
+        for n in ("scale", "initial_state", "output_final_state", "cu_seqlens"):
+            assert n in names
+        x = torch.zeros(1, 4, 2, 16)
+        with pytest.raises(ValueError):
+            fn(q=x, k=x, v=x, g=None)
+        with pytest.raises(ValueError):
+            fn(q=x, k=x, v=x, g=torch.zeros(1, 4, 3))
