@@ -3,6 +3,7 @@ palimpsa/ops/palimpsa/__init__.py:4-5."""
 from .chunk import ChunkPalimpsa, chunk_palimpsa
 from .fused_recurrent import FusedRecurrentPalimpsaFunction, fused_recurrent_palimpsa
 from .naive import palimpsa_ref
+from .decode import DecodeStep
 
 __all__ = [
     "chunk_palimpsa",
@@ -10,4 +11,5 @@ __all__ = [
     "palimpsa_ref",
     "ChunkPalimpsa",
     "FusedRecurrentPalimpsaFunction",
+    "DecodeStep",
 ]

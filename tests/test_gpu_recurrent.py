@@ -219,3 +219,61 @@ def test_bf16_rows_backward(gpu_device):
     # per-head reductions over all tokens of those rounded terms: the bf16 gradient bar
     for n in ["g", "Ip"]:
         assert hp.max_rel(got[n], ref[n]) <= hp.BF16_GRAD_NORM_TOL, n
+
+
+def test_bound_decode_step_matches_entry_point_and_replays_in_a_graph(gpu_device):
+    """DecodeStep binds tensors once and updates the state in place: same kernel as
+    fused_recurrent_palimpsa with T = 1, so results agree exactly; recorded into a HIP graph (the step
+    allocates nothing and records no memset) every replay agrees with the eager result too."""
+    from palimpsa_amd.ops.palimpsa import DecodeStep, fused_recurrent_palimpsa
+    B, H, dk, dv, steps = 5, 3, 64, 32, 6
+    dev = gpu_device
+    inp = hp.rounded(po.make_inputs(B, steps, H, dk, dv, seed=61), torch.bfloat16)
+    d = hp.to_device(inp, dev)
+    gen = torch.Generator().manual_seed(62)
+    mu0 = (torch.randn(B, H, dv, dk, generator=gen) * 0.1).to(dev)
+    I0 = (1.0 + torch.rand(B, H, dv, dk, generator=gen)).to(dev)
+    # eager entry point, state fed back
+    mu, I = mu0.clone(), I0.clone()
+    outs = []
+    for t in range(steps):
+        r = {n: d[n][:, t:t + 1].contiguous() for n in ("q", "k", "v", "b", "gt")}
+        (o, ov), mu, I = fused_recurrent_palimpsa(r["q"], r["k"], r["v"], r["b"], r["gt"], d["g"], d["Ip"],
+                                                  initial_mu_state=mu, initial_I_state=I, output_final_state=True,
+                                                  output_uncertainty=True)
+        outs.append((o, ov))
+    # bound step, rows copied into fixed buffers
+    dec = DecodeStep(B, H, dk, dv, dev, torch.bfloat16, output_uncertainty=True)
+    buf = {n: torch.empty_like(d[n][:, :1].contiguous()) for n in ("q", "k", "v", "b", "gt")}
+    mu_b, I_b = mu0.clone(), I0.clone()
+    dec.bind(buf["q"], buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"], mu_b, I_b)
+    for t in range(steps):
+        for n in buf:
+            buf[n].copy_(d[n][:, t:t + 1])
+        o = dec.step()
+        assert torch.equal(o, outs[t][0]) and torch.equal(dec.o_var, outs[t][1])
+    assert torch.equal(mu_b, mu) and torch.equal(I_b, I)
+    # the same steps from a captured graph, replayed with eager work in between
+    mu_b.copy_(mu0); I_b.copy_(I0)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        buf_warm = {n: buf[n].clone() for n in buf}
+        dec.step()                       # warm-up on the capture stream
+        mu_b.copy_(mu0); I_b.copy_(I0)
+        with torch.cuda.graph(graph, stream=side):
+            dec.step()
+    torch.cuda.current_stream().wait_stream(side)
+    for t in range(steps):
+        for n in buf:
+            buf[n].copy_(d[n][:, t:t + 1])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dec.o, outs[t][0]), t
+    assert torch.equal(mu_b, mu) and torch.equal(I_b, I)
+    with pytest.raises(ValueError):
+        dec.bind(buf["q"].float(), buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"], mu_b, I_b)
+    with pytest.raises(ValueError):
+        DecodeStep(B, H, 40, dv, dev)
