@@ -153,6 +153,17 @@ int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
  * max(|v|,|b|) * max(1,|k|^2) < 2^28 are required of the rows of a 64-token tile. */
 int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
+/* Chunked forward without the precision state (scalar-gated linear attention):
+ *   S_t = exp(-gt_t g) S_{t-1} + v_t k_t^T,  o_t = scale S_t q_t.
+ * Replaces the forward of fla.ops.simple_gla.chunk_simple_gla as the reference
+ * layer calls it with metaplasticity off (palimpsa/layers/palimpsa.py:18,
+ * :293-300; flash-linear-attention is a dependency of the reference, not part
+ * of its tree).  Reads q, k, v, gt, g, [init_mu], cu_seqlens + chunk tables;
+ * writes o, [final_mu] and chunk_mu (tile-start states S, [total_chunks,H,dv,dk]
+ * fp32).  b, Ip, o_var, init_I, final_I, chunk_I are ignored; PAL_FLAG_HAS_VAR
+ * is rejected with PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk]. */
+int pal_gla_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
+
 /* Chunked backward.  Replaces ChunkPalimpsa.backward + chunk_palimpsa_bwd_kernel
  * (chunk_palimpsa_forgetting_scalar.py:239-434, :519-620), including the host
  * side .sum(0) reductions of :609-613.  Needs chunk_mu / chunk_I as written by

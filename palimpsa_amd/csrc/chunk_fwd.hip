@@ -49,7 +49,9 @@ __device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_str
   }
 }
 
-template <typename TIn>
+// HAS_J = false drops the precision branch (b is not read, chunk_I is not written): the scalar-gated linear
+// attention that the layer uses without its precision state.
+template <typename TIn, bool HAS_J>
 __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
   const int H = a.H, dk = a.dk, dv = a.dv;
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
   }
   stage_transposed((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, (int64_t)H * dk, dk, clen, sKT, tid);
   stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sVT, tid);
-  stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sBT, tid);
+  if (HAS_J) stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sBT, tid);
   __syncthreads();
   float as[2][8];
 #pragma unroll
@@ -98,25 +100,27 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
         float vv[8], bb[8];
         *(f32x4*)&vv[0] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
         *(f32x4*)&vv[4] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
-        *(f32x4*)&bb[0] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
-        *(f32x4*)&bb[4] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
+        if (HAS_J) {
+          *(f32x4*)&bb[0] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
+          *(f32x4*)&bb[4] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           AM[ks][j] = (bf16_t)(as[ks][j] * vv[j]);
-          AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
+          if (HAS_J) AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
         }
       }
       f32x4 M = {0.f, 0.f, 0.f, 0.f}, J = {0.f, 0.f, 0.f, 0.f};
       M = mfma16(AM[0], BK[0], M);
-      J = mfma16(AJ[0], BKK[0], J);
+      if (HAS_J) J = mfma16(AJ[0], BKK[0], J);
       M = mfma16(AM[1], BK[1], M);
-      J = mfma16(AJ[1], BKK[1], J);
+      if (HAS_J) J = mfma16(AJ[1], BKK[1], J);
       // accumulator layout: rows d = 16dt + 4g + r, column n = 16nb + i
       const int64_t co = (((int64_t)cidx * H + h) * dv + 16 * dt + 4 * g) * dk + 16 * nb + i;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         a.chunk_mu[co + (int64_t)r * dk] = M[r];
-        a.chunk_I[co + (int64_t)r * dk] = J[r];
+        if (HAS_J) a.chunk_I[co + (int64_t)r * dk] = J[r];
       }
     }
   }
@@ -197,6 +201,54 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
     a.final_mu[so] = SM * fast_rcp(I);
     a.final_I[so] = I;
   }
+}
+
+// The same scan without the precision state: S_c = F_c S_{c-1} + Delta_c, the slots of chunk_mu end up
+// holding the state at the start of their tile, the last state goes to final_mu.
+__global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
+  __shared__ float sF[kScanTiles];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int64_t E = (int64_t)a.dv * a.dk;
+  const int nblk = (int)(E / 256);
+  const int blk = blockIdx.x % nblk;
+  const int nh = blockIdx.x / nblk;
+  const int h = nh % a.H, n = nh / a.H;
+  const int64_t e = (int64_t)blk * 256 + tid;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const int nchunks = (len + kC - 1) / kC;
+  const float gh = a.g[h] * kLog2e;
+  const int64_t so = (int64_t)nh * E + e;
+  float S = a.init_mu ? a.init_mu[so] : 0.f;
+  for (int c0 = 0; c0 < nchunks; c0 += kScanTiles) {
+    const int cn = min(kScanTiles, nchunks - c0);
+    __syncthreads();
+    for (int c = w; c < cn; c += 4) {
+      const int t = (c0 + c) * kC + lane;
+      const float gt = (t < len) ? load_gate(a.gt, (int64_t)(bos + t) * a.H + h, a.gate_bf16) : 0.f;
+      const float tot = wave_sum(-gt * gh);
+      if (lane == 0) sF[c] = fast_exp2(tot);
+    }
+    __syncthreads();
+    int c = 0;
+    for (; c + 8 <= cn; c += 8) {
+      float dS[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) dS[u] = a.chunk_mu[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        a.chunk_mu[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e] = S;
+        S = fmaf(sF[c + u], S, dS[u]);
+      }
+    }
+    for (; c < cn; ++c) {
+      const int64_t off = ((int64_t)(cbase + c0 + c) * a.H + h) * E + e;
+      const float dS = a.chunk_mu[off];
+      a.chunk_mu[off] = S;
+      S = fmaf(sF[c], S, dS);
+    }
+  }
+  if (a.final_mu) a.final_mu[so] = S;
 }
 
 // ------------------------------------------------------------------ kernel 2
@@ -473,6 +525,43 @@ void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
 
 }  // namespace pal
 
+namespace pal {
+
+// Tile-start states: local contributions, then the serial scan over the tiles of each sequence.
+// has_j = false leaves the precision state out (b, Ip, chunk_I, init_I, final_I are not touched).
+int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
+  {
+    const int64_t blocks = (int64_t)a.total_chunks * a.H;
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    const size_t lds = sizeof(float) * (kC + (size_t)(a.dk + (has_j ? 2 : 1) * a.dv) * kTS);
+    if (lds > kMaxLds) return PAL_E_HEADDIM;
+    const void* fn;
+    if (dtype == PAL_DTYPE_BF16)
+      fn = has_j ? (const void*)&chunk_delta_kernel<bf16_t, true> : (const void*)&chunk_delta_kernel<bf16_t, false>;
+    else
+      fn = has_j ? (const void*)&chunk_delta_kernel<float, true> : (const void*)&chunk_delta_kernel<float, false>;
+    if (int rc = allow_lds(fn, lds)) return rc;
+    if (dtype == PAL_DTYPE_BF16) {
+      if (has_j) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t, true>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+      else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t, false>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+    } else {
+      if (has_j) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float, true>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+      else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float, false>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+    }
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  {
+    const int64_t blocks = (int64_t)a.n_seqs * a.H * (((int64_t)a.dv * a.dk) / 256);
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    if (has_j) PAL_TIMED_LAUNCH(kKernChunkScan, s, chunk_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    else PAL_TIMED_LAUNCH(kKernChunkScan, s, gla_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  return PAL_OK;
+}
+
+}  // namespace pal
+
 extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
   using namespace pal;
   int rc = check_chunk_common(d, t);
@@ -480,26 +569,7 @@ extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* str
   ChunkArgs a;
   fill_chunk_args(a, d, t);
   hipStream_t s = (hipStream_t)stream;
-  {
-    const int64_t blocks = (int64_t)d->total_chunks * d->n_heads;
-    if (blocks > 0x7fffffff) return PAL_E_DIM;
-    const size_t lds = sizeof(float) * (kC + (size_t)(d->dk + 2 * d->dv) * kTS);
-    if (lds > kMaxLds) return PAL_E_HEADDIM;
-    if (d->dtype == PAL_DTYPE_BF16) {
-      if (int rc2 = allow_lds((const void*)&chunk_delta_kernel<bf16_t>, lds)) return rc2;
-      PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-    } else {
-      if (int rc2 = allow_lds((const void*)&chunk_delta_kernel<float>, lds)) return rc2;
-      PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-    }
-    PAL_HIP_LAUNCH_CHECK();
-  }
-  {
-    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk) / 256);
-    if (blocks > 0x7fffffff) return PAL_E_DIM;
-    PAL_TIMED_LAUNCH(kKernChunkScan, s, chunk_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
-    PAL_HIP_LAUNCH_CHECK();
-  }
+  if (int rc2 = launch_tile_states(a, d->dtype, true, s)) return rc2;
   if (d->dtype == PAL_DTYPE_BF16) return launch_out<bf16_t>(a, s);
   return launch_out<float>(a, s);
 }

@@ -16,6 +16,7 @@ enum KernelId {
   kKernBwdHeadReduce,
   kKernRecurrentBwdFwdPass,
   kKernRecurrentBwd,
+  kKernGlaOut,
   kKernCount
 };
 

@@ -47,7 +47,7 @@ static void drain() {
 static const char* kNames[kKernCount] = {
     "recurrent_fwd_kernel", "chunk_delta_kernel", "chunk_scan_kernel", "chunk_out_kernel", "chunk_bwd_local_kernel",
     "chunk_bwd_carry_scan_kernel", "chunk_bwd_carry_apply_kernel", "chunk_bwd_gate_kernel",
-    "chunk_bwd_head_reduce_kernel", "recurrent_bwd_state_kernel", "recurrent_bwd_kernel"};
+    "chunk_bwd_head_reduce_kernel", "recurrent_bwd_state_kernel", "recurrent_bwd_kernel", "gla_out_kernel"};
 
 }  // namespace pal
 

@@ -90,3 +90,82 @@ def test_packed_documents(gpu_device):
         o_ref, S_ref = _closed_form(q[:, sl], k[:, sl], v[:, sl], g[:, sl], dk ** -0.5)
         assert hp.max_abs(o[:, sl].float(), o_ref) <= hp.BF16_OUT_ABS_TOL
         assert hp.max_rel(S[j:j + 1], S_ref) <= 1e-2
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,dtype", [
+    (2, 64, 2, 64, 64, torch.bfloat16),      # exactly one tile
+    (1, 1, 1, 16, 16, torch.bfloat16),       # one token, smallest head dims
+    (2, 333, 3, 48, 80, torch.bfloat16),     # key dim not a multiple of 32, ragged last tile
+    (1, 257, 2, 128, 128, torch.bfloat16),
+    (1, 130, 1, 256, 256, torch.bfloat16),   # largest head dims
+    (1, 100, 2, 40, 24, torch.bfloat16),     # head dims padded by the host to multiples of 16
+    (2, 150, 2, 64, 32, torch.float32),      # fp32 rows (operands are rounded to bf16 in the kernel)
+])
+def test_forward_only_kernel_shapes(gpu_device, B, T, H, dk, dv, dtype):
+    """The forward of its own that chunk_simple_gla takes without autograd, against the closed form and against
+    the autograd path (the Palimpsa kernels on b = 0) on the same inputs."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 21)
+    q, k, v = (x.to(dtype) for x in (q, k, v))
+    dev = gpu_device
+    with torch.no_grad():
+        o, S = chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), scale=0.7,
+                                initial_state=S0.to(dev), output_final_state=True)
+    assert o.dtype == dtype and o.shape == (B, T, H, dv) and S.shape == (B, H, dk, dv)
+    o_ref, S_ref = _closed_form(q, k, v, g, 0.7, S0)
+    assert hp.max_abs(o.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_ref) <= 1e-2
+    if dk + 2 * dv > 600:
+        return          # beyond the LDS budget of the Palimpsa tile-state kernel, which stages k, v and b in fp32
+    qg = q.to(dev).requires_grad_(True)
+    o_g, S_g = chunk_simple_gla(q=qg, k=k.to(dev), v=v.to(dev), g=g.to(dev), scale=0.7,
+                                initial_state=S0.to(dev), output_final_state=True)
+    assert o_g.grad_fn is not None
+    assert hp.max_abs(o.float(), o_g.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_g) <= 1e-2
+
+
+def test_forward_only_strong_and_weak_decay(gpu_device):
+    """Decay so strong that a tile forgets its start, and none at all (g = 0: plain causal linear attention)."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    B, T, H, dk, dv = 1, 192, 2, 64, 64
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 22)
+    g = torch.stack([torch.full((B, T), -3.0), torch.zeros(B, T)], dim=-1)
+    dev = gpu_device
+    with torch.no_grad():
+        o, S = chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), initial_state=S0.to(dev),
+                                output_final_state=True)
+    o_ref, S_ref = _closed_form(q, k, v, g, dk ** -0.5, S0)
+    assert hp.max_abs(o.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_ref) <= 1e-2
+
+
+def test_forward_only_full_size_against_token_serial(gpu_device):
+    """Headline shape (B=8, T=2048, H=12, d=64): whole result against the token-serial fp32-state kernel, a slice
+    against the closed form."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    B, T, H, d = 8, 2048, 12, 64
+    q, k, v, g, S0 = _inputs(B, T, H, d, d, 23)
+    dev = gpu_device
+    args = dict(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), initial_state=S0.to(dev), output_final_state=True)
+    with torch.no_grad():
+        o, S = chunk_simple_gla(**args)
+        o_r, S_r = fused_recurrent_simple_gla(**args)
+    assert hp.max_abs(o.float(), o_r.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_r) <= 1e-2
+    bs, hs = [5], [0, 11]
+    sub = lambda x: x[bs][:, :512][:, :, hs]
+    o_ref, _ = _closed_form(sub(q), sub(k), sub(v), sub(g), d ** -0.5, S0[bs][:, hs])
+    assert hp.max_abs(o[bs][:, :512][:, :, hs].float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+
+
+def test_forward_only_rejects_bad_arguments(gpu_device):
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    q, k, v, g, _ = _inputs(2, 70, 2, 32, 32, 24)
+    dev = gpu_device
+    with pytest.raises(ValueError):
+        chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=None)
+    with pytest.raises(ValueError):
+        chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), cu_seqlens=torch.tensor([0, 70], device=dev))
+    with pytest.raises(ValueError):
+        chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g[:, :10].to(dev))
