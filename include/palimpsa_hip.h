@@ -164,6 +164,17 @@ int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
  * is rejected with PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk]. */
 int pal_gla_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
+/* Backward of pal_gla_chunk_fwd (replaces the backward of fla's chunk_simple_gla
+ * for the same call site).  t as in the forward call, with chunk_mu as that call
+ * left it, t->o any valid pointer (not read) and PAL_FLAG_STORE_FINAL clear.
+ * Reads gr->d_o; writes gr->dq, dk, dv (dtype), gr->dgt (fp32 [B,T,H], gradient
+ * of gt), gr->dg (fp32 [H], gradient of the per-head rate g) and, when not NULL,
+ * gr->d_init_mu (fp32 [N,H,dv,dk]).  d_o_var, db, dIp, d_init_I are ignored.
+ * Gradients flowing into the final state are not taken (as in pal_chunk_bwd). */
+size_t pal_gla_chunk_bwd_workspace_bytes(const PalDims *dims);
+int pal_gla_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* Chunked backward.  Replaces ChunkPalimpsa.backward + chunk_palimpsa_bwd_kernel
  * (chunk_palimpsa_forgetting_scalar.py:239-434, :519-620), including the host
  * side .sum(0) reductions of :609-613.  Needs chunk_mu / chunk_I as written by

@@ -76,11 +76,12 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [P(PalDims), P(PalFwdTensors), C.c_void_p]
-    for name in ("pal_recurrent_bwd", "pal_chunk_bwd"):
+    for name in ("pal_recurrent_bwd", "pal_chunk_bwd", "pal_gla_chunk_bwd"):
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [P(PalDims), P(PalFwdTensors), P(PalBwdTensors), C.c_void_p, C.c_size_t, C.c_void_p]
-    for name in ("pal_recurrent_bwd_workspace_bytes", "pal_chunk_bwd_workspace_bytes"):
+    for name in ("pal_recurrent_bwd_workspace_bytes", "pal_chunk_bwd_workspace_bytes",
+                 "pal_gla_chunk_bwd_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = C.c_size_t
         fn.argtypes = [P(PalDims)]

@@ -14,6 +14,11 @@
 namespace pal {
 
 constexpr int kC = PAL_CHUNK;  // tokens per tile
+constexpr int kScanTiles = 1024;   // per-tile decays a scan kernel keeps in LDS at a time
+
+// internal bit of ChunkArgs::flags (above the PAL_FLAG_* bits): chunk_delta_kernel weights token s with the decay
+// from the start of the tile up to s instead of from s to the end of the tile
+constexpr uint32_t kFlagDecayFromStart = 1u << 30;
 
 struct ChunkArgs {
   const void *q, *k, *v, *b, *gt;

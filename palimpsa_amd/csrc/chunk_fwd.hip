@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
     const float gh = a.g[h] * kLog2e;
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     const float cs = wave_inclusive_scan(-gt * gh, lane);
-    sA[lane] = fast_exp2(__shfl(cs, 63) - cs);
+    sA[lane] = fast_exp2((a.flags & kFlagDecayFromStart) ? cs : __shfl(cs, 63) - cs);
   }
   stage_transposed((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, (int64_t)H * dk, dk, clen, sKT, tid);
   stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sVT, tid);
@@ -132,8 +132,6 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
 // chunk_mu / chunk_I is overwritten with the state at the START of its tile in (mu, I) form
 // (what the reference stores as intermediate_*_state, chunk_palimpsa_forgetting_scalar.py:187-188);
 // the state after the last tile goes to final_mu / final_I (:214-218).
-constexpr int kScanTiles = 1024;   // per-tile decays kept in LDS at a time
-
 __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -527,9 +525,8 @@ void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
 
 namespace pal {
 
-// Tile-start states: local contributions, then the serial scan over the tiles of each sequence.
-// has_j = false leaves the precision state out (b, Ip, chunk_I, init_I, final_I are not touched).
-int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
+// Local contribution of every tile to the state, into chunk_mu (and chunk_I when has_j).
+int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
   {
     const int64_t blocks = (int64_t)a.total_chunks * a.H;
     if (blocks > 0x7fffffff) return PAL_E_DIM;
@@ -550,6 +547,13 @@ int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s)
     }
     PAL_HIP_LAUNCH_CHECK();
   }
+  return PAL_OK;
+}
+
+// Tile-start states: local contributions, then the serial scan over the tiles of each sequence.
+// has_j = false leaves the precision state out (b, Ip, chunk_I, init_I, final_I are not touched).
+int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
+  if (int rc = launch_tile_delta(a, dtype, has_j, s)) return rc;
   {
     const int64_t blocks = (int64_t)a.n_seqs * a.H * (((int64_t)a.dv * a.dk) / 256);
     if (blocks > 0x7fffffff) return PAL_E_DIM;

@@ -1,0 +1,481 @@
+// Chunked forward of scalar-gated linear attention: the Palimpsa recurrence without its precision
+// state (b = 0, I = 1, so mu = M),
+//     S_t = f_t S_{t-1} + v_t k_t^T ,   o_t = scale * S_t q_t ,   f_t = exp(-gt_t * g) .
+// It is what the reference layer runs when metaplasticity is off (the simple_gla pair imported at
+// palimpsa/layers/palimpsa.py:18 and called at :293-300).  Without the division by I_t the output of
+// a tile is two plain matrix products,
+//     O = ((Q K^T) o L) V + diag(F) Q S_0^T ,      L[t,s] = 2^{c_t - c_s} (s <= t),  F_t = 2^{c_t},
+// so nothing of the [tokens x dv x dk] state has to be materialised per token: the tile-start states
+// come from the same two kernels as in the Palimpsa forward (local contribution + serial scan, both
+// without the J branch) and the kernel below does the rest on the matrix cores.
+#include "chunk_common.h"
+#include "pal_host.h"
+#include "pal_profile.h"
+
+namespace pal {
+
+void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t);
+int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
+int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
+
+constexpr int kVT = 72;  // row stride (bf16) of the transposed value tile
+
+template <typename TIn>
+__device__ __forceinline__ bf16x8 load_bf16x8(const TIn* p) {
+  if constexpr (sizeof(TIn) == 2) {
+    return *(const bf16x8*)p;
+  } else {
+    const f32x4 x = *(const f32x4*)p, y = *(const f32x4*)(p + 4);
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { r[e] = (bf16_t)x[e]; r[4 + e] = (bf16_t)y[e]; }
+    return r;
+  }
+}
+
+// Arguments of gla_tile_kernel: the shared tile/gate bookkeeping plus the roles of the three row tensors.
+struct GlaTileArgs {
+  ChunkArgs c;            // T, H, tiles, gate (gt, g), scale
+  const void *X, *Y;      // rows [token][H][dc]: X plays the query, Y the key of the scores
+  const void* Z;          // rows [token][H][de]: what the scores mix
+  const float* St;        // per-tile states [tile][H][dv][dk]
+  void* out;              // rows [token][H][de]
+  const void* W;          // optional rows [token][H][de]: dot[token] = sum_e W out (fp32, before rounding)
+  float* dot;             // [token][H] or null
+  int32_t dc, de;         // contraction width of the scores, width of the output rows
+};
+
+// One kernel for the tile-parallel part of the forward and of the three input gradients.  For the 64
+// tokens of a tile, with x the token of the output row and y the tokens it attends to,
+//     out[x, e] = scale * ( w_x sum_c St[e, c] X[x, c]  +  sum_y  (X[x,:] . Y[y,:]) L(x, y) Z[y, e] )
+//   forward (REVERSE = false):  y <= x,  L = 2^{c_x - c_y},  w_x = 2^{c_x}         (decay since the tile start)
+//   reverse (REVERSE = true):   y >= x,  L = 2^{c_y - c_x},  w_x = 2^{c_end - c_x} (decay up to the tile end)
+//   o   : X = q,  Y = k,  Z = v,  St = tile-start state S [dv][dk]
+//   dq  : X = dO, Y = v,  Z = k,  St = S read transposed (STATE_T)
+//   dv  : X = k,  Y = q,  Z = dO, St = gradient of the tile-end state G [dv][dk],      reverse
+//   dk  : X = v,  Y = dO, Z = q,  St = G read transposed,                              reverse
+// One workgroup of 4 waves per (tile, head); wave w owns the tokens x in [16w, 16w+16).
+//   P^T[y,x]   = sum_c Y[y,c] X[x,c]           A = Y rows (LDS), B = the wave's X rows (registers)
+//   P^T       *= L(x,y), masked                in the accumulator layout (column x per lane, 4 rows y)
+//   out^T[e,x] = w_x sum_c St[e,c] X[x,c]      A = state rows (global fp32 -> bf16)
+//              + sum_y Z^T[e,y] P^T[y,x]       A = Z^T rows (LDS), B = P^T straight from the accumulators:
+// the contraction index of that last product is mapped to tokens as slot (g, j) -> y = 32p + 16(j/4) +
+// 4g + j%4, which is where the accumulators of two neighbouring blocks already sit, and Z^T is read
+// with the same map (two 8-byte LDS reads per operand).
+// KS = ceil(dc / 32) contraction steps of the scores (operands zero padded to 32 KS).
+template <typename TIn, int KS, bool REVERSE, bool STATE_T>
+__global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
+  extern __shared__ float smem[];
+  const ChunkArgs& a = A.c;
+  const int H = a.H, dc = A.dc, de = A.de;
+  constexpr int dcp = 32 * KS + 8;    // row stride (bf16) of the Y tile
+  float* sC = smem;                   // [64] running log2 decay inside the tile
+  bf16_t* sY = (bf16_t*)(sC + kC);    // [64][dcp]
+  bf16_t* sZT = sY + kC * dcp;        // [de][kVT]
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int tb = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  if (tb == 0) {
+    const float gh = a.g[h] * kLog2e;
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    sC[lane] = wave_inclusive_scan(-gt * gh, lane);
+  }
+  // the wave's 16 X rows as B operands (column x = 16 tb + i, contraction index c = 32 ks + 8 g + j)
+  const int x = 16 * tb + i;
+  bf16x8 Xr[KS];
+  {
+    const TIn* xp = (const TIn*)A.X + ((int64_t)(t0 + x) * H + h) * dc + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Xr[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (x < clen && 32 * ks + 8 * g < dc) Xr[ks] = load_bf16x8(xp + 32 * ks);
+    }
+  }
+  {
+    // Y rows, zero beyond the tile's tokens and beyond dc
+    const TIn* yp = (const TIn*)A.Y + ((int64_t)t0 * H + h) * dc;
+    constexpr int groups = 4 * KS;
+    for (int idx = tid; idx < kC * groups; idx += 256) {
+      const int s = idx / groups, c8 = idx - s * groups;
+      bf16x8 yx = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (s < clen && 8 * c8 < dc) yx = load_bf16x8(yp + (int64_t)s * H * dc + 8 * c8);
+      *(bf16x8*)&sY[s * dcp + 8 * c8] = yx;
+    }
+    // Z transposed (token index fastest), zero beyond the tile's tokens.  A work item is two consecutive
+    // tokens by eight columns: neighbouring lanes read neighbouring 16-byte pieces of a row, and a
+    // pair of tokens goes to LDS as one 32-bit word per column.
+    const TIn* zp = (const TIn*)A.Z + ((int64_t)t0 * H + h) * de;
+    const int zgroups = de >> 3;
+    for (int idx = tid; idx < (kC / 2) * zgroups; idx += 256) {
+      const int sp = idx / zgroups, c8 = idx - sp * zgroups;
+      bf16x8 z0 = {0, 0, 0, 0, 0, 0, 0, 0}, z1 = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (2 * sp < clen) z0 = load_bf16x8(zp + (int64_t)(2 * sp) * H * de + 8 * c8);
+      if (2 * sp + 1 < clen) z1 = load_bf16x8(zp + (int64_t)(2 * sp + 1) * H * de + 8 * c8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *(bf16x2*)&sZT[(8 * c8 + e) * kVT + 2 * sp] = bf16x2{z0[e], z1[e]};
+    }
+  }
+  __syncthreads();
+
+  const float cx = sC[16 * tb + i];
+  const float wx = fast_exp2(REVERSE ? sC[kC - 1] - cx : cx);
+
+  // decayed, masked scores of the wave's 16 tokens against the blocks on their causal side, as B operands
+  bf16x8 P[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int yb = 2 * p + half;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      if (REVERSE ? yb >= tb : yb <= tb) {
+        const bf16_t* yrow = sY + (16 * yb + i) * dcp + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) acc = mfma16(*(const bf16x8*)(yrow + 32 * ks), Xr[ks], acc);
+        const f32x4 cy = *(const f32x4*)&sC[16 * yb + 4 * g];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const bool live = yb != tb || (REVERSE ? 4 * g + r >= i : 4 * g + r <= i);
+          acc[r] = live ? acc[r] * fast_exp2(REVERSE ? cy[r] - cx : cx - cy[r]) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) P[p][4 * half + r] = (bf16_t)acc[r];
+    }
+  }
+
+  const float scale = a.scale;
+  const float* St = A.St + ((int64_t)cidx * H + h) * dc * de;
+  TIn* orow = (TIn*)A.out + ((int64_t)(t0 + x) * H + h) * de + 4 * g;
+  const TIn* wrow = (const TIn*)A.W + ((int64_t)(t0 + x) * H + h) * de + 4 * g;
+  const bool has_dot = A.dot != nullptr;
+  float dot = 0.f;
+  const int n_eb = de >> 4;
+  // four blocks of 16 output columns at a time, so that the loads of the state are in flight together
+  for (int eb0 = 0; eb0 < n_eb; eb0 += 4) {
+    f32x4 acc[4];
+    const float* srow[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int e = 16 * min(eb0 + u, n_eb - 1) + i;   // a block past the end repeats the last one
+      srow[u] = STATE_T ? St + (int64_t)(8 * g) * de + e : St + (int64_t)e * dc + 8 * g;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      bf16x8 Sa[4];
+      const bool ok = 32 * ks + 8 * g < dc;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        Sa[u] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (ok) {
+          if constexpr (STATE_T) {
+            // the state is stored [c][e]: eight rows apart, neighbouring lanes read neighbouring columns
+#pragma unroll
+            for (int j = 0; j < 8; ++j) Sa[u][j] = (bf16_t)srow[u][(int64_t)(32 * ks + j) * de];
+          } else {
+            Sa[u] = load_bf16x8(srow[u] + 32 * ks);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] = mfma16(Sa[u], Xr[ks], acc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int eb = min(eb0 + u, n_eb - 1);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[u][r] *= wx;
+      const bf16_t* zrow = sZT + (16 * eb + i) * kVT + 4 * g;
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        if (REVERSE ? 2 * p + 1 >= tb : 2 * p <= tb) {
+          const bf16x4 lo = *(const bf16x4*)(zrow + 32 * p), hi = *(const bf16x4*)(zrow + 32 * p + 16);
+          const bf16x8 Za = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          acc[u] = mfma16(Za, P[p], acc[u]);
+        }
+      }
+      if (x < clen && eb0 + u < n_eb) {
+        const float res[4] = {acc[u][0] * scale, acc[u][1] * scale, acc[u][2] * scale, acc[u][3] * scale};
+        store_vec<4>(orow + 16 * eb, res);
+        if (has_dot) {
+          float wv[4];
+          load_vec<4>(wrow + 16 * eb, wv);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) dot = fmaf(wv[r], res[r], dot);
+        }
+      }
+    }
+  }
+  if (has_dot) {
+    dot = rows4_sum(dot);
+    if (g == 0 && x < clen) A.dot[(int64_t)(t0 + x) * H + h] = dot;
+  }
+}
+
+enum GlaRole { kGlaOut = 0, kGlaDq, kGlaDv, kGlaDk };
+
+template <typename TIn, int KS, bool REVERSE, bool STATE_T>
+static int launch_gla_tile_ks(const GlaTileArgs& A, int kern_id, hipStream_t s) {
+  const size_t lds = sizeof(float) * kC + sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+  const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
+  if (blocks > 0x7fffffff) return PAL_E_DIM;
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  if (int rc = allow_lds((const void*)&gla_tile_kernel<TIn, KS, REVERSE, STATE_T>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kern_id, s, (gla_tile_kernel<TIn, KS, REVERSE, STATE_T>), dim3((unsigned)blocks), dim3(256), lds, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+template <typename TIn, bool REVERSE, bool STATE_T>
+static int launch_gla_tile_rs(const GlaTileArgs& A, int kern_id, hipStream_t s) {
+  switch ((A.dc + 31) / 32) {
+    case 1: return launch_gla_tile_ks<TIn, 1, REVERSE, STATE_T>(A, kern_id, s);
+    case 2: return launch_gla_tile_ks<TIn, 2, REVERSE, STATE_T>(A, kern_id, s);
+    case 3: return launch_gla_tile_ks<TIn, 3, REVERSE, STATE_T>(A, kern_id, s);
+    case 4: return launch_gla_tile_ks<TIn, 4, REVERSE, STATE_T>(A, kern_id, s);
+    case 5: return launch_gla_tile_ks<TIn, 5, REVERSE, STATE_T>(A, kern_id, s);
+    case 6: return launch_gla_tile_ks<TIn, 6, REVERSE, STATE_T>(A, kern_id, s);
+    case 7: return launch_gla_tile_ks<TIn, 7, REVERSE, STATE_T>(A, kern_id, s);
+    case 8: return launch_gla_tile_ks<TIn, 8, REVERSE, STATE_T>(A, kern_id, s);
+    default: return PAL_E_HEADDIM;
+  }
+}
+
+template <typename TIn>
+static int launch_gla_tile(const GlaTileArgs& A, GlaRole role, hipStream_t s) {
+  switch (role) {
+    case kGlaOut: return launch_gla_tile_rs<TIn, false, false>(A, kKernGlaOut, s);
+    case kGlaDq: return launch_gla_tile_rs<TIn, false, true>(A, kKernGlaDq, s);
+    case kGlaDv: return launch_gla_tile_rs<TIn, true, false>(A, kKernGlaDv, s);
+    default: return launch_gla_tile_rs<TIn, true, true>(A, kKernGlaDk, s);
+  }
+}
+
+static int launch_gla_tile_dt(const GlaTileArgs& A, int dtype, GlaRole role, hipStream_t s) {
+  return dtype == PAL_DTYPE_BF16 ? launch_gla_tile<bf16_t>(A, role, s) : launch_gla_tile<float>(A, role, s);
+}
+
+// argument checks shared by the forward and the backward entry points
+static int check_gla(const PalDims* d, const PalFwdTensors* t) {
+  int rc = pal_validate_dims(d);
+  if (rc) return rc;
+  if (!t) return PAL_E_NULL;
+  if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o || !t->chunk_mu) return PAL_E_NULL;
+  if (d->flags & PAL_FLAG_HAS_VAR) return PAL_E_STATE;   // no precision state, no output variance
+  if (((d->flags & PAL_FLAG_HAS_INIT) != 0) != (t->init_mu != nullptr)) return PAL_E_STATE;
+  if (((d->flags & PAL_FLAG_STORE_FINAL) != 0) != (t->final_mu != nullptr)) return PAL_E_STATE;
+  const bool varlen = d->flags & PAL_FLAG_VARLEN;
+  if (varlen != (t->cu_seqlens != nullptr)) return PAL_E_CU_SEQLENS;
+  if (varlen && (!t->chunk_table || !t->chunk_offsets)) return PAL_E_NULL;
+  if (d->total_chunks <= 0) return PAL_E_CHUNK;
+  const int64_t per = ((int64_t)d->seq_len + PAL_CHUNK - 1) / PAL_CHUNK;
+  if (varlen) {
+    if (d->total_chunks < per || d->total_chunks > (int64_t)d->seq_len / PAL_CHUNK + d->n_seqs) return PAL_E_CHUNK;
+  } else if ((int64_t)d->total_chunks != per * d->batch) {
+    return PAL_E_CHUNK;
+  }
+  const void* ptrs[] = {t->q, t->k, t->v, t->o, t->init_mu, t->final_mu, t->chunk_mu};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  return PAL_OK;
+}
+
+// the shared argument block carries no precision tensors on this path
+static void fill_gla_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
+  PalFwdTensors tt = *t;
+  tt.b = nullptr; tt.Ip = nullptr; tt.o_var = nullptr;
+  tt.init_I = nullptr; tt.final_I = nullptr; tt.chunk_I = nullptr;
+  fill_chunk_args(a, d, &tt);
+}
+
+// ------------------------------------------------------------------ backward
+// Gradient of the state at the END of every tile, G_c = F_{c+1} G_{c+1} + D_{c+1}, from the tiles' own
+// contributions D_c = sum_t F_t dO_t q_t^T parked in buf by chunk_delta_kernel: the forward scan run
+// backwards.  One thread per (sequence, head, state entry); slot c of buf ends up holding G_c.  What is
+// left after the first tile, times scale, is the gradient of the initial state.
+__global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, float* buf, float* d_init) {
+  __shared__ float sF[kScanTiles];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int64_t E = (int64_t)a.dv * a.dk;
+  const int nblk = (int)(E / 256);
+  const int blk = blockIdx.x % nblk;
+  const int nh = blockIdx.x / nblk;
+  const int h = nh % a.H, n = nh / a.H;
+  const int64_t e = (int64_t)blk * 256 + tid;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const int nchunks = (len + kC - 1) / kC;
+  const float gh = a.g[h] * kLog2e;
+  float G = 0.f;
+  for (int c_hi = nchunks; c_hi > 0; c_hi -= kScanTiles) {
+    const int c0 = max(0, c_hi - kScanTiles), cn = c_hi - c0;
+    __syncthreads();
+    for (int c = w; c < cn; c += 4) {
+      const int t = (c0 + c) * kC + lane;
+      const float gt = (t < len) ? load_gate(a.gt, (int64_t)(bos + t) * a.H + h, a.gate_bf16) : 0.f;
+      const float tot = wave_sum(-gt * gh);
+      if (lane == 0) sF[c] = fast_exp2(tot);
+    }
+    __syncthreads();
+    int c = cn;
+    for (; c >= 8; c -= 8) {
+      float D[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) D[u] = buf[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        buf[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e] = G;
+        G = fmaf(sF[c - 1 - u], G, D[u]);
+      }
+    }
+    for (; c >= 1; --c) {
+      const int64_t off = ((int64_t)(cbase + c0 + c - 1) * a.H + h) * E + e;
+      const float D = buf[off];
+      buf[off] = G;
+      G = fmaf(sF[c - 1], G, D);
+    }
+  }
+  if (d_init) d_init[(int64_t)nh * E + e] = a.scale * G;
+}
+
+// Gate gradients.  With C_t the running sum of the log decay l_t = -gt_t g over a sequence, q_t enters
+// the output only as q_t e^{C_t} and k_t only as k_t e^{-C_t}, so dC_t = q_t . dq_t - k_t . dk_t (the two
+// dot products come from the dq and dk kernels in fp32) and dl_t is the sum of dC over the tokens from t
+// to the end of the sequence.  One wave per (sequence, head) walks the tiles from the last to the first;
+// dgt_t = -g dl_t, and the wave's share of dg = -sum_t gt_t dl_t goes to dg_part[seq][head].
+__global__ __launch_bounds__(64) void gla_bwd_gate_kernel(ChunkArgs a, const float* qdq, const float* kdk, float* dgt,
+                                                          float* dg_part) {
+  const int lane = threadIdx.x;
+  const int h = blockIdx.x % a.H, n = blockIdx.x / a.H;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const float gh = a.g[h];
+  float carry = 0.f, acc = 0.f;
+  for (int base = ((len - 1) / kC) * kC; base >= 0; base -= kC) {
+    const int t = base + lane;
+    const int64_t off = (int64_t)(bos + t) * a.H + h;
+    float x = (t < len) ? qdq[off] - kdk[off] : 0.f;
+    // inclusive suffix sum over the 64 lanes
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float y = __shfl_down(x, d);
+      if (lane + d < 64) x += y;
+    }
+    const float dl = x + carry;
+    carry += __shfl(x, 0);
+    if (t < len) {
+      dgt[off] = -gh * dl;
+      acc = fmaf(load_gate(a.gt, off, a.gate_bf16), dl, acc);
+    }
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) dg_part[(int64_t)n * a.H + h] = -acc;
+}
+
+// dg[h] = sum over the sequences, in a fixed order
+__global__ void gla_bwd_head_reduce_kernel(const float* dg_part, float* dg, int n_seqs, int H) {
+  const int h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= H) return;
+  float s = 0.f;
+  for (int n = 0; n < n_seqs; ++n) s += dg_part[(int64_t)n * H + h];
+  dg[h] = s;
+}
+
+// workspace of the backward: G tiles, the two dot-product rows, per-sequence shares of dg
+struct GlaBwdWorkspace {
+  size_t g_tiles, qdq, kdk, dg_part, total;
+};
+static GlaBwdWorkspace gla_bwd_layout(const PalDims* d) {
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  GlaBwdWorkspace w;
+  const size_t tokens = (size_t)d->batch * d->seq_len;
+  w.g_tiles = 0;
+  w.qdq = w.g_tiles + up(sizeof(float) * (size_t)d->total_chunks * d->n_heads * d->dv * d->dk);
+  w.kdk = w.qdq + up(sizeof(float) * tokens * d->n_heads);
+  w.dg_part = w.kdk + up(sizeof(float) * tokens * d->n_heads);
+  w.total = w.dg_part + up(sizeof(float) * (size_t)d->n_seqs * d->n_heads);
+  return w;
+}
+
+}  // namespace pal
+
+extern "C" size_t pal_gla_chunk_bwd_workspace_bytes(const PalDims* d) {
+  if (pal_validate_dims(d) != PAL_OK || d->total_chunks <= 0) return 0;
+  return pal::gla_bwd_layout(d).total;
+}
+
+extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const PalBwdTensors* gr, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  using namespace pal;
+  if (int rc = check_gla(d, t)) return rc;
+  if (!gr) return PAL_E_NULL;
+  if (!gr->d_o || !gr->dq || !gr->dk || !gr->dv || !gr->dgt || !gr->dg) return PAL_E_NULL;
+  if (gr->d_init_mu && !(d->flags & PAL_FLAG_HAS_INIT)) return PAL_E_STATE;
+  const void* ptrs[] = {gr->d_o, gr->dq, gr->dk, gr->dv, gr->d_init_mu, workspace};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  const GlaBwdWorkspace w = gla_bwd_layout(d);
+  if (!workspace || workspace_bytes < w.total) return PAL_E_WORKSPACE;
+  char* ws = (char*)workspace;
+  float* g_tiles = (float*)(ws + w.g_tiles);
+  float* qdq = (float*)(ws + w.qdq);
+  float* kdk = (float*)(ws + w.kdk);
+  float* dg_part = (float*)(ws + w.dg_part);
+  hipStream_t s = (hipStream_t)stream;
+
+  ChunkArgs a;
+  fill_gla_args(a, d, t);
+  a.final_mu = nullptr;
+  // D_c = sum_t F_t dO_t q_t^T per tile, then the reverse scan over the tiles of each sequence
+  {
+    ChunkArgs b = a;
+    b.k = t->q; b.v = gr->d_o; b.chunk_mu = g_tiles; b.flags |= kFlagDecayFromStart;
+    if (int rc = launch_tile_delta(b, d->dtype, false, s)) return rc;
+    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk) / 256);
+    if (blocks > 0x7fffffff) return PAL_E_DIM;
+    PAL_TIMED_LAUNCH(kKernGlaBwdScan, s, gla_bwd_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, g_tiles,
+                     gr->d_init_mu);
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  GlaTileArgs A{};
+  A.c = a;
+  // dq: X = dO, Y = v, Z = k, tile-start states read transposed; q . dq on the side
+  A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = t->chunk_mu; A.out = gr->dq; A.W = t->q; A.dot = qdq;
+  A.dc = d->dv; A.de = d->dk;
+  if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDq, s)) return rc;
+  // dv: X = k, Y = q, Z = dO, tile-end state gradients
+  A.X = t->k; A.Y = t->q; A.Z = gr->d_o; A.St = g_tiles; A.out = gr->dv; A.W = nullptr; A.dot = nullptr;
+  A.dc = d->dk; A.de = d->dv;
+  if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDv, s)) return rc;
+  // dk: X = v, Y = dO, Z = q, tile-end state gradients read transposed; k . dk on the side
+  A.X = t->v; A.Y = gr->d_o; A.Z = t->q; A.St = g_tiles; A.out = gr->dk; A.W = t->k; A.dot = kdk;
+  A.dc = d->dv; A.de = d->dk;
+  if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDk, s)) return rc;
+  {
+    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads;
+    PAL_TIMED_LAUNCH(kKernGlaBwdGate, s, gla_bwd_gate_kernel, dim3((unsigned)blocks), dim3(64), 0, s, a, qdq, kdk, gr->dgt,
+                     dg_part);
+    PAL_HIP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gla_bwd_head_reduce_kernel, dim3((d->n_heads + 63) / 64), dim3(64), 0, s, dg_part, gr->dg,
+                       d->n_seqs, d->n_heads);
+    PAL_HIP_LAUNCH_CHECK();
+  }
+  return PAL_OK;
+}
+
+extern "C" int pal_gla_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
+  using namespace pal;
+  if (int rc = check_gla(d, t)) return rc;
+  ChunkArgs a;
+  fill_gla_args(a, d, t);
+  hipStream_t s = (hipStream_t)stream;
+  if (int rc = launch_tile_states(a, d->dtype, false, s)) return rc;
+  GlaTileArgs A{};
+  A.c = a;
+  A.X = t->q; A.Y = t->k; A.Z = t->v; A.St = t->chunk_mu; A.out = t->o;
+  A.dc = d->dk; A.de = d->dv;
+  return launch_gla_tile_dt(A, d->dtype, kGlaOut, s);
+}

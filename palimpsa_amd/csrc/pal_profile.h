@@ -17,6 +17,11 @@ enum KernelId {
   kKernRecurrentBwdFwdPass,
   kKernRecurrentBwd,
   kKernGlaOut,
+  kKernGlaDq,
+  kKernGlaDv,
+  kKernGlaDk,
+  kKernGlaBwdScan,
+  kKernGlaBwdGate,
   kKernCount
 };
 

@@ -21,6 +21,7 @@ still runs (on zeros) and the call costs what the Palimpsa operator costs.
 """
 from __future__ import annotations
 
+import ctypes as C
 from typing import Optional
 
 import torch
@@ -55,65 +56,115 @@ def _run(op, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, *
     return out, None
 
 
-def _chunk_forward_only(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens):
-    """Forward without the precision state through ``pal_gla_chunk_fwd``; nothing is kept for a backward."""
+class ChunkSimpleGLA(torch.autograd.Function):
+    """forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens) -> (o, final_state | None)
+    on ``pal_gla_chunk_fwd`` / ``pal_gla_chunk_bwd``.  The state is ``[N, H, dk, dv]`` at this boundary and
+    ``[N, H, dv, dk]`` inside.  Gradients reaching the final state are not propagated (as in ChunkPalimpsa)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens):
+        H = q.shape[2]
+        dev = q.device
+        # f_t = exp(-gt_t * rate): the kernels take g itself as gt with a rate of -1
+        rate = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
+        S0 = None
+        if initial_state is not None:
+            S0 = initial_state.float().transpose(-1, -2).contiguous()       # [N,H,dk,dv] -> [N,H,dv,dk]
+        p = cm.prepare_inputs(q, k, v, v, g, rate, rate, S0, S0, cu_seqlens, recurrent=False)
+        B, T = p.q.shape[:2]
+        table = offsets = None
+        flags = 0
+        if p.cu_seqlens is not None:
+            meta, total_chunks = _chunk_meta(cu_seqlens)
+            meta = meta.to(dev)
+            offsets, table = meta[: p.n_seqs + 1], meta[p.n_seqs + 1:]
+            flags |= L.PAL_FLAG_VARLEN
+        else:
+            total_chunks = _count_chunks(T, B)
+        if p.init_mu is not None:
+            flags |= L.PAL_FLAG_HAS_INIT
+        o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
+        tile_S = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+        final = None
+        if output_final_state:
+            final = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+        dims = cm.make_dims(p, scale, flags | (L.PAL_FLAG_STORE_FINAL if output_final_state else 0), total_chunks)
+        pt = cm._ptr
+        tens = L.PalFwdTensors(q=pt(p.q), k=pt(p.k), v=pt(p.v), gt=pt(p.gt), g=pt(p.g), o=pt(o), init_mu=pt(p.init_mu),
+                               final_mu=pt(final), cu_seqlens=pt(p.cu_seqlens), chunk_table=pt(table),
+                               chunk_offsets=pt(offsets), chunk_mu=pt(tile_S))
+        with torch.cuda.device(dev):
+            rc = L.load().pal_gla_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
+        L.check(rc, "pal_gla_chunk_fwd")
+        if any(ctx.needs_input_grad):
+            ctx.set_materialize_grads(False)
+            ctx.save_for_backward(p.q, p.k, p.v, p.gt, p.g, p.init_mu, p.cu_seqlens, table, offsets, tile_S)
+            ctx.meta = dict(dk=p.dk, dv=p.dv, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype, scale=float(scale),
+                            flags=flags, total_chunks=total_chunks, in_dtypes=(q.dtype, k.dtype, v.dtype, g.dtype),
+                            init_dtype=None if initial_state is None else initial_state.dtype)
+        o = cm.unpad_last(o, p.dv).to(q.dtype)
+        if final is not None:
+            final = cm.unpad_state(final, p).transpose(-1, -2).contiguous()
+        return o, final
+
+    @staticmethod
+    def backward(ctx, do, d_final=None):
+        q, k, v, gt, rate, init, cu, table, offsets, tile_S = ctx.saved_tensors
+        m = ctx.meta
+        dev = q.device
+        B, T, H, dk_p = q.shape
+        dv_p = v.shape[-1]
+        cd = m["compute_dtype"]
+        if do is None:
+            do = torch.zeros(B, T, H, m["dv"], dtype=cd, device=dev)
+        do = do.to(cd)
+        if dv_p != m["dv"]:
+            do = torch.nn.functional.pad(do, (0, dv_p - m["dv"]))
+        do = do.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dg_tok = torch.empty(B, T, H, dtype=torch.float32, device=dev)
+        d_rate = torch.empty(H, dtype=torch.float32, device=dev)
+        d_init = torch.empty_like(init) if init is not None else None
+        dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p,
+                         total_chunks=m["total_chunks"], dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype),
+                         var_dtype=cm._pal_dtype(cd), flags=m["flags"], scale=m["scale"])
+        pt = cm._ptr
+        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), gt=pt(gt), g=pt(rate), o=pt(do), init_mu=pt(init),
+                               cu_seqlens=pt(cu), chunk_table=pt(table), chunk_offsets=pt(offsets), chunk_mu=pt(tile_S))
+        grads = L.PalBwdTensors(d_o=pt(do), dq=pt(dq), dk=pt(dk), dv=pt(dv), dgt=pt(dg_tok), dg=pt(d_rate),
+                                d_init_mu=pt(d_init))
+        lib = L.load()
+        ws_bytes = int(lib.pal_gla_chunk_bwd_workspace_bytes(dims))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.pal_gla_chunk_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, cm.current_stream_ptr(dev))
+        L.check(rc, "pal_gla_chunk_bwd")
+        dts = m["in_dtypes"]
+        dq = cm.unpad_last(dq, m["dk"]).to(dts[0])
+        dk = cm.unpad_last(dk, m["dk"]).to(dts[1])
+        dv = cm.unpad_last(dv, m["dv"]).to(dts[2])
+        if d_init is not None:
+            d_init = d_init[:, :, :m["dv"], :m["dk"]].transpose(-1, -2).contiguous().to(m["init_dtype"])
+        return dq, dk, dv, dg_tok.to(dts[3]), None, d_init, None, None
+
+
+def _check_chunk_args(q, g, cu_seqlens):
     if g is None:
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
     if g.shape != q.shape[:3]:
         raise ValueError(f"g must have shape {tuple(q.shape[:3])}, got {tuple(g.shape)}")
     if cu_seqlens is not None and q.shape[0] != 1:
         raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
-    if scale is None:
-        scale = q.shape[-1] ** -0.5
-    H = q.shape[2]
-    dev = q.device
-    # f_t = exp(-gt_t * rate): the kernels take g itself as gt with a rate of -1
-    rate = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
-    S0 = None
-    if initial_state is not None:
-        S0 = initial_state.float().transpose(-1, -2).contiguous()       # [N,H,dk,dv] -> [N,H,dv,dk]
-    p = cm.prepare_inputs(q, k, v, v, g, rate, rate, S0, S0, cu_seqlens, recurrent=False)
-    B, T = p.q.shape[:2]
-    table = offsets = None
-    flags = 0
-    if p.cu_seqlens is not None:
-        meta, total_chunks = _chunk_meta(cu_seqlens)
-        meta = meta.to(dev)
-        offsets, table = meta[: p.n_seqs + 1], meta[p.n_seqs + 1:]
-        flags |= L.PAL_FLAG_VARLEN
-    else:
-        total_chunks = _count_chunks(T, B)
-    o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
-    tile_S = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
-    final = None
-    if output_final_state:
-        final = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
-        flags |= L.PAL_FLAG_STORE_FINAL
-    if p.init_mu is not None:
-        flags |= L.PAL_FLAG_HAS_INIT
-    dims = cm.make_dims(p, scale, flags, total_chunks)
-    pt = cm._ptr
-    tens = L.PalFwdTensors(q=pt(p.q), k=pt(p.k), v=pt(p.v), gt=pt(p.gt), g=pt(p.g), o=pt(o), init_mu=pt(p.init_mu),
-                           final_mu=pt(final), cu_seqlens=pt(p.cu_seqlens), chunk_table=pt(table),
-                           chunk_offsets=pt(offsets), chunk_mu=pt(tile_S))
-    with torch.cuda.device(dev):
-        rc = L.load().pal_gla_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
-    L.check(rc, "pal_gla_chunk_fwd")
-    o = cm.unpad_last(o, p.dv).to(q.dtype)
-    if final is not None:
-        final = cm.unpad_state(final, p).transpose(-1, -2).contiguous()
-    return o, final
 
 
 def chunk_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optional[torch.Tensor] = None,
                      scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                      output_final_state: bool = False, cu_seqlens: Optional[torch.Tensor] = None):
     """Chunked (training / prefill) form; returns ``(o, final_state | None)``."""
-    needs_grad = torch.is_grad_enabled() and any(
-        isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, g, initial_state))
-    if not needs_grad:
-        return _chunk_forward_only(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
-    return _run(chunk_palimpsa, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, chunk_size=64)
+    _check_chunk_args(q, g, cu_seqlens)
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    return ChunkSimpleGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
 
 
 def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optional[torch.Tensor] = None,

@@ -102,8 +102,7 @@ def test_packed_documents(gpu_device):
     (2, 150, 2, 64, 32, torch.float32),      # fp32 rows (operands are rounded to bf16 in the kernel)
 ])
 def test_forward_only_kernel_shapes(gpu_device, B, T, H, dk, dv, dtype):
-    """The forward of its own that chunk_simple_gla takes without autograd, against the closed form and against
-    the autograd path (the Palimpsa kernels on b = 0) on the same inputs."""
+    """pal_gla_chunk_fwd against the closed form and against the Palimpsa kernels on b = 0, Ip = 1."""
     from palimpsa_amd.ops.simple_gla import chunk_simple_gla
     q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 21)
     q, k, v = (x.to(dtype) for x in (q, k, v))
@@ -117,12 +116,99 @@ def test_forward_only_kernel_shapes(gpu_device, B, T, H, dk, dv, dtype):
     assert hp.max_rel(S, S_ref) <= 1e-2
     if dk + 2 * dv > 600:
         return          # beyond the LDS budget of the Palimpsa tile-state kernel, which stages k, v and b in fp32
-    qg = q.to(dev).requires_grad_(True)
-    o_g, S_g = chunk_simple_gla(q=qg, k=k.to(dev), v=v.to(dev), g=g.to(dev), scale=0.7,
-                                initial_state=S0.to(dev), output_final_state=True)
-    assert o_g.grad_fn is not None
-    assert hp.max_abs(o.float(), o_g.float()) <= hp.BF16_OUT_ABS_TOL
-    assert hp.max_rel(S, S_g) <= 1e-2
+    # second implementation: the Palimpsa kernels on b = 0, Ip = 1
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    ones = torch.ones(H, device=dev)
+    with torch.no_grad():
+        o_p, mu_p, _ = chunk_palimpsa(q.to(dev), k.to(dev), v.to(dev), torch.zeros_like(v).to(dev), -g.to(dev), ones, ones,
+                                      scale=0.7, initial_mu_state=S0.transpose(-1, -2).contiguous().to(dev),
+                                      initial_I_state=torch.ones(B, H, dv, dk, device=dev), output_final_state=True)
+    assert hp.max_abs(o.float(), o_p.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, mu_p.transpose(-1, -2)) <= 1e-2
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,dtype", [
+    (2, 64, 2, 64, 64, torch.bfloat16),
+    (1, 1, 1, 16, 16, torch.bfloat16),
+    (2, 333, 3, 48, 80, torch.bfloat16),
+    (1, 257, 2, 128, 128, torch.bfloat16),
+    (1, 130, 1, 256, 256, torch.bfloat16),
+    (1, 100, 2, 40, 24, torch.bfloat16),
+    (2, 150, 2, 64, 32, torch.float32),
+])
+def test_backward_shapes_against_closed_form(gpu_device, B, T, H, dk, dv, dtype):
+    """Gradients of q, k, v, g and the initial state from pal_gla_chunk_bwd against autograd through the dense
+    float64 closed form; normalised by the largest reference entry, bar as for the other bf16-input kernels."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 31)
+    q, k, v = (x.to(dtype) for x in (q, k, v))
+    gen = torch.Generator().manual_seed(32)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    dev = gpu_device
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o, _ = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], initial_state=leaves[4], scale=0.5)
+    (o.float() * do.to(dev)).sum().backward()
+    ref_leaves = [x.double().clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o_ref, _ = _closed_form(*ref_leaves[:4], 0.5, ref_leaves[4])
+    (o_ref * do.double()).sum().backward()
+    assert hp.max_abs(o.float(), o_ref.detach()) <= hp.BF16_OUT_ABS_TOL
+    for name, x, r in zip(("q", "k", "v", "g", "S0"), leaves, ref_leaves):
+        assert x.grad.shape == r.grad.shape and x.grad.dtype == x.dtype
+        err = hp.max_rel(x.grad, r.grad)
+        assert err <= hp.BF16_GRAD_NORM_TOL, (name, err)
+
+
+def test_backward_packed_documents(gpu_device):
+    """Every document of a packed batch gets the gradients of a run of its own (gate gradients do not leak
+    across document boundaries)."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    H, dk, dv = 2, 32, 64
+    cu = [0, 70, 71, 200, 264]
+    q, k, v, g, _ = _inputs(1, cu[-1], H, dk, dv, 33)
+    gen = torch.Generator().manual_seed(34)
+    do = torch.randn(1, cu[-1], H, dv, generator=gen)
+    dev = gpu_device
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    o, _ = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], cu_seqlens=torch.tensor(cu, device=dev))
+    (o.float() * do.to(dev)).sum().backward()
+    for j in range(len(cu) - 1):
+        sl = slice(cu[j], cu[j + 1])
+        ref_leaves = [x[:, sl].double().clone().requires_grad_(True) for x in (q, k, v, g)]
+        o_ref, _ = _closed_form(*ref_leaves, dk ** -0.5)
+        (o_ref * do[:, sl].double()).sum().backward()
+        for name, x, r in zip(("q", "k", "v", "g"), leaves, ref_leaves):
+            err = hp.max_rel(x.grad[:, sl], r.grad)
+            assert err <= hp.BF16_GRAD_NORM_TOL, (j, name, err)
+
+
+def test_backward_full_size_against_palimpsa_kernels(gpu_device):
+    """Headline shape: gradients against those of the Palimpsa kernels on b = 0, Ip = 1 (independent code), and
+    the result is bitwise reproducible."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    B, T, H, d = 8, 2048, 12, 64
+    q, k, v, g, _ = _inputs(B, T, H, d, d, 35)
+    gen = torch.Generator().manual_seed(36)
+    do = torch.randn(B, T, H, d, generator=gen).bfloat16()
+    dev = gpu_device
+
+    def run():
+        leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+        o, _ = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3])
+        o.backward(do.to(dev))
+        return o, [x.grad for x in leaves]
+
+    o, grads = run()
+    o2, grads2 = run()
+    assert torch.equal(o, o2) and all(torch.equal(a, b) for a, b in zip(grads, grads2))
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    ones = torch.ones(H, device=dev)
+    o_p = chunk_palimpsa(leaves[0], leaves[1], leaves[2], torch.zeros_like(leaves[2]), -leaves[3], ones, ones)
+    o_p.backward(do.to(dev))
+    assert hp.max_abs(o.float(), o_p.float()) <= hp.BF16_OUT_ABS_TOL
+    for name, x, r in zip(("q", "k", "v", "g"), grads, leaves):
+        err = hp.max_rel(x, r.grad)
+        assert err <= hp.BF16_GRAD_NORM_TOL, (name, err)
 
 
 def test_forward_only_strong_and_weak_decay(gpu_device):
