@@ -1,7 +1,7 @@
 #!/usr/bin/env python
 """Benchmark of the Palimpsa attention operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla]
 
 Headline workload (the metric's own configuration): chunked forward+backward at
 B=8, T=2048, H=12, dk=dv=64, bf16 rows, fp32 gates/states, 64-token tiles,
@@ -12,6 +12,8 @@ One JSON line is printed; it also carries
                 duration from HIP events recorded around every launch of the timed region
   cpu_baseline  the naive fp32 recurrence (oracle port) timed on this host's cores
   extra.decode  config 3 (B=256, H=16, d=128, 1024 single-token steps) against the HBM peak
+  extra.simple_gla  the operator pair without the precision state (chunk_simple_gla forward+backward) on the
+                headline shape, its tile kernel against the HBM peak
 """
 from __future__ import annotations
 
@@ -160,6 +162,52 @@ def bench_decode(torch, dev, steps):
     }
 
 
+def bench_simple_gla(torch, dev, steps, warmup):
+    """chunk_simple_gla forward+backward (what the layer runs with its precision state switched off) on the
+    headline shape; g = -gt so that the decays are those of the headline workload."""
+    from palimpsa_amd import _lib as L
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+
+    B, T, H, d = 8, 2048, 12, 64
+    inp = make_inputs(torch, B, T, H, d, d, 0, torch.bfloat16)
+    leaves = {n: inp[n].to(dev).requires_grad_(True) for n in ("q", "k", "v")}
+    leaves["g"] = (-inp["gt"]).to(dev).requires_grad_(True)
+    do = torch.randn(B, T, H, d, generator=torch.Generator().manual_seed(1)).to(dev, torch.bfloat16)
+
+    def step():
+        for x in leaves.values():
+            x.grad = None
+        o, _ = chunk_simple_gla(q=leaves["q"], k=leaves["k"], v=leaves["v"], g=leaves["g"])
+        o.backward(do)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    L.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kern = L.profile_read()
+    L.profile_enable(False)
+    ms = elapsed * 1e3 / steps
+    # algorithmic bytes of one launch of the forward tile kernel: q, k, v rows in, tile-start state in, o out, gates
+    tiles = B * (T // CHUNK) * H
+    bytes_out = tiles * (CHUNK * (2 * d + d) * 2 + d * d * 4 + CHUNK * d * 2 + CHUNK * 4)
+    ms_out, n_out = kern.get("gla_out_kernel", (float("nan"), 1))
+    avg_out_ms = ms_out / max(n_out, 1)
+    achieved = bytes_out / (avg_out_ms * 1e-3) / 1e9
+    kernels = {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()}
+    return {"workload": "chunk_simple_gla fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates",
+            "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms, "kernel_ms_per_step": sum(v[0] for v in kern.values()) / steps,
+            "kernels": kernels,
+            "roofline": {"bound": "hbm", "kernel": "gla_out_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "algorithmic_bytes_per_launch": bytes_out, "avg_launch_ms": avg_out_ms}}
+
+
 def cpu_baseline(torch):
     """Naive fp32 recurrence (CPU oracle, a port of the reference's palimpsa_ref) with autograd, on a bounded
     sample of the headline workload: batch rows 0-3 of 8, all heads, all 2048 tokens (about 15 s on 16 cores,
@@ -191,6 +239,7 @@ def main():
     ap.add_argument("--decode-steps", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-simple-gla", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -217,6 +266,8 @@ def main():
     extra = {"kernels": res["kernels"], "ms_per_step_no_events": res["ms_per_step_no_events"]}
     if not args.no_decode:
         extra["decode"] = bench_decode(torch, dev, args.decode_steps)
+    if not args.no_simple_gla:
+        extra["simple_gla"] = bench_simple_gla(torch, dev, args.steps, args.warmup)
     line = {
         "metric": "chunk fwd+bwd tokens/s (H=12,d=64,T=2048) %MFMA peak; decode tokens/s %HBM BW",
         "value": res["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

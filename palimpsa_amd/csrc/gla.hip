@@ -344,35 +344,67 @@ __global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, float* b
 // Gate gradients.  With C_t the running sum of the log decay l_t = -gt_t g over a sequence, q_t enters
 // the output only as q_t e^{C_t} and k_t only as k_t e^{-C_t}, so dC_t = q_t . dq_t - k_t . dk_t (the two
 // dot products come from the dq and dk kernels in fp32) and dl_t is the sum of dC over the tokens from t
-// to the end of the sequence.  One wave per (sequence, head) walks the tiles from the last to the first;
-// dgt_t = -g dl_t, and the wave's share of dg = -sum_t gt_t dl_t goes to dg_part[seq][head].
-__global__ __launch_bounds__(64) void gla_bwd_gate_kernel(ChunkArgs a, const float* qdq, const float* kdk, float* dgt,
-                                                          float* dg_part) {
-  const int lane = threadIdx.x;
+// to the end of the sequence.  One workgroup per (sequence, head) walks the sequence from its end in
+// pieces of 1024 tokens: four consecutive tokens per thread, a suffix scan over the lanes of each wave,
+// the four wave totals through LDS.  dgt_t = -g dl_t, and the workgroup's share of
+// dg = -sum_t gt_t dl_t goes to dg_part[seq][head].
+constexpr int kGateTok = 4;                    // consecutive tokens per thread
+constexpr int kGatePiece = 256 * kGateTok;     // tokens per step of a workgroup
+
+__global__ __launch_bounds__(256) void gla_bwd_gate_kernel(ChunkArgs a, const float* qdq, const float* kdk, float* dgt,
+                                                           float* dg_part) {
+  __shared__ float sTot[2][4];
+  __shared__ float sAcc[4];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int h = blockIdx.x % a.H, n = blockIdx.x / a.H;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const float gh = a.g[h];
   float carry = 0.f, acc = 0.f;
-  for (int base = ((len - 1) / kC) * kC; base >= 0; base -= kC) {
-    const int t = base + lane;
-    const int64_t off = (int64_t)(bos + t) * a.H + h;
-    float x = (t < len) ? qdq[off] - kdk[off] : 0.f;
-    // inclusive suffix sum over the 64 lanes
+  int it = 0;
+  for (int base = ((len - 1) / kGatePiece) * kGatePiece; base >= 0; base -= kGatePiece, ++it) {
+    const int tf = base + kGateTok * tid;
+    float x[kGateTok];
+#pragma unroll
+    for (int j = 0; j < kGateTok; ++j) {
+      const int64_t off = (int64_t)(bos + tf + j) * a.H + h;
+      x[j] = (tf + j < len) ? qdq[off] - kdk[off] : 0.f;
+    }
+    // suffix sums inside the thread, then over the lanes of the wave (exclusive of the thread itself)
+#pragma unroll
+    for (int j = kGateTok - 2; j >= 0; --j) x[j] += x[j + 1];
+    float s = x[0];
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
-      const float y = __shfl_down(x, d);
-      if (lane + d < 64) x += y;
+      const float y = __shfl_down(s, d);
+      if (lane + d < 64) s += y;
     }
-    const float dl = x + carry;
-    carry += __shfl(x, 0);
-    if (t < len) {
-      dgt[off] = -gh * dl;
-      acc = fmaf(load_gate(a.gt, off, a.gate_bf16), dl, acc);
+    const float wave_tot = __shfl(s, 0);
+    const float after = s - x[0];             // tokens of later lanes of this wave
+    if (lane == 0) sTot[it & 1][w] = wave_tot;
+    __syncthreads();
+    float later = carry, piece = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float tu = sTot[it & 1][u];
+      piece += tu;
+      if (u > w) later += tu;
+    }
+    carry += piece;
+#pragma unroll
+    for (int j = 0; j < kGateTok; ++j) {
+      if (tf + j < len) {
+        const int64_t off = (int64_t)(bos + tf + j) * a.H + h;
+        const float dl = x[j] + after + later;
+        dgt[off] = -gh * dl;
+        acc = fmaf(load_gate(a.gt, off, a.gate_bf16), dl, acc);
+      }
     }
   }
   acc = wave_sum(acc);
-  if (lane == 0) dg_part[(int64_t)n * a.H + h] = -acc;
+  if (lane == 0) sAcc[w] = acc;
+  __syncthreads();
+  if (tid == 0) dg_part[(int64_t)n * a.H + h] = -(sAcc[0] + sAcc[1] + sAcc[2] + sAcc[3]);
 }
 
 // dg[h] = sum over the sequences, in a fixed order
@@ -456,7 +488,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDk, s)) return rc;
   {
     const int64_t blocks = (int64_t)d->n_seqs * d->n_heads;
-    PAL_TIMED_LAUNCH(kKernGlaBwdGate, s, gla_bwd_gate_kernel, dim3((unsigned)blocks), dim3(64), 0, s, a, qdq, kdk, gr->dgt,
+    PAL_TIMED_LAUNCH(kKernGlaBwdGate, s, gla_bwd_gate_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, qdq, kdk, gr->dgt,
                      dg_part);
     PAL_HIP_LAUNCH_CHECK();
     hipLaunchKernelGGL(gla_bwd_head_reduce_kernel, dim3((d->n_heads + 63) / 64), dim3(64), 0, s, dg_part, gr->dg,

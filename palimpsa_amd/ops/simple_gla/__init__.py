@@ -1,23 +1,22 @@
-"""Scalar-gated linear attention served by the Palimpsa kernels.
+"""Scalar-gated linear attention: the layer's operator pair without the precision state.
 
 The reference layer falls back to ``fla.ops.simple_gla`` when its precision state is switched off
 (``metaplasticity=False``: palimpsa/layers/palimpsa.py:18, :293-300).  With ``b = 0`` and ``Ip = 1``
 the Palimpsa recurrence has ``I = 1`` everywhere, so ``mu = M`` and
 
-    S_t = exp(g_t) S_{t-1} + k_t^T v_t ,   o_t = scale * q_t S_t
+    S_t = exp(g_t) S_{t-1} + k_t^T v_t ,   o_t = scale * q_t S_t .
 
-is exactly what the kernels compute with ``gt = -g`` and a unit per-head rate.  ``chunk_simple_gla`` and
-``fused_recurrent_simple_gla`` keep the keyword names of the layer's call sites (``q, k, v, g,
-scale, initial_state, output_final_state, cu_seqlens``), the default ``scale = dk ** -0.5`` and the
-``(o, final_state)`` return; the state is ``[N, H, dk, dv]`` fp32 (the transpose of the kernels'
-``[N, H, dv, dk]``).  flash-linear-attention itself is not part of the reference tree, so its own
-conventions beyond these call sites are not pinned; the arithmetic is pinned by the closed form
-``o = scale * ((Q K^T) * L) V`` in the tests.
+``chunk_simple_gla`` and ``fused_recurrent_simple_gla`` keep the keyword names of the layer's call sites
+(``q, k, v, g, scale, initial_state, output_final_state, cu_seqlens``), the default
+``scale = dk ** -0.5`` and the ``(o, final_state)`` return; the state is ``[N, H, dk, dv]`` fp32 (the
+transpose of the kernels' ``[N, H, dv, dk]``).  flash-linear-attention itself is not part of the reference
+tree, so its own conventions beyond these call sites are not pinned; the arithmetic is pinned by the
+closed form ``o = scale * ((Q K^T) * L) V`` in the tests.
 
-``chunk_simple_gla`` without autograd (prefill, evaluation) runs a forward of its own
-(``pal_gla_chunk_fwd``): without the division by ``I`` a tile's output is two plain matrix products, so
-the per-token state never has to exist.  With autograd, and on the token-serial path, the precision branch
-still runs (on zeros) and the call costs what the Palimpsa operator costs.
+``chunk_simple_gla`` runs kernels of its own (``pal_gla_chunk_fwd`` / ``pal_gla_chunk_bwd``): without the
+division by ``I`` a tile's output is two plain matrix products, so the per-token state never has to exist.
+``fused_recurrent_simple_gla`` runs the Palimpsa token-serial kernel with ``b = 0``, ``Ip = 1`` and
+``gt = -g`` under a unit per-head rate (the precision branch then works on zeros).
 """
 from __future__ import annotations
 
