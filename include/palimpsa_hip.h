@@ -183,6 +183,80 @@ size_t pal_chunk_bwd_workspace_bytes(const PalDims *dims);
 int pal_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------ layer glue around the op */
+
+/* The element-wise work the reference layer does either side of the operator
+ * (palimpsa/layers/palimpsa.py:266-279 before, :337-343 after), each as one
+ * kernel forward and one backward instead of a dozen framework kernels.
+ * Rows are token-major; tokens = B*T (or the packed total). */
+typedef struct PalGlueDims {
+  int32_t tokens;
+  int32_t n_heads;      /* H: heads of v/b/o (num_v_heads)                     */
+  int32_t n_qk_heads;   /* heads of q_raw/k_raw; H is a multiple of it (:266-267) */
+  int32_t dk, dv;       /* head dims, multiples of 8 in [8,256]                */
+  int32_t dtype;        /* PAL_DTYPE_* of every row tensor                     */
+  float eps;            /* prologue: clamp of the L2 norm (F.normalize, 1e-12);
+                           epilogue: eps of the RMS norm                       */
+} PalGlueDims;
+
+typedef struct PalPrologueTensors {
+  const void *q_raw, *k_raw;       /* dtype [tokens,Hqk,dk] (after conv/SiLU)  */
+  const void *x;                   /* dtype [tokens,H,dv]   (after conv/SiLU)  */
+  const void *dt_raw, *bs_raw;     /* dtype [tokens,H]: dt_proj, bs_proj outputs */
+  const void *b_raw;               /* dtype [tokens,H,dv]: b_proj output, or NULL */
+  const float *dt_bias, *b_scale;  /* fp32 [H]                                 */
+  void *q, *k;                     /* dtype [tokens,H,dk]                      */
+  void *v, *b;                     /* dtype [tokens,H,dv]; b NULL iff b_raw NULL */
+  float *gt;                       /* fp32 [tokens,H]                          */
+} PalPrologueTensors;
+
+typedef struct PalPrologueGrads {
+  const void *dq, *dk;             /* dtype [tokens,H,dk]                      */
+  const void *dv, *db;             /* dtype [tokens,H,dv]; db NULL iff b_raw NULL */
+  const float *dgt;                /* fp32 [tokens,H]                          */
+  void *dq_raw, *dk_raw;           /* dtype [tokens,Hqk,dk]                    */
+  void *dx, *db_raw;               /* dtype [tokens,H,dv]                      */
+  void *ddt_raw, *dbs_raw;         /* dtype [tokens,H]                         */
+  float *ddt_bias, *db_scale;      /* fp32 [H]                                 */
+} PalPrologueGrads;
+
+/* Operator inputs from the projections (layers/palimpsa.py:266-279):
+ *   q, k = l2norm(q_raw), l2norm(k_raw), heads repeated H/Hqk times
+ *   bs = sigmoid(bs_raw) rounded to dtype;  v = x * bs
+ *   b = sigmoid(b_raw) * softplus(b_scale) * bs          (when b_raw given)
+ *   gt = softplus(dt_raw + dt_bias)                      (fp32)            */
+int pal_prologue_fwd(const PalGlueDims *dims, const PalPrologueTensors *t, void *stream);
+/* Its backward.  workspace: pal_prologue_bwd_workspace_bytes(dims) bytes of
+ * device memory for the per-head partial sums of ddt_bias / db_scale. */
+size_t pal_prologue_bwd_workspace_bytes(const PalGlueDims *dims);
+int pal_prologue_bwd(const PalGlueDims *dims, const PalPrologueTensors *t, const PalPrologueGrads *gr,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+typedef struct PalEpilogueTensors {
+  const void *o;        /* dtype [tokens,H,dv]: operator output               */
+  const void *x;        /* dtype [tokens,H,dv] or NULL (no residual, :337)    */
+  const float *D;       /* fp32 [H] (with x)                                   */
+  const void *gate;     /* dtype [tokens,H,dv]: g_proj output, or NULL (:340-343) */
+  const float *weight;  /* fp32 [dv]: RMS norm weight                          */
+  void *y;              /* dtype [tokens,H,dv]                                 */
+  float *rstd;          /* fp32 [tokens,H]: 1/rms, kept for the backward       */
+} PalEpilogueTensors;
+
+typedef struct PalEpilogueGrads {
+  const void *dy;       /* dtype [tokens,H,dv]                                 */
+  void *d_o, *dx, *dgate; /* dtype [tokens,H,dv]; dx / dgate NULL iff x / gate NULL */
+  float *dD;            /* fp32 [H] (with x)                                   */
+  float *dweight;       /* fp32 [dv]                                           */
+} PalEpilogueGrads;
+
+/* y = rmsnorm(o + x*D) * weight * gate*sigmoid(gate)   (layers/palimpsa.py:337-343;
+ * the gated norm is fla.modules.FusedRMSNormGated, a dependency outside the
+ * reference tree: RMS norm over dv, then a swish gate). */
+int pal_epilogue_fwd(const PalGlueDims *dims, const PalEpilogueTensors *t, void *stream);
+size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims *dims);
+int pal_epilogue_bwd(const PalGlueDims *dims, const PalEpilogueTensors *t, const PalEpilogueGrads *gr,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------ measurement */
 
 /* Per-kernel timing aid; no counterpart in the reference.  While enabled, every

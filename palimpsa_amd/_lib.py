@@ -44,6 +44,28 @@ class PalBwdTensors(C.Structure):
         "d_o", "d_o_var", "dq", "dk", "dv", "db", "dgt", "dg", "dIp", "d_init_mu", "d_init_I")]
 
 
+class PalGlueDims(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("tokens", "n_heads", "n_qk_heads", "dk", "dv", "dtype")] + [("eps", C.c_float)]
+
+
+class PalPrologueTensors(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "q_raw", "k_raw", "x", "dt_raw", "bs_raw", "b_raw", "dt_bias", "b_scale", "q", "k", "v", "b", "gt")]
+
+
+class PalPrologueGrads(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "dq", "dk", "dv", "db", "dgt", "dq_raw", "dk_raw", "dx", "db_raw", "ddt_raw", "dbs_raw", "ddt_bias", "db_scale")]
+
+
+class PalEpilogueTensors(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("o", "x", "D", "gate", "weight", "y", "rstd")]
+
+
+class PalEpilogueGrads(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("dy", "d_o", "dx", "dgate", "dD", "dweight")]
+
+
 class PalimpsaHipError(RuntimeError):
     def __init__(self, code: int, where: str, text: str):
         super().__init__(f"{where} failed with code {code}: {text}")
@@ -85,6 +107,20 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_size_t
         fn.argtypes = [P(PalDims)]
+    lib.pal_prologue_fwd.restype = C.c_int
+    lib.pal_prologue_fwd.argtypes = [P(PalGlueDims), P(PalPrologueTensors), C.c_void_p]
+    lib.pal_prologue_bwd.restype = C.c_int
+    lib.pal_prologue_bwd.argtypes = [P(PalGlueDims), P(PalPrologueTensors), P(PalPrologueGrads), C.c_void_p, C.c_size_t,
+                                     C.c_void_p]
+    lib.pal_epilogue_fwd.restype = C.c_int
+    lib.pal_epilogue_fwd.argtypes = [P(PalGlueDims), P(PalEpilogueTensors), C.c_void_p]
+    lib.pal_epilogue_bwd.restype = C.c_int
+    lib.pal_epilogue_bwd.argtypes = [P(PalGlueDims), P(PalEpilogueTensors), P(PalEpilogueGrads), C.c_void_p, C.c_size_t,
+                                     C.c_void_p]
+    for name in ("pal_prologue_bwd_workspace_bytes", "pal_epilogue_bwd_workspace_bytes"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_size_t
+        fn.argtypes = [P(PalGlueDims)]
     lib.pal_profile_enable.restype = C.c_int
     lib.pal_profile_enable.argtypes = [C.c_int]
     lib.pal_profile_kernel_count.restype = C.c_int

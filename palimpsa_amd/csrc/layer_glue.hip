@@ -1,0 +1,540 @@
+// Element-wise work of the reference layer either side of the operator, one kernel per direction:
+//   prologue (palimpsa/layers/palimpsa.py:266-279): L2-normalised q, k (heads repeated), v = x * bs,
+//     b = sigmoid(b_raw) * softplus(b_scale) * bs, gt = softplus(dt_raw + dt_bias);
+//   epilogue (:337-343): y = rmsnorm(o + x * D) * weight * swish(gate).
+// All of it is bound by HBM: every row is read once and written once.  A row of d elements is handled
+// by a group of GL lanes (the power of two >= d/8), eight consecutive elements per lane (16-byte
+// accesses for bf16 rows); a workgroup of 256 threads owns one head and a range of tokens, so that the
+// per-head sums of the backward are accumulated in a fixed order (no atomics).
+#include "pal_common.h"
+#include "pal_host.h"
+#include "pal_profile.h"
+
+namespace pal {
+
+constexpr int kGlueIter = 8;   // rows per row slot of a workgroup
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float* x) {
+  load_vec<4>(p, x);
+  load_vec<4>(p + 4, x + 4);
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const float* x) {
+  store_vec<4>(p, x);
+  store_vec<4>(p + 4, x + 4);
+}
+// sum over the GL lanes of a row group (GL a power of two <= 32); every lane of the group gets it
+__device__ __forceinline__ float group_sum(float x, int GL) {
+  for (int m = 1; m < GL; m <<= 1) x += __shfl_xor(x, m);
+  return x;
+}
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+// softplus as torch computes it (threshold 20)
+__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
+template <typename T>
+__device__ __forceinline__ float round_to(float x) { return to_f32(from_f32<T>(x)); }
+
+struct GlueGeom {
+  int GLk, GLv;     // lanes per q/k row and per v row
+  int tok_per_block;
+};
+static GlueGeom glue_geom(const PalGlueDims* d) {
+  auto pow2 = [](int n) { int p = 1; while (p < n) p <<= 1; return p; };
+  GlueGeom g;
+  g.GLk = pow2(d->dk / 8);
+  g.GLv = pow2(d->dv / 8);
+  const int GLmax = g.GLk > g.GLv ? g.GLk : g.GLv;
+  g.tok_per_block = (256 / GLmax) * kGlueIter;
+  return g;
+}
+
+// ------------------------------------------------------------------ prologue
+struct PrologueArgs {
+  PalPrologueTensors t;
+  PalPrologueGrads g;
+  float* part;          // backward: [H][n_token_blocks][2] partial sums (ddt_bias, db_scale)
+  int tokens, H, Hqk, dk, dv, GLk, GLv, tok_per_block;
+  float eps;
+};
+
+// grid (token blocks, heads, 3): z = 0 rows of q, z = 1 rows of k (heads of q_raw / k_raw), z = 2 rows of v, b and gt
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
+  const int tid = threadIdx.x, task = blockIdx.z, h = blockIdx.y;
+  const int tok0 = blockIdx.x * A.tok_per_block;
+  const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
+  if (task < 2) {
+    if (h >= A.Hqk) return;
+    const int GL = A.GLk, d = A.dk, rep = A.H / A.Hqk;
+    const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+    const T* src = (const T*)(task ? A.t.k_raw : A.t.q_raw);
+    T* dst = (T*)(task ? A.t.k : A.t.q);
+    const bool on = 8 * l < d;
+    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+      float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (on) load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, x);
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+      ss = group_sum(ss, GL);
+      const float inv = 1.f / fmaxf(sqrtf(ss), A.eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= inv;
+      if (on)
+        for (int r = 0; r < rep; ++r) store8(dst + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, x);
+    }
+  } else {
+    const int GL = A.GLv, d = A.dv;
+    const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+    const bool on = 8 * l < d;
+    const float sp = A.t.b_raw ? softplusf_(A.t.b_scale[h]) : 0.f;
+    const float bias = A.t.dt_bias[h];
+    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+      const int64_t th = (int64_t)tok * A.H + h;
+      const float bs = round_to<T>(sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th])));
+      if (l == 0) A.t.gt[th] = softplusf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias);
+      if (!on) continue;
+      float x[8];
+      load8((const T*)A.t.x + th * d + 8 * l, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= bs;
+      store8((T*)A.t.v + th * d + 8 * l, x);
+      if (A.t.b_raw) {
+        float br[8];
+        load8((const T*)A.t.b_raw + th * d + 8 * l, br);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) br[e] = sigmoidf_(br[e]) * sp * bs;
+        store8((T*)A.t.b + th * d + 8 * l, br);
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
+  __shared__ float sRed[4][2];
+  const int tid = threadIdx.x, task = blockIdx.z, h = blockIdx.y;
+  const int tok0 = blockIdx.x * A.tok_per_block;
+  const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
+  if (task < 2) {
+    if (h >= A.Hqk) return;
+    // y = x / n, n = max(|x|, eps):  dx = (s - y (y . s)) / n with s the sum of the gradients of the repeated heads
+    // (for |x| < eps the norm is the constant eps and dx = s / eps)
+    const int GL = A.GLk, d = A.dk, rep = A.H / A.Hqk;
+    const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+    const T* src = (const T*)(task ? A.t.k_raw : A.t.q_raw);
+    const T* gsrc = (const T*)(task ? A.g.dk : A.g.dq);
+    T* dst = (T*)(task ? A.g.dk_raw : A.g.dq_raw);
+    const bool on = 8 * l < d;
+    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+      float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (on) {
+        load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, x);
+        for (int r = 0; r < rep; ++r) {
+          float gy[8];
+          load8(gsrc + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, gy);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s[e] += gy[e];
+        }
+      }
+      float ss = 0.f, xs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { ss = fmaf(x[e], x[e], ss); xs = fmaf(x[e], s[e], xs); }
+      ss = group_sum(ss, GL);
+      xs = group_sum(xs, GL);
+      const float nrm = sqrtf(ss);
+      const bool clamped = nrm < A.eps;
+      const float inv = 1.f / fmaxf(nrm, A.eps);
+      const float c = clamped ? 0.f : xs * inv * inv * inv;   // (y . s) / n^2 * ... folded: dx = s/n - x (x.s)/n^3
+      float out[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = s[e] * inv - x[e] * c;
+      if (on) store8(dst + ((int64_t)tok * A.Hqk + h) * d + 8 * l, out);
+    }
+  } else {
+    const int GL = A.GLv, d = A.dv;
+    const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+    const bool on = 8 * l < d;
+    const bool has_b = A.t.b_raw != nullptr;
+    const float sp = has_b ? softplusf_(A.t.b_scale[h]) : 0.f;
+    const float bias = A.t.dt_bias[h];
+    float acc_dt = 0.f, acc_bs = 0.f;   // this thread's share of ddt_bias[h] and of sum db * sigmoid(b_raw) * bs
+    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+      const int64_t th = (int64_t)tok * A.H + h;
+      const float sg = sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th]));
+      const float bs = round_to<T>(sg);
+      float dbs = 0.f, dsp = 0.f;
+      if (on) {
+        float x[8], gv[8];
+        load8((const T*)A.t.x + th * d + 8 * l, x);
+        load8((const T*)A.g.dv + th * d + 8 * l, gv);
+        float dx[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dx[e] = gv[e] * bs; dbs = fmaf(gv[e], x[e], dbs); }
+        store8((T*)A.g.dx + th * d + 8 * l, dx);
+        if (has_b) {
+          float br[8], gb[8], out[8];
+          load8((const T*)A.t.b_raw + th * d + 8 * l, br);
+          load8((const T*)A.g.db + th * d + 8 * l, gb);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float s = sigmoidf_(br[e]);
+            out[e] = gb[e] * sp * bs * s * (1.f - s);
+            dsp = fmaf(gb[e], s, dsp);
+          }
+          store8((T*)A.g.db_raw + th * d + 8 * l, out);
+        }
+      }
+      dbs = group_sum(fmaf(dsp, sp, dbs), GL);   // d/d bs of v = x bs and b = s sp bs
+      if (l == 0) {
+        ((T*)A.g.dbs_raw)[th] = from_f32<T>(dbs * sg * (1.f - sg));
+        const float ddt = A.g.dgt[th] * sigmoidf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias);
+        ((T*)A.g.ddt_raw)[th] = from_f32<T>(ddt);
+        acc_dt += ddt;
+      }
+      acc_bs = fmaf(dsp, bs, acc_bs);
+    }
+    // workgroup totals in a fixed order: lanes, then waves
+    acc_dt = wave_sum(acc_dt);
+    acc_bs = wave_sum(acc_bs);
+    if ((tid & 63) == 0) { sRed[tid >> 6][0] = acc_dt; sRed[tid >> 6][1] = acc_bs; }
+    __syncthreads();
+    if (tid == 0) {
+      float* p = A.part + ((int64_t)h * gridDim.x + blockIdx.x) * 2;
+      p[0] = sRed[0][0] + sRed[1][0] + sRed[2][0] + sRed[3][0];
+      p[1] = sRed[0][1] + sRed[1][1] + sRed[2][1] + sRed[3][1];
+    }
+  }
+}
+
+// ddt_bias[h], db_scale[h] from the per-workgroup partial sums; db_scale picks up softplus'(b_scale) = sigmoid(b_scale)
+__global__ void prologue_bwd_reduce_kernel(PrologueArgs A, int n_blocks) {
+  const int h = blockIdx.x, lane = threadIdx.x;
+  float a = 0.f, b = 0.f;
+  for (int j = lane; j < n_blocks; j += 64) {
+    a += A.part[((int64_t)h * n_blocks + j) * 2];
+    b += A.part[((int64_t)h * n_blocks + j) * 2 + 1];
+  }
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if (lane == 0) {
+    A.g.ddt_bias[h] = a;
+    if (A.g.db_scale) A.g.db_scale[h] = A.t.b_raw ? b * sigmoidf_(A.t.b_scale[h]) : 0.f;
+  }
+}
+
+// ------------------------------------------------------------------ epilogue
+struct EpilogueArgs {
+  PalEpilogueTensors t;
+  PalEpilogueGrads g;
+  float* part_w;        // backward: [H][n_token_blocks][dv] partial sums of dweight
+  float* part_D;        // backward: [H][n_token_blocks]
+  int tokens, H, dv, GL, tok_per_block;
+  float eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void epilogue_fwd_kernel(EpilogueArgs A) {
+  const int tid = threadIdx.x, h = blockIdx.y;
+  const int tok0 = blockIdx.x * A.tok_per_block;
+  const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
+  const int GL = A.GL, d = A.dv;
+  const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+  const bool on = 8 * l < d;
+  const float Dh = A.t.x ? A.t.D[h] : 0.f;
+  float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (on) load8(A.t.weight + 8 * l, w);
+  const float inv_d = 1.f / (float)d;
+  for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+    const int64_t th = (int64_t)tok * A.H + h;
+    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (on) {
+      load8((const T*)A.t.o + th * d + 8 * l, r);
+      if (A.t.x) {
+        float x[8];
+        load8((const T*)A.t.x + th * d + 8 * l, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = fmaf(x[e], Dh, r[e]);
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(r[e], r[e], ss);
+    ss = group_sum(ss, GL);
+    const float rstd = rsqrtf(ss * inv_d + A.eps);
+    if (l == 0) A.t.rstd[th] = rstd;
+    if (!on) continue;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = r[e] * rstd * w[e];
+    if (A.t.gate) {
+      float gt[8];
+      load8((const T*)A.t.gate + th * d + 8 * l, gt);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] *= gt[e] * sigmoidf_(gt[e]);
+    }
+    store8((T*)A.t.y + th * d + 8 * l, y);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void epilogue_bwd_kernel(EpilogueArgs A) {
+  extern __shared__ float sW[];   // [rows][dv padded to 8 GL] dweight shares of the row slots
+  __shared__ float sRed[4];
+  const int tid = threadIdx.x, h = blockIdx.y;
+  const int tok0 = blockIdx.x * A.tok_per_block;
+  const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
+  const int GL = A.GL, d = A.dv;
+  const int slot = tid / GL, l = tid % GL, rows = 256 / GL;
+  const bool on = 8 * l < d;
+  const float Dh = A.t.x ? A.t.D[h] : 0.f;
+  float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (on) load8(A.t.weight + 8 * l, w);
+  const float inv_d = 1.f / (float)d;
+  float dw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float accD = 0.f;
+  for (int tok = tok0 + slot; tok < tok1; tok += rows) {
+    const int64_t th = (int64_t)tok * A.H + h;
+    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float gy[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float sw[8], dsw[8];   // swish(gate) and its derivative
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sw[e] = 1.f; dsw[e] = 0.f; }
+    if (on) {
+      load8((const T*)A.t.o + th * d + 8 * l, r);
+      load8((const T*)A.g.dy + th * d + 8 * l, gy);
+      if (A.t.x) {
+        load8((const T*)A.t.x + th * d + 8 * l, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = fmaf(x[e], Dh, r[e]);
+      }
+      if (A.t.gate) {
+        float gt[8];
+        load8((const T*)A.t.gate + th * d + 8 * l, gt);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float s = sigmoidf_(gt[e]);
+          sw[e] = gt[e] * s;
+          dsw[e] = s * (1.f + gt[e] * (1.f - s));
+        }
+      }
+    }
+    const float rstd = A.t.rstd[th];
+    // n = r rstd;  y = n w sw;  dn = dy w sw;  dr = rstd (dn - n mean(dn n))
+    float n[8], dn[8], dot = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      n[e] = r[e] * rstd;
+      dn[e] = gy[e] * w[e] * sw[e];
+      dot = fmaf(dn[e], n[e], dot);
+      dw[e] = fmaf(gy[e] * n[e], sw[e], dw[e]);
+    }
+    dot = group_sum(dot, GL) * inv_d;
+    if (!on) continue;
+    float dr[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dr[e] = rstd * (dn[e] - n[e] * dot);
+    store8((T*)A.g.d_o + th * d + 8 * l, dr);
+    if (A.t.x) {
+      float dx[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { dx[e] = dr[e] * Dh; accD = fmaf(dr[e], x[e], accD); }
+      store8((T*)A.g.dx + th * d + 8 * l, dx);
+    }
+    if (A.t.gate) {
+      float dg[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dg[e] = gy[e] * n[e] * w[e] * dsw[e];
+      store8((T*)A.g.dgate + th * d + 8 * l, dg);
+    }
+  }
+  // dweight: the row slots' shares are added in slot order
+  const int dpad = 8 * GL;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sW[slot * dpad + 8 * l + e] = dw[e];
+  accD = wave_sum(accD);
+  if ((tid & 63) == 0) sRed[tid >> 6] = accD;
+  __syncthreads();
+  const int64_t blk = (int64_t)h * gridDim.x + blockIdx.x;
+  for (int c = tid; c < d; c += 256) {
+    float s = 0.f;
+    for (int r = 0; r < rows; ++r) s += sW[r * dpad + c];
+    A.part_w[blk * d + c] = s;
+  }
+  if (tid == 0 && A.t.x) A.part_D[blk] = sRed[0] + sRed[1] + sRed[2] + sRed[3];
+}
+
+// dweight[c] = sum over heads and token blocks; dD[h] = sum over token blocks (fixed order)
+__global__ void epilogue_bwd_reduce_kernel(EpilogueArgs A, int n_blocks) {
+  const int lane = threadIdx.x;
+  if ((int)blockIdx.x < A.dv) {
+    const int c = blockIdx.x;
+    float s = 0.f;
+    for (int64_t j = lane; j < (int64_t)A.H * n_blocks; j += 64) s += A.part_w[j * A.dv + c];
+    s = wave_sum(s);
+    if (lane == 0) A.g.dweight[c] = s;
+  } else if (A.t.x) {
+    const int h = blockIdx.x - A.dv;
+    float s = 0.f;
+    for (int j = lane; j < n_blocks; j += 64) s += A.part_D[(int64_t)h * n_blocks + j];
+    s = wave_sum(s);
+    if (lane == 0) A.g.dD[h] = s;
+  }
+}
+
+static int check_glue_dims(const PalGlueDims* d) {
+  if (!d) return PAL_E_NULL;
+  if (d->tokens <= 0 || d->n_heads <= 0 || d->n_qk_heads <= 0 || d->n_heads % d->n_qk_heads != 0) return PAL_E_DIM;
+  if (d->n_heads > 65535) return PAL_E_DIM;
+  if (d->dk < 8 || d->dk > 256 || d->dk % 8 || d->dv < 8 || d->dv > 256 || d->dv % 8) return PAL_E_HEADDIM;
+  if (d->dtype != PAL_DTYPE_BF16 && d->dtype != PAL_DTYPE_F32) return PAL_E_DTYPE;
+  if (!(d->eps >= 0.f)) return PAL_E_DIM;
+  return PAL_OK;
+}
+
+static int check_prologue(const PalGlueDims* d, const PalPrologueTensors* t) {
+  if (int rc = check_glue_dims(d)) return rc;
+  if (!t) return PAL_E_NULL;
+  if (!t->q_raw || !t->k_raw || !t->x || !t->dt_raw || !t->bs_raw || !t->dt_bias || !t->q || !t->k || !t->v || !t->gt)
+    return PAL_E_NULL;
+  if ((t->b_raw != nullptr) != (t->b != nullptr)) return PAL_E_STATE;
+  if (t->b_raw && !t->b_scale) return PAL_E_NULL;
+  const void* ptrs[] = {t->q_raw, t->k_raw, t->x, t->b_raw, t->q, t->k, t->v, t->b};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  return PAL_OK;
+}
+
+static void fill_prologue(PrologueArgs& A, const PalGlueDims* d, const PalPrologueTensors* t) {
+  const GlueGeom g = glue_geom(d);
+  A.t = *t;
+  A.tokens = d->tokens; A.H = d->n_heads; A.Hqk = d->n_qk_heads; A.dk = d->dk; A.dv = d->dv;
+  A.GLk = g.GLk; A.GLv = g.GLv; A.tok_per_block = g.tok_per_block;
+  A.eps = d->eps;
+  A.part = nullptr;
+}
+
+static int check_epilogue(const PalGlueDims* d, const PalEpilogueTensors* t) {
+  if (int rc = check_glue_dims(d)) return rc;
+  if (!t) return PAL_E_NULL;
+  if (!t->o || !t->weight || !t->y || !t->rstd) return PAL_E_NULL;
+  if (t->x && !t->D) return PAL_E_NULL;
+  const void* ptrs[] = {t->o, t->x, t->gate, t->weight, t->y};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  return PAL_OK;
+}
+
+static void fill_epilogue(EpilogueArgs& A, const PalGlueDims* d, const PalEpilogueTensors* t) {
+  const GlueGeom g = glue_geom(d);
+  A.t = *t;
+  A.tokens = d->tokens; A.H = d->n_heads; A.dv = d->dv;
+  A.GL = g.GLv; A.tok_per_block = (256 / g.GLv) * kGlueIter;
+  A.eps = d->eps;
+  A.part_w = nullptr; A.part_D = nullptr;
+}
+
+static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace pal
+
+extern "C" int pal_prologue_fwd(const PalGlueDims* d, const PalPrologueTensors* t, void* stream) {
+  using namespace pal;
+  if (int rc = check_prologue(d, t)) return rc;
+  PrologueArgs A{};
+  fill_prologue(A, d, t);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((d->tokens + A.tok_per_block - 1) / A.tok_per_block, d->n_heads, 3);
+  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernPrologueFwd, s, prologue_fwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
+  else PAL_TIMED_LAUNCH(kKernPrologueFwd, s, prologue_fwd_kernel<float>, grid, dim3(256), 0, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+extern "C" size_t pal_prologue_bwd_workspace_bytes(const PalGlueDims* d) {
+  using namespace pal;
+  if (check_glue_dims(d) != PAL_OK) return 0;
+  const GlueGeom g = glue_geom(d);
+  const size_t nb = (d->tokens + g.tok_per_block - 1) / g.tok_per_block;
+  return up256(sizeof(float) * 2 * nb * d->n_heads);
+}
+
+extern "C" int pal_prologue_bwd(const PalGlueDims* d, const PalPrologueTensors* t, const PalPrologueGrads* gr,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace pal;
+  if (int rc = check_prologue(d, t)) return rc;
+  if (!gr) return PAL_E_NULL;
+  if (!gr->dq || !gr->dk || !gr->dv || !gr->dgt || !gr->dq_raw || !gr->dk_raw || !gr->dx || !gr->ddt_raw ||
+      !gr->dbs_raw || !gr->ddt_bias)
+    return PAL_E_NULL;
+  if (t->b_raw && (!gr->db || !gr->db_raw || !gr->db_scale)) return PAL_E_NULL;
+  const void* ptrs[] = {gr->dq, gr->dk, gr->dv, gr->db, gr->dq_raw, gr->dk_raw, gr->dx, gr->db_raw, workspace};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  if (!workspace || workspace_bytes < pal_prologue_bwd_workspace_bytes(d)) return PAL_E_WORKSPACE;
+  PrologueArgs A{};
+  fill_prologue(A, d, t);
+  A.g = *gr;
+  A.part = (float*)workspace;
+  hipStream_t s = (hipStream_t)stream;
+  const int nb = (d->tokens + A.tok_per_block - 1) / A.tok_per_block;
+  const dim3 grid(nb, d->n_heads, 3);
+  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernPrologueBwd, s, prologue_bwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
+  else PAL_TIMED_LAUNCH(kKernPrologueBwd, s, prologue_bwd_kernel<float>, grid, dim3(256), 0, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(prologue_bwd_reduce_kernel, dim3(d->n_heads), dim3(64), 0, s, A, nb);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+extern "C" int pal_epilogue_fwd(const PalGlueDims* d, const PalEpilogueTensors* t, void* stream) {
+  using namespace pal;
+  if (int rc = check_epilogue(d, t)) return rc;
+  EpilogueArgs A{};
+  fill_epilogue(A, d, t);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((d->tokens + A.tok_per_block - 1) / A.tok_per_block, d->n_heads);
+  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_fwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
+  else PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_fwd_kernel<float>, grid, dim3(256), 0, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+extern "C" size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims* d) {
+  using namespace pal;
+  if (check_glue_dims(d) != PAL_OK) return 0;
+  const GlueGeom g = glue_geom(d);
+  const int tpb = (256 / g.GLv) * kGlueIter;
+  const size_t nb = (d->tokens + tpb - 1) / tpb;
+  return up256(sizeof(float) * nb * d->n_heads * d->dv) + up256(sizeof(float) * nb * d->n_heads);
+}
+
+extern "C" int pal_epilogue_bwd(const PalGlueDims* d, const PalEpilogueTensors* t, const PalEpilogueGrads* gr,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace pal;
+  if (int rc = check_epilogue(d, t)) return rc;
+  if (!gr) return PAL_E_NULL;
+  if (!gr->dy || !gr->d_o || !gr->dweight) return PAL_E_NULL;
+  if (t->x && (!gr->dx || !gr->dD)) return PAL_E_NULL;
+  if (t->gate && !gr->dgate) return PAL_E_NULL;
+  const void* ptrs[] = {gr->dy, gr->d_o, gr->dx, gr->dgate, workspace};
+  for (const void* p : ptrs)
+    if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  if (!workspace || workspace_bytes < pal_epilogue_bwd_workspace_bytes(d)) return PAL_E_WORKSPACE;
+  EpilogueArgs A{};
+  fill_epilogue(A, d, t);
+  A.g = *gr;
+  const int nb = (d->tokens + A.tok_per_block - 1) / A.tok_per_block;
+  A.part_w = (float*)workspace;
+  A.part_D = (float*)((char*)workspace + up256(sizeof(float) * (size_t)nb * d->n_heads * d->dv));
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(nb, d->n_heads);
+  const size_t lds = sizeof(float) * (256 / A.GL) * 8 * A.GL;   // = 8 KB
+  if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernEpilogueBwd, s, epilogue_bwd_kernel<bf16_t>, grid, dim3(256), lds, s, A);
+  else PAL_TIMED_LAUNCH(kKernEpilogueBwd, s, epilogue_bwd_kernel<float>, grid, dim3(256), lds, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(epilogue_bwd_reduce_kernel, dim3(d->dv + d->n_heads), dim3(64), 0, s, A, nb);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}

@@ -22,6 +22,10 @@ enum KernelId {
   kKernGlaDk,
   kKernGlaBwdScan,
   kKernGlaBwdGate,
+  kKernPrologueFwd,
+  kKernPrologueBwd,
+  kKernEpilogueFwd,
+  kKernEpilogueBwd,
   kKernCount
 };
 

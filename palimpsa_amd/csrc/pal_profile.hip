@@ -48,7 +48,8 @@ static const char* kNames[kKernCount] = {
     "recurrent_fwd_kernel", "chunk_delta_kernel", "chunk_scan_kernel", "chunk_out_kernel", "chunk_bwd_local_kernel",
     "chunk_bwd_carry_scan_kernel", "chunk_bwd_carry_apply_kernel", "chunk_bwd_gate_kernel",
     "chunk_bwd_head_reduce_kernel", "recurrent_bwd_state_kernel", "recurrent_bwd_kernel", "gla_out_kernel",
-    "gla_dq_kernel", "gla_dv_kernel", "gla_dk_kernel", "gla_bwd_scan_kernel", "gla_bwd_gate_kernel"};
+    "gla_dq_kernel", "gla_dv_kernel", "gla_dk_kernel", "gla_bwd_scan_kernel", "gla_bwd_gate_kernel",
+    "prologue_fwd_kernel", "prologue_bwd_kernel", "epilogue_fwd_kernel", "epilogue_bwd_kernel"};
 
 }  // namespace pal
 

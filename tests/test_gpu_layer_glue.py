@@ -1,0 +1,162 @@
+"""pal_prologue_* / pal_epilogue_* (the layer's element-wise work either side of the operator) against the
+CPU restatement of the reference lines (oracle/layer_glue_oracle.py), forward and backward.
+
+Bars: fp32 rows max relative error <= 1e-4 (measured against the largest reference entry); bf16 rows <= 2e-2
+absolute on the outputs (all O(1)) and <= 5e-2 on gradients normalised by the largest reference entry.
+"""
+import pytest
+import torch
+
+from oracle import layer_glue_oracle as lo
+from tests import helpers as hp
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(lead, Hqk, H, dk, dv, seed, dtype):
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    a = dict(q_raw=r(*lead, Hqk, dk), k_raw=r(*lead, Hqk, dk), x=r(*lead, H, dv), dt_raw=r(*lead, H) - 2.0,
+             dt_bias=r(H), bs_raw=r(*lead, H), b_raw=r(*lead, H, dv), b_scale=r(H) + 1.0)
+    for n in ("q_raw", "k_raw", "x", "dt_raw", "bs_raw", "b_raw"):
+        a[n] = a[n].to(dtype)
+    return a
+
+
+NAMES = ("q_raw", "k_raw", "x", "dt_raw", "dt_bias", "bs_raw", "b_raw", "b_scale")
+SHAPES = [
+    ((2, 70), 4, 4, 64, 64, torch.bfloat16),
+    ((1, 33), 2, 6, 48, 48, torch.bfloat16),     # repeated q/k heads, 6 lanes of an 8-lane group
+    ((3, 17), 3, 3, 96, 192, torch.bfloat16),
+    ((5,), 1, 2, 8, 256, torch.bfloat16),
+    ((2, 40), 2, 4, 32, 64, torch.float32),
+]
+
+
+@pytest.mark.parametrize("lead,Hqk,H,dk,dv,dtype", SHAPES)
+@pytest.mark.parametrize("with_b", [True, False])
+def test_prologue_forward_backward(gpu_device, lead, Hqk, H, dk, dv, dtype, with_b):
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs
+    a = _inputs(lead, Hqk, H, dk, dv, 0, dtype)
+    if not with_b:
+        a["b_raw"] = a["b_scale"] = None
+    dev = gpu_device
+    leaves = {n: (None if a[n] is None else a[n].to(dev).clone().requires_grad_(True)) for n in NAMES}
+    outs = palimpsa_inputs(**leaves)
+    ref_leaves = {n: (None if a[n] is None else a[n].double().clone().requires_grad_(True)) for n in NAMES}
+    refs = lo.prologue(**ref_leaves, model_dtype=dtype)
+    out_tol, grad_tol = (hp.BF16_OUT_ABS_TOL, hp.BF16_GRAD_NORM_TOL) if dtype == torch.bfloat16 else (1e-4, 1e-4)
+    gen = torch.Generator().manual_seed(1)
+    loss = 0.0
+    loss_ref = 0.0
+    for name, y, r in zip(("q", "k", "v", "b", "gt"), outs, refs):
+        if r is None:
+            assert y is None
+            continue
+        assert y.shape == r.shape, name
+        assert y.dtype == (torch.float32 if name == "gt" else dtype)
+        assert hp.max_abs(y.float(), r) <= out_tol * max(1.0, r.abs().max().item()), name
+        wgt = torch.randn(r.shape, generator=gen).to(y.dtype)
+        loss = loss + (y.float() * wgt.to(dev).float()).sum()
+        loss_ref = loss_ref + (r * wgt.double()).sum()
+    loss.backward()
+    loss_ref.backward()
+    for n in NAMES:
+        if a[n] is None:
+            continue
+        g, r = leaves[n].grad, ref_leaves[n].grad
+        assert g.shape == r.shape and g.dtype == leaves[n].dtype, n
+        err = hp.max_rel(g, r)
+        assert err <= grad_tol, (n, err)
+
+
+def test_prologue_zero_rows_and_reproducibility(gpu_device):
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs
+    a = _inputs((4, 300), 2, 4, 64, 64, 2, torch.bfloat16)
+    a["q_raw"][0, 5] = 0     # a zero row: the norm is clamped, the output row is zero, gradients stay finite
+    dev = gpu_device
+
+    def run():
+        leaves = {n: a[n].to(dev).clone().requires_grad_(True) for n in NAMES}
+        outs = palimpsa_inputs(**leaves)
+        sum((y.float() ** 2).sum() for y in outs).backward()
+        return outs, [leaves[n].grad for n in NAMES]
+
+    o1, g1 = run()
+    o2, g2 = run()
+    assert (o1[0][0, 5] == 0).all()
+    for x in list(o1) + g1:
+        assert torch.isfinite(x.float()).all()
+    for x, y in zip(list(o1) + g1, list(o2) + g2):
+        assert torch.equal(x, y)       # per-head sums are taken in a fixed order
+
+
+@pytest.mark.parametrize("lead,H,dv,dtype", [
+    ((2, 70), 4, 64, torch.bfloat16),
+    ((1, 33), 6, 48, torch.bfloat16),
+    ((3, 17), 3, 192, torch.bfloat16),
+    ((5,), 2, 256, torch.bfloat16),
+    ((2, 40), 4, 64, torch.float32),
+])
+@pytest.mark.parametrize("residual,gated", [(True, True), (False, True), (True, False), (False, False)])
+def test_epilogue_forward_backward(gpu_device, lead, H, dv, dtype, residual, gated):
+    from palimpsa_amd.ops.layer_glue import palimpsa_output_norm
+    gen = torch.Generator().manual_seed(3)
+    o = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+    x = torch.randn(*lead, H, dv, generator=gen).to(dtype) if residual else None
+    D = torch.randn(H, generator=gen) if residual else None
+    gate = torch.randn(*lead, H, dv, generator=gen).to(dtype) if gated else None
+    w = 1.0 + 0.2 * torch.randn(dv, generator=gen)
+    dy = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+    eps = 1e-6
+    dev = gpu_device
+    ts = [o, x, D, gate, w]
+    leaves = [None if t is None else t.to(dev).clone().requires_grad_(True) for t in ts]
+    y = palimpsa_output_norm(leaves[0], leaves[1], leaves[2], leaves[3], leaves[4], eps)
+    y.backward(dy.to(dev))
+    refs = [None if t is None else t.double().clone().requires_grad_(True) for t in ts]
+    y_ref = lo.epilogue(refs[0], refs[1], refs[2], refs[3], refs[4], eps)
+    y_ref.backward(dy.double())
+    out_tol, grad_tol = (hp.BF16_OUT_ABS_TOL, hp.BF16_GRAD_NORM_TOL) if dtype == torch.bfloat16 else (1e-4, 1e-4)
+    assert y.dtype == dtype and y.shape == y_ref.shape
+    assert hp.max_abs(y.float(), y_ref) <= out_tol * max(1.0, y_ref.abs().max().item())
+    for name, t, r in zip(("o", "x", "D", "gate", "weight"), leaves, refs):
+        if t is None:
+            continue
+        assert t.grad.shape == r.grad.shape and t.grad.dtype == t.dtype, name
+        err = hp.max_rel(t.grad, r.grad)
+        assert err <= grad_tol, (name, err)
+
+
+def test_layer_slice_end_to_end(gpu_device):
+    """Projections' outputs -> prologue -> chunk_palimpsa -> epilogue, with autograd through all three, against the
+    same chain built from the oracles (the operator one in float64)."""
+    from oracle import palimpsa_oracle as po
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs, palimpsa_output_norm
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    B, T, H, d = 1, 96, 2, 32
+    a = _inputs((B, T), H, H, d, d, 4, torch.bfloat16)
+    gen = torch.Generator().manual_seed(5)
+    gate = torch.randn(B, T, H, d, generator=gen).bfloat16()
+    w = 1.0 + 0.1 * torch.randn(d, generator=gen)
+    Dp = torch.randn(H, generator=gen)
+    A = torch.rand(H, generator=gen) * 4 + 0.5
+    Ip = torch.ones(H)
+    dy = torch.randn(B, T, H, d, generator=gen).bfloat16()
+    dev = gpu_device
+    leaves = {n: a[n].to(dev).clone().requires_grad_(True) for n in NAMES}
+    q, k, v, b, gt = palimpsa_inputs(**leaves)
+    o = chunk_palimpsa(q, k, v, b, gt, A.to(dev), Ip.to(dev), chunk_size=64)
+    y = palimpsa_output_norm(o, leaves["x"], Dp.to(dev), gate.to(dev), w.to(dev), 1e-6)
+    y.backward(dy.to(dev))
+
+    refl = {n: a[n].double().clone().requires_grad_(True) for n in NAMES}
+    q_r, k_r, v_r, b_r, gt_r = lo.prologue(**refl, model_dtype=torch.bfloat16)
+    o_r, _, _, _ = po.palimpsa_recurrence(q_r, k_r, v_r, b_r, gt_r, A.double(), Ip.double(), scale=d ** -0.5,
+                                          compute_dtype=torch.float64)
+    y_r = lo.epilogue(o_r, refl["x"], Dp, gate, w, 1e-6)
+    y_r.backward(dy.double())
+    assert hp.max_abs(y.float(), y_r) <= 2 * hp.BF16_OUT_ABS_TOL * max(1.0, y_r.abs().max().item())
+    for n in NAMES:
+        err = hp.max_rel(leaves[n].grad, refl[n].grad)
+        assert err <= 2 * hp.BF16_GRAD_NORM_TOL, (n, err)
