@@ -1,7 +1,7 @@
 #!/usr/bin/env python
 """Benchmark of the Palimpsa attention operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla] [--no-layer-slice]
 
 Headline workload (the metric's own configuration): chunked forward+backward at
 B=8, T=2048, H=12, dk=dv=64, bf16 rows, fp32 gates/states, 64-token tiles,
@@ -14,6 +14,8 @@ One JSON line is printed; it also carries
   extra.decode  config 3 (B=256, H=16, d=128, 1024 single-token steps) against the HBM peak
   extra.simple_gla  the operator pair without the precision state (chunk_simple_gla forward+backward) on the
                 headline shape, its tile kernel against the HBM peak
+  extra.layer_slice  fused prologue -> chunk_palimpsa -> fused epilogue, forward+backward, on the headline shape
+                (the layer between its projections and o_proj), the prologue backward against the HBM peak
 """
 from __future__ import annotations
 
@@ -208,6 +210,67 @@ def bench_simple_gla(torch, dev, steps, warmup):
                          "algorithmic_bytes_per_launch": bytes_out, "avg_launch_ms": avg_out_ms}}
 
 
+def bench_layer_slice(torch, dev, steps, warmup):
+    """What the reference layer does between its projections and o_proj (layers/palimpsa.py:263-343): inputs of
+    the operator from the projections' outputs, the operator, residual + gated RMS norm; forward and backward."""
+    from palimpsa_amd import _lib as L
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs, palimpsa_output_norm
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+
+    B, T, H, d = 8, 2048, 12, 64
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    r = lambda *shape: torch.randn(*shape, generator=gen)
+    bf = torch.bfloat16
+    leaves = dict(q_raw=r(B, T, H, d).to(bf), k_raw=r(B, T, H, d).to(bf), x=r(B, T, H, d).to(bf),
+                  dt_raw=(r(B, T, H) - 1.0).to(bf), dt_bias=r(H), bs_raw=r(B, T, H).to(bf),
+                  b_raw=r(B, T, H, d).to(bf), b_scale=torch.ones(H))
+    leaves = {n: v.to(dev).requires_grad_(True) for n, v in leaves.items()}
+    gate = r(B, T, H, d).to(dev, bf).requires_grad_(True)
+    weight = torch.ones(d, device=dev, requires_grad=True)
+    D = torch.ones(H, device=dev, requires_grad=True)
+    A = torch.ones(H, device=dev, requires_grad=True)
+    Ip = torch.ones(H, device=dev)
+    dy = r(B, T, H, d).to(dev, bf)
+    params = list(leaves.values()) + [gate, weight, D, A]
+
+    def step():
+        for x in params:
+            x.grad = None
+        q, k, v, b, gt = palimpsa_inputs(**leaves)
+        o = chunk_palimpsa(q, k, v, b, gt, A, Ip, chunk_size=CHUNK)
+        y = palimpsa_output_norm(o, leaves["x"], D, gate, weight, 1e-6)
+        y.backward(dy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    L.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kern = L.profile_read()
+    L.profile_enable(False)
+    ms = elapsed * 1e3 / steps
+    rows = B * T * H
+    # algorithmic bytes of the prologue backward: q_raw, k_raw, dq, dk, x, dv, b_raw, db in; dq_raw, dk_raw, dx, db_raw
+    # out (bf16 rows), plus the per-(token, head) scalars dt_raw, bs_raw (bf16) and dgt (fp32) in, ddt_raw, dbs_raw out
+    bytes_pb = rows * (12 * d * 2 + 2 * 2 + 4 + 2 * 2)
+    ms_pb, n_pb = kern.get("prologue_bwd_kernel", (float("nan"), 1))
+    avg_pb = ms_pb / max(n_pb, 1)
+    achieved = bytes_pb / (avg_pb * 1e-3) / 1e9
+    glue = ("prologue_fwd_kernel", "prologue_bwd_kernel", "epilogue_fwd_kernel", "epilogue_bwd_kernel")
+    return {"workload": "prologue -> chunk_palimpsa -> epilogue, fwd+bwd, B=8 T=2048 H=12 dk=dv=64 bf16",
+            "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms,
+            "glue_kernel_ms_per_step": sum(kern[k][0] for k in glue if k in kern) / steps,
+            "kernels": {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()},
+            "roofline": {"bound": "hbm", "kernel": "prologue_bwd_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "algorithmic_bytes_per_launch": bytes_pb, "avg_launch_ms": avg_pb}}
+
+
 def cpu_baseline(torch):
     """Naive fp32 recurrence (CPU oracle, a port of the reference's palimpsa_ref) with autograd, on a bounded
     sample of the headline workload: batch rows 0-3 of 8, all heads, all 2048 tokens (about 15 s on 16 cores,
@@ -240,6 +303,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-simple-gla", action="store_true")
+    ap.add_argument("--no-layer-slice", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -268,6 +332,8 @@ def main():
         extra["decode"] = bench_decode(torch, dev, args.decode_steps)
     if not args.no_simple_gla:
         extra["simple_gla"] = bench_simple_gla(torch, dev, args.steps, args.warmup)
+    if not args.no_layer_slice:
+        extra["layer_slice"] = bench_layer_slice(torch, dev, args.steps, args.warmup)
     line = {
         "metric": "chunk fwd+bwd tokens/s (H=12,d=64,T=2048) %MFMA peak; decode tokens/s %HBM BW",
         "value": res["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
