@@ -202,7 +202,33 @@ def bench_simple_gla(torch, dev, steps, warmup):
     avg_out_ms = ms_out / max(n_out, 1)
     achieved = bytes_out / (avg_out_ms * 1e-3) / 1e9
     kernels = {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()}
-    return {"workload": "chunk_simple_gla fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates",
+    # decode on the shape of config 3 (B=256, H=16, d=128): single-token steps, state [N,H,dk,dv] fed back
+    from palimpsa_amd.ops.simple_gla import fused_recurrent_simple_gla
+    Bd, Hd, dd, dsteps = 256, 16, 128, 256
+    gen = torch.Generator(device="cpu").manual_seed(2)
+    rows = [torch.randn(Bd, 1, Hd, dd, generator=gen).to(dev, torch.bfloat16) for _ in range(3)]
+    gd = (-torch.rand(Bd, 1, Hd, generator=gen)).to(dev)
+    S = (torch.randn(Bd, Hd, dd, dd, generator=gen) * 0.1).to(dev)
+    with torch.no_grad():
+        for _ in range(3):
+            _, S = fused_recurrent_simple_gla(q=rows[0], k=rows[1], v=rows[2], g=gd, initial_state=S, output_final_state=True)
+        torch.cuda.synchronize()
+        L.profile_enable(True)
+        t0 = time.perf_counter()
+        for _ in range(dsteps):
+            _, S = fused_recurrent_simple_gla(q=rows[0], k=rows[1], v=rows[2], g=gd, initial_state=S, output_final_state=True)
+        torch.cuda.synchronize()
+        d_elapsed = time.perf_counter() - t0
+        dk_ms, dk_n = L.profile_read().get("gla_recurrent_fwd_kernel", (float("nan"), 1))
+        L.profile_enable(False)
+    bytes_dec = Bd * Hd * (8 * dd * dd + 2 * (2 * dd + dd) + 4 + 2 * dd)     # state in+out fp32, q,k,v bf16, gate, o
+    dec_gbs = bytes_dec / (dk_ms / max(dk_n, 1) * 1e-3) / 1e9
+    decode = {"workload": "fused_recurrent_simple_gla B=256 H=16 dk=dv=128, single-token steps, state fed back",
+              "tokens_per_s": Bd * dsteps / d_elapsed, "ms_per_step": d_elapsed * 1e3 / dsteps,
+              "roofline": {"bound": "hbm", "kernel": "gla_recurrent_fwd_kernel", "achieved": dec_gbs, "peak": PEAK_HBM_GBS,
+                           "unit": "GB/s", "frac": dec_gbs / PEAK_HBM_GBS, "traffic": None,
+                           "algorithmic_bytes_per_launch": bytes_dec, "avg_launch_ms": dk_ms / max(dk_n, 1)}}
+    return {"workload": "chunk_simple_gla fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates", "decode": decode,
             "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms, "kernel_ms_per_step": sum(v[0] for v in kern.values()) / steps,
             "kernels": kernels,
             "roofline": {"bound": "hbm", "kernel": "gla_out_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,

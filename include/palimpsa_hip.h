@@ -164,6 +164,14 @@ int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
  * is rejected with PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk]. */
 int pal_gla_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
+/* Token-serial forward without the precision state (T >= 1; T == 1 is a decode
+ * step).  Replaces fla.ops.simple_gla.fused_recurrent_simple_gla as called at
+ * palimpsa/layers/palimpsa.py:298.  Same tensors as pal_gla_chunk_fwd without
+ * the chunk arguments, except that init_mu / final_mu hold the state as
+ * S [N,H,dk,dv] (the layout of the layer's cache on this path), so a step
+ * streams the state once in and once out; they may be the same buffer. */
+int pal_gla_recurrent_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
+
 /* Backward of pal_gla_chunk_fwd (replaces the backward of fla's chunk_simple_gla
  * for the same call site).  t as in the forward call, with chunk_mu as that call
  * left it, t->o any valid pointer (not read) and PAL_FLAG_STORE_FINAL clear.

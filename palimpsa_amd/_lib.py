@@ -94,7 +94,7 @@ def load() -> C.CDLL:
     lib.pal_validate_dims.argtypes = [P(PalDims)]
     lib.pal_build_chunk_table.restype = C.c_int
     lib.pal_build_chunk_table.argtypes = [P(C.c_int64), C.c_int32, P(C.c_int32), C.c_int32, P(C.c_int32)]
-    for name in ("pal_recurrent_fwd", "pal_chunk_fwd", "pal_gla_chunk_fwd"):
+    for name in ("pal_recurrent_fwd", "pal_chunk_fwd", "pal_gla_chunk_fwd", "pal_gla_recurrent_fwd"):
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [P(PalDims), P(PalFwdTensors), C.c_void_p]

@@ -26,6 +26,7 @@ enum KernelId {
   kKernPrologueBwd,
   kKernEpilogueFwd,
   kKernEpilogueBwd,
+  kKernGlaRecurrentFwd,
   kKernCount
 };
 

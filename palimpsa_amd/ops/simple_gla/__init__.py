@@ -15,8 +15,9 @@ closed form ``o = scale * ((Q K^T) * L) V`` in the tests.
 
 ``chunk_simple_gla`` runs kernels of its own (``pal_gla_chunk_fwd`` / ``pal_gla_chunk_bwd``): without the
 division by ``I`` a tile's output is two plain matrix products, so the per-token state never has to exist.
-``fused_recurrent_simple_gla`` runs the Palimpsa token-serial kernel with ``b = 0``, ``Ip = 1`` and
-``gt = -g`` under a unit per-head rate (the precision branch then works on zeros).
+``fused_recurrent_simple_gla`` without autograd runs ``pal_gla_recurrent_fwd``, which keeps the state in the
+caller's ``[N, H, dk, dv]`` layout; with autograd it runs the Palimpsa token-serial kernels with ``b = 0``,
+``Ip = 1`` and ``gt = -g`` under a unit per-head rate (the precision branch then works on zeros).
 """
 from __future__ import annotations
 
@@ -169,5 +170,40 @@ def chunk_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optio
 def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optional[torch.Tensor] = None,
                                scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                                output_final_state: bool = False, cu_seqlens: Optional[torch.Tensor] = None):
-    """Token-serial (decode) form; returns ``(o, final_state | None)``."""
-    return _run(fused_recurrent_palimpsa, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
+    """Token-serial (decode) form; returns ``(o, final_state | None)``.  Without autograd it runs a kernel that keeps
+    the state in the ``[N, H, dk, dv]`` layout of the caller (one read and one write of the state per call; the
+    result may be written over ``initial_state`` by passing it again as the next call's initial state)."""
+    needs_grad = torch.is_grad_enabled() and any(
+        isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, g, initial_state))
+    if needs_grad:
+        return _run(fused_recurrent_palimpsa, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
+    _check_chunk_args(q, g, cu_seqlens)
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    H = q.shape[2]
+    dev = q.device
+    rate = torch.full((H,), -1.0, dtype=torch.float32, device=dev)    # f_t = exp(-g_t * rate)
+    p = cm.prepare_inputs(q, k, v, v, g, rate, rate, None, None, cu_seqlens, recurrent=False)
+    S0 = None
+    if initial_state is not None:
+        if tuple(initial_state.shape) != (p.n_seqs, H, p.dk, p.dv):
+            raise ValueError(f"initial_state must be {(p.n_seqs, H, p.dk, p.dv)}, got {tuple(initial_state.shape)}")
+        S0 = initial_state.float().contiguous()
+        if p.dk_p != p.dk or p.dv_p != p.dv:
+            S0 = torch.nn.functional.pad(S0, (0, p.dv_p - p.dv, 0, p.dk_p - p.dk))
+    B, T = p.q.shape[:2]
+    o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
+    final = torch.empty(p.n_seqs, H, p.dk_p, p.dv_p, dtype=torch.float32, device=dev) if output_final_state else None
+    flags = (L.PAL_FLAG_VARLEN if p.cu_seqlens is not None else 0) | (L.PAL_FLAG_HAS_INIT if S0 is not None else 0) \
+        | (L.PAL_FLAG_STORE_FINAL if output_final_state else 0)
+    dims = cm.make_dims(p, scale, flags)
+    pt = cm._ptr
+    tens = L.PalFwdTensors(q=pt(p.q), k=pt(p.k), v=pt(p.v), gt=pt(p.gt), g=pt(p.g), o=pt(o), init_mu=pt(S0),
+                           final_mu=pt(final), cu_seqlens=pt(p.cu_seqlens))
+    with torch.cuda.device(dev):
+        rc = L.load().pal_gla_recurrent_fwd(dims, tens, cm.current_stream_ptr(dev))
+    L.check(rc, "pal_gla_recurrent_fwd")
+    o = cm.unpad_last(o, p.dv).to(q.dtype)
+    if final is not None and (p.dk_p != p.dk or p.dv_p != p.dv):
+        final = final[:, :, :p.dk, :p.dv].contiguous()
+    return o, final

@@ -255,3 +255,81 @@ def test_forward_only_rejects_bad_arguments(gpu_device):
         chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), cu_seqlens=torch.tensor([0, 70], device=dev))
     with pytest.raises(ValueError):
         chunk_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g[:, :10].to(dev))
+
+
+@pytest.mark.parametrize("H,dk,dv", [(16, 48, 96), (16, 96, 192), (4, 96, 96)])
+def test_reference_config_shapes(gpu_device, H, dk, dv):
+    """Head shapes of the reference's configurations that run this path (mamba2_170M: state 48, head 96;
+    mamba2_760M and not_palimpsa_760M: 96 / 192), scale = 1 as the Mamba2-style layer passes it: chunked forward
+    and backward, token-serial forward."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    B, T = 1, 200
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 41)
+    gen = torch.Generator().manual_seed(42)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    dev = gpu_device
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o, S = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], initial_state=leaves[4], scale=1.0,
+                            output_final_state=True)
+    (o.float() * do.to(dev)).sum().backward()
+    ref_leaves = [x.double().clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o_ref, S_ref = _closed_form(*ref_leaves[:4], 1.0, ref_leaves[4])
+    (o_ref * do.double()).sum().backward()
+    tol = hp.BF16_OUT_ABS_TOL * max(1.0, o_ref.abs().max().item())
+    assert hp.max_abs(o.float(), o_ref.detach()) <= tol
+    assert hp.max_rel(S, S_ref.detach()) <= 1e-2
+    for name, x, r in zip(("q", "k", "v", "g", "S0"), leaves, ref_leaves):
+        err = hp.max_rel(x.grad, r.grad)
+        assert err <= hp.BF16_GRAD_NORM_TOL, (name, err)
+    with torch.no_grad():
+        o_r, S_r = fused_recurrent_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), scale=1.0,
+                                              initial_state=S0.to(dev), output_final_state=True)
+    assert hp.max_abs(o_r.float(), o_ref.detach()) <= tol
+    assert hp.max_rel(S_r, S_ref.detach()) <= hp.FP32_REL_TOL
+
+
+def test_decode_steps_in_place_and_packed(gpu_device):
+    """Single-token calls with the state fed back equal one multi-token call; packed documents equal separate
+    runs; fp32 rows meet the fp32 bar."""
+    from palimpsa_amd.ops.simple_gla import fused_recurrent_simple_gla
+    B, T, H, dk, dv = 3, 12, 2, 64, 80
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 43)
+    q, k, v = q.float(), k.float(), v.float()
+    dev = gpu_device
+    qd, kd, vd, gd = (x.to(dev) for x in (q, k, v, g))
+    S = S0.to(dev)
+    outs = []
+    with torch.no_grad():
+        for t in range(T):
+            o, S = fused_recurrent_simple_gla(q=qd[:, t:t + 1], k=kd[:, t:t + 1], v=vd[:, t:t + 1], g=gd[:, t:t + 1],
+                                              initial_state=S, output_final_state=True)
+            outs.append(o)
+        o_all, S_all = fused_recurrent_simple_gla(q=qd, k=kd, v=vd, g=gd, initial_state=S0.to(dev), output_final_state=True)
+    o_steps = torch.cat(outs, dim=1)
+    o_ref, S_ref = _closed_form(q, k, v, g, dk ** -0.5, S0)
+    assert hp.max_rel(o_steps, o_ref) <= hp.FP32_REL_TOL and hp.max_rel(o_all, o_ref) <= hp.FP32_REL_TOL
+    assert hp.max_rel(S, S_ref) <= hp.FP32_REL_TOL and hp.max_rel(S_all, S_ref) <= hp.FP32_REL_TOL
+    # packed documents
+    cu = [0, 5, 6, 20, 36]
+    q2, k2, v2, g2, _ = _inputs(1, cu[-1], H, dk, dv, 44)
+    with torch.no_grad():
+        o2, S2 = fused_recurrent_simple_gla(q=q2.to(dev), k=k2.to(dev), v=v2.to(dev), g=g2.to(dev), output_final_state=True,
+                                            cu_seqlens=torch.tensor(cu, device=dev))
+    for j in range(len(cu) - 1):
+        sl = slice(cu[j], cu[j + 1])
+        o_r, S_r = _closed_form(q2[:, sl], k2[:, sl], v2[:, sl], g2[:, sl], dk ** -0.5)
+        assert hp.max_abs(o2[:, sl].float(), o_r) <= hp.BF16_OUT_ABS_TOL
+        assert hp.max_rel(S2[j:j + 1], S_r) <= hp.FP32_REL_TOL
+
+
+def test_recurrent_with_autograd_still_differentiates(gpu_device):
+    from palimpsa_amd.ops.simple_gla import fused_recurrent_simple_gla
+    q, k, v, g, S0 = _inputs(1, 40, 2, 32, 32, 45)
+    dev = gpu_device
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    o, _ = fused_recurrent_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], scale=0.4)
+    o.float().sum().backward()
+    ref_leaves = [x.double().clone().requires_grad_(True) for x in (q, k, v, g)]
+    _closed_form(*ref_leaves, 0.4)[0].sum().backward()
+    for name, x, r in zip(("q", "k", "v", "g"), leaves, ref_leaves):
+        assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
