@@ -186,7 +186,9 @@ int pal_gla_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
 /* Chunked backward.  Replaces ChunkPalimpsa.backward + chunk_palimpsa_bwd_kernel
  * (chunk_palimpsa_forgetting_scalar.py:239-434, :519-620), including the host
  * side .sum(0) reductions of :609-613.  Needs chunk_mu / chunk_I as written by
- * pal_chunk_fwd on the same inputs. */
+ * pal_chunk_fwd on the same inputs.  Head dims: one kernel keeps a dk x dv
+ * carry tile in LDS, so 4 dk (dv + 8) + 256 (max(dk, dv) + 4) + 32 dv + 288 must
+ * not exceed 163840 (up to 128x192, 192x128, 256x64); PAL_E_HEADDIM otherwise. */
 size_t pal_chunk_bwd_workspace_bytes(const PalDims *dims);
 int pal_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
                   void *workspace, size_t workspace_bytes, void *stream);

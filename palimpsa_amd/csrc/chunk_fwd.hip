@@ -27,12 +27,16 @@ namespace pal {
 // MFMA operand is one contiguous run of tokens), then wave w produces the 16x16 blocks of the state
 // whose key columns are [16w, 16w+16) (+64, ...).  The result is parked in the tile's slot of
 // chunk_mu / chunk_I until the scan below replaces it.
-constexpr int kTS = 68;  // row stride (floats) of the transposed staging tiles
+// Row stride (elements) of the transposed staging tiles: fp32 tiles while they fit in LDS, bf16 tiles (half the
+// size; the operands are rounded to bf16 anyway) for the largest head dims.
+template <typename TS>
+struct StageStride { static constexpr int value = sizeof(TS) == 4 ? 68 : 72; };
 
-template <typename TIn>
-__device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_stride, int width, int clen, float* dst,
+template <typename TIn, typename TS>
+__device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_stride, int width, int clen, TS* dst,
                                                  int tid) {
-  // src: [64 tokens][width] rows -> dst[width][kTS] (token index fastest), rows >= clen are zero
+  // src: [64 tokens][width] rows -> dst[width][stride] (token index fastest), rows >= clen are zero
+  constexpr int kTS = StageStride<TS>::value;
   const int groups = width >> 3;
   for (int idx = tid; idx < kC * groups; idx += 256) {
     const int s = idx & (kC - 1), c8 = idx >> 6;
@@ -45,20 +49,32 @@ __device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_str
       for (int e = 0; e < 8; ++e) x[e] = 0.f;
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dst[(8 * c8 + e) * kTS + s] = x[e];
+    for (int e = 0; e < 8; ++e) dst[(8 * c8 + e) * kTS + s] = from_f32<TS>(x[e]);
   }
+}
+
+// eight consecutive staged elements (16-byte aligned) as fp32
+__device__ __forceinline__ void staged8(const float* p, float* out) {
+  *(f32x4*)&out[0] = *(const f32x4*)p;
+  *(f32x4*)&out[4] = *(const f32x4*)(p + 4);
+}
+__device__ __forceinline__ void staged8(const bf16_t* p, float* out) {
+  const bf16x8 x = *(const bf16x8*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (float)x[e];
 }
 
 // HAS_J = false drops the precision branch (b is not read, chunk_I is not written): the scalar-gated linear
 // attention that the layer uses without its precision state.
-template <typename TIn, bool HAS_J>
+template <typename TIn, bool HAS_J, typename TS>
 __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
+  constexpr int kTS = StageStride<TS>::value;
   const int H = a.H, dk = a.dk, dv = a.dv;
   float* sA = smem;                 // [64] decay from token s to the end of the tile
-  float* sKT = sA + kC;             // [dk][kTS]
-  float* sVT = sKT + dk * kTS;      // [dv][kTS]
-  float* sBT = sVT + dv * kTS;      // [dv][kTS]
+  TS* sKT = (TS*)(sA + kC);         // [dk][kTS]
+  TS* sVT = sKT + dk * kTS;         // [dv][kTS]
+  TS* sBT = sVT + dv * kTS;         // [dv][kTS]
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
   const int NB = dk >> 4, ND = dv >> 4;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
@@ -76,17 +92,13 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
   __syncthreads();
   float as[2][8];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    *(f32x4*)&as[ks][0] = *(const f32x4*)&sA[8 * g + 32 * ks];
-    *(f32x4*)&as[ks][4] = *(const f32x4*)&sA[8 * g + 32 * ks + 4];
-  }
+  for (int ks = 0; ks < 2; ++ks) staged8(&sA[8 * g + 32 * ks], as[ks]);
   for (int nb = w; nb < NB; nb += 4) {
     bf16x8 BK[2], BKK[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       float kv[8];
-      *(f32x4*)&kv[0] = *(const f32x4*)&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks];
-      *(f32x4*)&kv[4] = *(const f32x4*)&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks + 4];
+      staged8(&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks], kv);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         BK[ks][j] = (bf16_t)kv[j];
@@ -98,12 +110,8 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         float vv[8], bb[8];
-        *(f32x4*)&vv[0] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
-        *(f32x4*)&vv[4] = *(const f32x4*)&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
-        if (HAS_J) {
-          *(f32x4*)&bb[0] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks];
-          *(f32x4*)&bb[4] = *(const f32x4*)&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks + 4];
-        }
+        staged8(&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks], vv);
+        if (HAS_J) staged8(&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks], bb);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           AM[ks][j] = (bf16_t)(as[ks][j] * vv[j]);
@@ -526,28 +534,29 @@ void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
 namespace pal {
 
 // Local contribution of every tile to the state, into chunk_mu (and chunk_I when has_j).
-int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
-  {
-    const int64_t blocks = (int64_t)a.total_chunks * a.H;
-    if (blocks > 0x7fffffff) return PAL_E_DIM;
-    const size_t lds = sizeof(float) * (kC + (size_t)(a.dk + (has_j ? 2 : 1) * a.dv) * kTS);
-    if (lds > kMaxLds) return PAL_E_HEADDIM;
-    const void* fn;
-    if (dtype == PAL_DTYPE_BF16)
-      fn = has_j ? (const void*)&chunk_delta_kernel<bf16_t, true> : (const void*)&chunk_delta_kernel<bf16_t, false>;
-    else
-      fn = has_j ? (const void*)&chunk_delta_kernel<float, true> : (const void*)&chunk_delta_kernel<float, false>;
-    if (int rc = allow_lds(fn, lds)) return rc;
-    if (dtype == PAL_DTYPE_BF16) {
-      if (has_j) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t, true>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-      else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<bf16_t, false>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-    } else {
-      if (has_j) PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float, true>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-      else PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<float, false>), dim3((unsigned)blocks), dim3(256), lds, s, a);
-    }
-    PAL_HIP_LAUNCH_CHECK();
-  }
+template <typename TIn, bool HAS_J, typename TS>
+static int launch_tile_delta_t(const ChunkArgs& a, hipStream_t s) {
+  const int64_t blocks = (int64_t)a.total_chunks * a.H;
+  if (blocks > 0x7fffffff) return PAL_E_DIM;
+  const size_t lds = sizeof(float) * kC + sizeof(TS) * (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<TS>::value;
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  if (int rc = allow_lds((const void*)&chunk_delta_kernel<TIn, HAS_J, TS>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<TIn, HAS_J, TS>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+  PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
+}
+
+template <typename TIn, bool HAS_J>
+static int launch_tile_delta_j(const ChunkArgs& a, hipStream_t s) {
+  const size_t lds_f32 = sizeof(float) * (kC + (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<float>::value);
+  if (lds_f32 <= kMaxLds) return launch_tile_delta_t<TIn, HAS_J, float>(a, s);
+  return launch_tile_delta_t<TIn, HAS_J, bf16_t>(a, s);
+}
+
+int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
+  if (dtype == PAL_DTYPE_BF16)
+    return has_j ? launch_tile_delta_j<bf16_t, true>(a, s) : launch_tile_delta_j<bf16_t, false>(a, s);
+  return has_j ? launch_tile_delta_j<float, true>(a, s) : launch_tile_delta_j<float, false>(a, s);
 }
 
 // Tile-start states: local contributions, then the serial scan over the tiles of each sequence.

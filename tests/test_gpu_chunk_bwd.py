@@ -207,3 +207,28 @@ def test_forward_and_backward_are_bitwise_reproducible(gpu_device):
     runs = [_run_bwd(inp, gpu_device, do, dovar, cu=cu) for _ in range(2)]
     for n in NAMES:
         assert torch.equal(runs[0][n], runs[1][n]), n
+
+
+@pytest.mark.parametrize("dk,dv,ok", [(128, 192, True), (192, 128, True), (256, 64, True), (192, 192, False), (256, 256, False)])
+def test_head_dim_envelope_of_the_backward(gpu_device, dk, dv, ok):
+    """The carry tile of the backward has to fit in LDS: the largest supported pairs work end to end, larger ones
+    are refused with a ValueError before any kernel runs (the forward has already succeeded)."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    B, T, H = 1, 100, 1
+    inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=6), torch.bfloat16)
+    gen = torch.Generator().manual_seed(7)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    dev = gpu_device
+    leaves = {n: inp[n].to(dev).clone().requires_grad_(True) for n in ("q", "k", "v", "b", "gt", "g", "Ip")}
+    o = chunk_palimpsa(*[leaves[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")], chunk_size=64)
+    loss = (o.float() * do.to(dev)).sum()
+    if not ok:
+        with pytest.raises(ValueError, match="carry tile"):
+            loss.backward()
+        return
+    loss.backward()
+    ref = hp.oracle_grads(inp, do)
+    assert hp.max_abs(o.float(), ref["o"]) <= hp.BF16_OUT_ABS_TOL
+    for n in ("q", "k", "v", "b", "gt", "g", "Ip"):
+        err = hp.max_rel(leaves[n].grad, ref[n])
+        assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)

@@ -159,3 +159,20 @@ def test_windowed_no_grad_forward_equals_single_call(gpu_device, monkeypatch):
     o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0.cpu(), I0=I0.cpu())
     assert hp.max_abs(o_w.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_rel(mu_w, mu_ref) <= STATE_REL_TOL
+
+
+@pytest.mark.parametrize("dk,dv", [(256, 256), (128, 256), (208, 240)])
+def test_largest_head_dims_forward(gpu_device, dk, dv):
+    """Head dims whose fp32 staging tiles exceed the LDS: the tile-state kernel stages them in bf16 instead."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    B, T, H = 1, 130, 2
+    inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=5), torch.bfloat16)
+    dev = gpu_device
+    d = hp.to_device(inp, dev)
+    with torch.no_grad():
+        (o, ov), mu, I = chunk_palimpsa(d["q"], d["k"], d["v"], d["b"], d["gt"], d["g"], d["Ip"], chunk_size=64,
+                                        output_final_state=True, output_uncertainty=True)
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, want_var=True)
+    assert hp.max_abs(o.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_abs(ov.float(), ov_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
