@@ -195,9 +195,9 @@ def bench_simple_gla(torch, dev, steps, warmup):
     kern = L.profile_read()
     L.profile_enable(False)
     ms = elapsed * 1e3 / steps
-    # algorithmic bytes of one launch of the forward tile kernel: q, k, v rows in, tile-start state in, o out, gates
+    # algorithmic bytes of one launch of the forward tile kernel: q, k, v rows in, tile-start state (bf16) in, o out, gates
     tiles = B * (T // CHUNK) * H
-    bytes_out = tiles * (CHUNK * (2 * d + d) * 2 + d * d * 4 + CHUNK * d * 2 + CHUNK * 4)
+    bytes_out = tiles * (CHUNK * (2 * d + d) * 2 + d * d * 2 + CHUNK * d * 2 + CHUNK * 4)
     ms_out, n_out = kern.get("gla_out_kernel", (float("nan"), 1))
     avg_out_ms = ms_out / max(n_out, 1)
     achieved = bytes_out / (avg_out_ms * 1e-3) / 1e9

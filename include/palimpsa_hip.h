@@ -159,9 +159,11 @@ int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
  * layer calls it with metaplasticity off (palimpsa/layers/palimpsa.py:18,
  * :293-300; flash-linear-attention is a dependency of the reference, not part
  * of its tree).  Reads q, k, v, gt, g, [init_mu], cu_seqlens + chunk tables;
- * writes o, [final_mu] and chunk_mu (tile-start states S, [total_chunks,H,dv,dk]
- * fp32).  b, Ip, o_var, init_I, final_I, chunk_I are ignored; PAL_FLAG_HAS_VAR
- * is rejected with PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk]. */
+ * writes o, [final_mu] and, on this path, two buffers of total_chunks*H*dv*dk
+ * entries: chunk_mu is fp32 scratch (free after the call), chunk_I receives the
+ * tile-start states S in bf16 (2 bytes per entry; what the backward needs).
+ * b, Ip, o_var, init_I, final_I are ignored; PAL_FLAG_HAS_VAR is rejected with
+ * PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk] fp32. */
 int pal_gla_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
 /* Token-serial forward without the precision state (T >= 1; T == 1 is a decode
@@ -173,8 +175,9 @@ int pal_gla_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream)
 int pal_gla_recurrent_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
 /* Backward of pal_gla_chunk_fwd (replaces the backward of fla's chunk_simple_gla
- * for the same call site).  t as in the forward call, with chunk_mu as that call
- * left it, t->o any valid pointer (not read) and PAL_FLAG_STORE_FINAL clear.
+ * for the same call site).  t as in the forward call, with chunk_I (bf16 tile
+ * states) as that call left it, chunk_mu unused (may be NULL), t->o any valid
+ * pointer (not read) and PAL_FLAG_STORE_FINAL clear.
  * Reads gr->d_o; writes gr->dq, dk, dv (dtype), gr->dgt (fp32 [B,T,H], gradient
  * of gt), gr->dg (fp32 [H], gradient of the per-head rate g) and, when not NULL,
  * gr->d_init_mu (fp32 [N,H,dv,dk]).  d_o_var, db, dIp, d_init_I are ignored.

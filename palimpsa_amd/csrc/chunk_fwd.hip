@@ -209,9 +209,11 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
   }
 }
 
-// The same scan without the precision state: S_c = F_c S_{c-1} + Delta_c, the slots of chunk_mu end up
-// holding the state at the start of their tile, the last state goes to final_mu.
+// The same scan without the precision state: S_c = F_c S_{c-1} + Delta_c with Delta_c read from chunk_mu (fp32).
+// The state at the start of every tile is written in bf16 (what its readers feed to the matrix cores) to the
+// buffer handed over in the chunk_I slot; the running state stays fp32 and its last value goes to final_mu.
 __global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
+  bf16_t* tile_S = (bf16_t*)a.chunk_I;
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t E = (int64_t)a.dv * a.dk;
@@ -243,14 +245,14 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
       for (int u = 0; u < 8; ++u) dS[u] = a.chunk_mu[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        a.chunk_mu[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e] = S;
+        tile_S[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e] = (bf16_t)S;
         S = fmaf(sF[c + u], S, dS[u]);
       }
     }
     for (; c < cn; ++c) {
       const int64_t off = ((int64_t)(cbase + c0 + c) * a.H + h) * E + e;
       const float dS = a.chunk_mu[off];
-      a.chunk_mu[off] = S;
+      tile_S[off] = (bf16_t)S;
       S = fmaf(sF[c], S, dS);
     }
   }

@@ -38,7 +38,7 @@ struct GlaTileArgs {
   ChunkArgs c;            // T, H, tiles, gate (gt, g), scale
   const void *X, *Y;      // rows [token][H][dc]: X plays the query, Y the key of the scores
   const void* Z;          // rows [token][H][de]: what the scores mix
-  const float* St;        // per-tile states [tile][H][dv][dk]
+  const bf16_t* St;       // per-tile states [tile][H][dv][dk], bf16
   void* out;              // rows [token][H][de]
   const void* W;          // optional rows [token][H][de]: dot[token] = sum_e W out (fp32, before rounding)
   float* dot;             // [token][H] or null
@@ -54,49 +54,82 @@ struct GlaTileArgs {
 //   dq  : X = dO, Y = v,  Z = k,  St = S read transposed (STATE_T)
 //   dv  : X = k,  Y = q,  Z = dO, St = gradient of the tile-end state G [dv][dk],      reverse
 //   dk  : X = v,  Y = dO, Z = q,  St = G read transposed,                              reverse
-// One workgroup of 4 waves per (tile, head); wave w owns the tokens x in [16w, 16w+16).
-//   P^T[y,x]   = sum_c Y[y,c] X[x,c]           A = Y rows (LDS), B = the wave's X rows (registers)
-//   P^T       *= L(x,y), masked                in the accumulator layout (column x per lane, 4 rows y)
-//   out^T[e,x] = w_x sum_c St[e,c] X[x,c]      A = state rows (global fp32 -> bf16)
-//              + sum_y Z^T[e,y] P^T[y,x]       A = Z^T rows (LDS), B = P^T straight from the accumulators:
-// the contraction index of that last product is mapped to tokens as slot (g, j) -> y = 32p + 16(j/4) +
-// 4g + j%4, which is where the accumulators of two neighbouring blocks already sit, and Z^T is read
-// with the same map (two 8-byte LDS reads per operand).
-// KS = ceil(dc / 32) contraction steps of the scores (operands zero padded to 32 KS).
-template <typename TIn, int KS, bool REVERSE, bool STATE_T>
+// One workgroup of 4 waves per (tile, head), two phases.
+//  (1) Scores: wave w owns the tokens x in [16w, 16w+16).
+//        P^T[y,x] = sum_c Y[y,c] X[x,c]        A = Y rows (LDS), B = the wave's X rows (global)
+//        P^T     *= L(x,y), masked             in the accumulator layout (column x per lane, 4 rows y)
+//      The accumulators of two neighbouring y blocks, rounded to bf16, ARE a B operand of the second
+//      product when its contraction index is mapped to tokens as slot (g, j) -> y = 32p + 16(j/4) + 4g + j%4;
+//      they are parked in LDS so that every wave can use the scores of all 64 tokens.
+//  (2) Output: wave w owns the blocks of 16 output columns [w EB, (w+1) EB) for all 64 tokens.
+//        out^T[e,x] = w_x sum_c St[e,c] X[x,c]  A = state rows (global, bf16), loaded once and used
+//                                               for the four token blocks, B = X rows (global, L1)
+//                   + sum_y Z^T[e,y] P^T[y,x]   A = Z^T rows (LDS, read with the token map above)
+//      so every state entry is read by exactly one wave of the workgroup.
+// EB = ceil(de / 64) column blocks per wave.
+template <typename TIn, int EB, bool REVERSE, bool STATE_T>
 __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
   extern __shared__ float smem[];
   const ChunkArgs& a = A.c;
   const int H = a.H, dc = A.dc, de = A.de;
-  constexpr int dcp = 32 * KS + 8;    // row stride (bf16) of the Y tile
+  const int KS = (dc + 31) >> 5;      // contraction steps of the scores and of the state term
+  const int dcp = 32 * KS + 8;        // row stride (bf16) of the Y tile
   float* sC = smem;                   // [64] running log2 decay inside the tile
-  bf16_t* sY = (bf16_t*)(sC + kC);    // [64][dcp]
+  float* sDot = sC + kC;              // [4][64] partial dot products of the waves
+  bf16x8* sP = (bf16x8*)(sDot + 4 * kC);   // [4 token blocks][2][64 lanes] score operands
+  bf16_t* sY = (bf16_t*)(sP + 4 * 2 * 64); // [64][dcp]
   bf16_t* sZT = sY + kC * dcp;        // [de][kVT]
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
-  const int tb = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
   chunk_lookup(a, cidx, seq, t0, clen, cis);
-  if (tb == 0) {
+  if (w == 0) {
     const float gh = a.g[h] * kLog2e;
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     sC[lane] = wave_inclusive_scan(-gt * gh, lane);
   }
-  // the wave's 16 X rows as B operands (column x = 16 tb + i, contraction index c = 32 ks + 8 g + j)
-  const int x = 16 * tb + i;
-  bf16x8 Xr[KS];
-  {
-    const TIn* xp = (const TIn*)A.X + ((int64_t)(t0 + x) * H + h) * dc + 8 * g;
+  const TIn* xbase = (const TIn*)A.X + ((int64_t)t0 * H + h) * dc + 8 * g;
+  // X rows of token block xb as a B operand (column x = 16 xb + i, contraction index c = 32 ks + 8 g + j)
+  auto x_operand = [&](int xb, int ks) {
+    bf16x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int x = 16 * xb + i;
+    if (x < clen && 32 * ks + 8 * g < dc) r = load_bf16x8(xbase + (int64_t)x * H * dc + 32 * ks);
+    return r;
+  };
+  // State operands of this wave: blocks of 16 output columns [w EB, (w+1) EB), rows e = 16 eb + i, contraction
+  // index c = 32 ks + 8 g + j.  The first step is requested before the staging below so that its latency
+  // overlaps the staging's, every further step one step ahead of its use.
+  const bf16_t* St = A.St + ((int64_t)cidx * H + h) * dc * de;
+  const int n_eb = de >> 4;
+  const bf16_t* srow[EB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Xr[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (x < clen && 32 * ks + 8 * g < dc) Xr[ks] = load_bf16x8(xp + 32 * ks);
-    }
+  for (int el = 0; el < EB; ++el) {
+    const int e = 16 * min(w * EB + el, n_eb - 1) + i;   // a block past the end repeats the last one (not stored)
+    srow[el] = STATE_T ? St + (int64_t)(8 * g) * de + e : St + (int64_t)e * dc + 8 * g;
   }
+  bf16x8 raw[EB];
+  auto fetch_state = [&](int ks) {
+    const bool ok = 32 * ks + 8 * g < dc;
+#pragma unroll
+    for (int el = 0; el < EB; ++el) {
+      raw[el] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (ok) {
+        if constexpr (STATE_T) {
+          // the state is stored [c][e]: eight rows apart, neighbouring lanes read neighbouring columns
+#pragma unroll
+          for (int j = 0; j < 8; ++j) raw[el][j] = srow[el][(int64_t)(32 * ks + j) * de];
+        } else {
+          raw[el] = *(const bf16x8*)(srow[el] + 32 * ks);
+        }
+      }
+    }
+  };
+  fetch_state(0);
   {
     // Y rows, zero beyond the tile's tokens and beyond dc
     const TIn* yp = (const TIn*)A.Y + ((int64_t)t0 * H + h) * dc;
-    constexpr int groups = 4 * KS;
+    const int groups = 4 * KS;
     for (int idx = tid; idx < kC * groups; idx += 256) {
       const int s = idx / groups, c8 = idx - s * groups;
       bf16x8 yx = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -119,127 +152,139 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
   }
   __syncthreads();
 
-  const float cx = sC[16 * tb + i];
-  const float wx = fast_exp2(REVERSE ? sC[kC - 1] - cx : cx);
-
-  // decayed, masked scores of the wave's 16 tokens against the blocks on their causal side, as B operands
-  bf16x8 P[2];
+  // ---- phase 1: decayed, masked scores of token block w against the blocks on its causal side
+  {
+    const int tb = w;
+    f32x4 accS[4];
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
+    for (int yb = 0; yb < 4; ++yb) accS[yb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 Xo = x_operand(tb, ks);
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int yb = 2 * p + half;
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      if (REVERSE ? yb >= tb : yb <= tb) {
-        const bf16_t* yrow = sY + (16 * yb + i) * dcp + 8 * g;
+      for (int yb = 0; yb < 4; ++yb)
+        if (REVERSE ? yb >= tb : yb <= tb)
+          accS[yb] = mfma16(*(const bf16x8*)(sY + (16 * yb + i) * dcp + 8 * g + 32 * ks), Xo, accS[yb]);
+    }
+    const float cx = sC[16 * tb + i];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) acc = mfma16(*(const bf16x8*)(yrow + 32 * ks), Xr[ks], acc);
+    for (int p = 0; p < 2; ++p) {
+      bf16x8 P;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int yb = 2 * p + half;
         const f32x4 cy = *(const f32x4*)&sC[16 * yb + 4 * g];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const bool live = yb != tb || (REVERSE ? 4 * g + r >= i : 4 * g + r <= i);
-          acc[r] = live ? acc[r] * fast_exp2(REVERSE ? cy[r] - cx : cx - cy[r]) : 0.f;
+          const bool side = REVERSE ? yb >= tb : yb <= tb;
+          const bool live = side && (yb != tb || (REVERSE ? 4 * g + r >= i : 4 * g + r <= i));
+          const float val = live ? accS[yb][r] * fast_exp2(REVERSE ? cy[r] - cx : cx - cy[r]) : 0.f;
+          P[4 * half + r] = (bf16_t)val;
         }
       }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) P[p][4 * half + r] = (bf16_t)acc[r];
+      sP[(tb * 2 + p) * 64 + lane] = P;
     }
   }
+  __syncthreads();
 
+  // ---- phase 2: output columns of this wave for all four token blocks
   const float scale = a.scale;
-  const float* St = A.St + ((int64_t)cidx * H + h) * dc * de;
-  TIn* orow = (TIn*)A.out + ((int64_t)(t0 + x) * H + h) * de + 4 * g;
-  const TIn* wrow = (const TIn*)A.W + ((int64_t)(t0 + x) * H + h) * de + 4 * g;
+  float wx[4];
+#pragma unroll
+  for (int xb = 0; xb < 4; ++xb) {
+    const float cx = sC[16 * xb + i];
+    wx[xb] = fast_exp2(REVERSE ? sC[kC - 1] - cx : cx);
+  }
+  f32x4 acc[EB][4];
+#pragma unroll
+  for (int el = 0; el < EB; ++el)
+#pragma unroll
+    for (int xb = 0; xb < 4; ++xb) acc[el][xb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int ks = 0; ks < KS; ++ks) {
+    bf16x8 Sa[EB];
+#pragma unroll
+    for (int el = 0; el < EB; ++el) Sa[el] = raw[el];
+    if (ks + 1 < KS) fetch_state(ks + 1);     // in flight while this step's products run
+    bf16x8 Xo[4];
+#pragma unroll
+    for (int xb = 0; xb < 4; ++xb) Xo[xb] = x_operand(xb, ks);
+#pragma unroll
+    for (int el = 0; el < EB; ++el)
+#pragma unroll
+      for (int xb = 0; xb < 4; ++xb) acc[el][xb] = mfma16(Sa[el], Xo[xb], acc[el][xb]);
+  }
+  bf16x8 P[4][2];
+#pragma unroll
+  for (int xb = 0; xb < 4; ++xb)
+#pragma unroll
+    for (int p = 0; p < 2; ++p) P[xb][p] = sP[(xb * 2 + p) * 64 + lane];
+  float dot[4] = {0.f, 0.f, 0.f, 0.f};
   const bool has_dot = A.dot != nullptr;
-  float dot = 0.f;
-  const int n_eb = de >> 4;
-  // four blocks of 16 output columns at a time, so that the loads of the state are in flight together
-  for (int eb0 = 0; eb0 < n_eb; eb0 += 4) {
-    f32x4 acc[4];
-    const float* srow[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int e = 16 * min(eb0 + u, n_eb - 1) + i;   // a block past the end repeats the last one
-      srow[u] = STATE_T ? St + (int64_t)(8 * g) * de + e : St + (int64_t)e * dc + 8 * g;
+  for (int el = 0; el < EB; ++el) {
+    const int eb = min(w * EB + el, n_eb - 1);
+    const bool valid = w * EB + el < n_eb;
+    const bf16_t* zrow = sZT + (16 * eb + i) * kVT + 4 * g;
+    bf16x8 Za[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const bf16x4 lo = *(const bf16x4*)(zrow + 32 * p), hi = *(const bf16x4*)(zrow + 32 * p + 16);
+      Za[p] = bf16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      bf16x8 Sa[4];
-      const bool ok = 32 * ks + 8 * g < dc;
+    for (int xb = 0; xb < 4; ++xb) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        Sa[u] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (ok) {
-          if constexpr (STATE_T) {
-            // the state is stored [c][e]: eight rows apart, neighbouring lanes read neighbouring columns
+      for (int r = 0; r < 4; ++r) acc[el][xb][r] *= wx[xb];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) Sa[u][j] = (bf16_t)srow[u][(int64_t)(32 * ks + j) * de];
-          } else {
-            Sa[u] = load_bf16x8(srow[u] + 32 * ks);
-          }
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) acc[u] = mfma16(Sa[u], Xr[ks], acc[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int eb = min(eb0 + u, n_eb - 1);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[u][r] *= wx;
-      const bf16_t* zrow = sZT + (16 * eb + i) * kVT + 4 * g;
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        if (REVERSE ? 2 * p + 1 >= tb : 2 * p <= tb) {
-          const bf16x4 lo = *(const bf16x4*)(zrow + 32 * p), hi = *(const bf16x4*)(zrow + 32 * p + 16);
-          const bf16x8 Za = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          acc[u] = mfma16(Za, P[p], acc[u]);
-        }
-      }
-      if (x < clen && eb0 + u < n_eb) {
-        const float res[4] = {acc[u][0] * scale, acc[u][1] * scale, acc[u][2] * scale, acc[u][3] * scale};
-        store_vec<4>(orow + 16 * eb, res);
+      for (int p = 0; p < 2; ++p)
+        if ((REVERSE ? 2 * p + 1 >= xb : 2 * p <= xb)) acc[el][xb] = mfma16(Za[p], P[xb][p], acc[el][xb]);
+      const int x = 16 * xb + i;
+      if (valid && x < clen) {
+        const float res[4] = {acc[el][xb][0] * scale, acc[el][xb][1] * scale, acc[el][xb][2] * scale,
+                              acc[el][xb][3] * scale};
+        const int64_t off = ((int64_t)(t0 + x) * H + h) * de + 16 * eb + 4 * g;
+        store_vec<4>((TIn*)A.out + off, res);
         if (has_dot) {
           float wv[4];
-          load_vec<4>(wrow + 16 * eb, wv);
+          load_vec<4>((const TIn*)A.W + off, wv);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) dot = fmaf(wv[r], res[r], dot);
+          for (int r = 0; r < 4; ++r) dot[xb] = fmaf(wv[r], res[r], dot[xb]);
         }
       }
     }
   }
   if (has_dot) {
-    dot = rows4_sum(dot);
-    if (g == 0 && x < clen) A.dot[(int64_t)(t0 + x) * H + h] = dot;
+    // rows g of a wave hold different output columns of the same token: sum them, then the four waves
+    const float tot = rows4_sum_x4(dot[0], dot[1], dot[2], dot[3]);   // lanes of row g: token block g
+    sDot[w * kC + lane] = tot;                                        // lane = 16 g + i = token
+    __syncthreads();
+    if (w == 0 && lane < clen)
+      A.dot[(int64_t)(t0 + lane) * H + h] = (sDot[lane] + sDot[kC + lane]) + (sDot[2 * kC + lane] + sDot[3 * kC + lane]);
   }
 }
 
 enum GlaRole { kGlaOut = 0, kGlaDq, kGlaDv, kGlaDk };
 
-template <typename TIn, int KS, bool REVERSE, bool STATE_T>
-static int launch_gla_tile_ks(const GlaTileArgs& A, int kern_id, hipStream_t s) {
-  const size_t lds = sizeof(float) * kC + sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+template <typename TIn, int EB, bool REVERSE, bool STATE_T>
+static int launch_gla_tile_eb(const GlaTileArgs& A, int kern_id, hipStream_t s) {
+  const int KS = (A.dc + 31) / 32;
+  const size_t lds = sizeof(float) * (kC + 4 * kC) + 16 * 4 * 2 * 64 +
+                     sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;
-  if (int rc = allow_lds((const void*)&gla_tile_kernel<TIn, KS, REVERSE, STATE_T>, lds)) return rc;
-  PAL_TIMED_LAUNCH(kern_id, s, (gla_tile_kernel<TIn, KS, REVERSE, STATE_T>), dim3((unsigned)blocks), dim3(256), lds, s, A);
+  if (int rc = allow_lds((const void*)&gla_tile_kernel<TIn, EB, REVERSE, STATE_T>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kern_id, s, (gla_tile_kernel<TIn, EB, REVERSE, STATE_T>), dim3((unsigned)blocks), dim3(256), lds, s, A);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
 
 template <typename TIn, bool REVERSE, bool STATE_T>
 static int launch_gla_tile_rs(const GlaTileArgs& A, int kern_id, hipStream_t s) {
-  switch ((A.dc + 31) / 32) {
-    case 1: return launch_gla_tile_ks<TIn, 1, REVERSE, STATE_T>(A, kern_id, s);
-    case 2: return launch_gla_tile_ks<TIn, 2, REVERSE, STATE_T>(A, kern_id, s);
-    case 3: return launch_gla_tile_ks<TIn, 3, REVERSE, STATE_T>(A, kern_id, s);
-    case 4: return launch_gla_tile_ks<TIn, 4, REVERSE, STATE_T>(A, kern_id, s);
-    case 5: return launch_gla_tile_ks<TIn, 5, REVERSE, STATE_T>(A, kern_id, s);
-    case 6: return launch_gla_tile_ks<TIn, 6, REVERSE, STATE_T>(A, kern_id, s);
-    case 7: return launch_gla_tile_ks<TIn, 7, REVERSE, STATE_T>(A, kern_id, s);
-    case 8: return launch_gla_tile_ks<TIn, 8, REVERSE, STATE_T>(A, kern_id, s);
+  switch ((A.de + 63) / 64) {
+    case 1: return launch_gla_tile_eb<TIn, 1, REVERSE, STATE_T>(A, kern_id, s);
+    case 2: return launch_gla_tile_eb<TIn, 2, REVERSE, STATE_T>(A, kern_id, s);
+    case 3: return launch_gla_tile_eb<TIn, 3, REVERSE, STATE_T>(A, kern_id, s);
+    case 4: return launch_gla_tile_eb<TIn, 4, REVERSE, STATE_T>(A, kern_id, s);
     default: return PAL_E_HEADDIM;
   }
 }
@@ -263,7 +308,7 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   int rc = pal_validate_dims(d);
   if (rc) return rc;
   if (!t) return PAL_E_NULL;
-  if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o || !t->chunk_mu) return PAL_E_NULL;
+  if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o || !t->chunk_I) return PAL_E_NULL;
   if (d->flags & PAL_FLAG_HAS_VAR) return PAL_E_STATE;   // no precision state, no output variance
   if (((d->flags & PAL_FLAG_HAS_INIT) != 0) != (t->init_mu != nullptr)) return PAL_E_STATE;
   if (((d->flags & PAL_FLAG_STORE_FINAL) != 0) != (t->final_mu != nullptr)) return PAL_E_STATE;
@@ -277,7 +322,7 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   } else if ((int64_t)d->total_chunks != per * d->batch) {
     return PAL_E_CHUNK;
   }
-  const void* ptrs[] = {t->q, t->k, t->v, t->o, t->init_mu, t->final_mu, t->chunk_mu};
+  const void* ptrs[] = {t->q, t->k, t->v, t->o, t->init_mu, t->final_mu, t->chunk_mu, t->chunk_I};
   for (const void* p : ptrs)
     if (p && !is_aligned16(p)) return PAL_E_ALIGN;
   return PAL_OK;
@@ -287,16 +332,16 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
 static void fill_gla_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
   PalFwdTensors tt = *t;
   tt.b = nullptr; tt.Ip = nullptr; tt.o_var = nullptr;
-  tt.init_I = nullptr; tt.final_I = nullptr; tt.chunk_I = nullptr;
+  tt.init_I = nullptr; tt.final_I = nullptr;
   fill_chunk_args(a, d, &tt);
 }
 
 // ------------------------------------------------------------------ backward
 // Gradient of the state at the END of every tile, G_c = F_{c+1} G_{c+1} + D_{c+1}, from the tiles' own
 // contributions D_c = sum_t F_t dO_t q_t^T parked in buf by chunk_delta_kernel: the forward scan run
-// backwards.  One thread per (sequence, head, state entry); slot c of buf ends up holding G_c.  What is
-// left after the first tile, times scale, is the gradient of the initial state.
-__global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, float* buf, float* d_init) {
+// backwards.  One thread per (sequence, head, state entry); slot c of g_tiles gets G_c in bf16 (the running
+// value stays fp32).  What is left after the first tile, times scale, is the gradient of the initial state.
+__global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, const float* buf, bf16_t* g_tiles, float* d_init) {
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t E = (int64_t)a.dv * a.dk;
@@ -327,14 +372,14 @@ __global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, float* b
       for (int u = 0; u < 8; ++u) D[u] = buf[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        buf[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e] = G;
+        g_tiles[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e] = (bf16_t)G;
         G = fmaf(sF[c - 1 - u], G, D[u]);
       }
     }
     for (; c >= 1; --c) {
       const int64_t off = ((int64_t)(cbase + c0 + c - 1) * a.H + h) * E + e;
       const float D = buf[off];
-      buf[off] = G;
+      g_tiles[off] = (bf16_t)G;
       G = fmaf(sF[c - 1], G, D);
     }
   }
@@ -416,16 +461,19 @@ __global__ void gla_bwd_head_reduce_kernel(const float* dg_part, float* dg, int 
   dg[h] = s;
 }
 
-// workspace of the backward: G tiles, the two dot-product rows, per-sequence shares of dg
+// workspace of the backward: per-tile contributions D (fp32), G tiles (bf16), the two dot-product rows,
+// per-sequence shares of dg
 struct GlaBwdWorkspace {
-  size_t g_tiles, qdq, kdk, dg_part, total;
+  size_t d_tiles, g_tiles, qdq, kdk, dg_part, total;
 };
 static GlaBwdWorkspace gla_bwd_layout(const PalDims* d) {
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   GlaBwdWorkspace w;
   const size_t tokens = (size_t)d->batch * d->seq_len;
-  w.g_tiles = 0;
-  w.qdq = w.g_tiles + up(sizeof(float) * (size_t)d->total_chunks * d->n_heads * d->dv * d->dk);
+  const size_t entries = (size_t)d->total_chunks * d->n_heads * d->dv * d->dk;
+  w.d_tiles = 0;
+  w.g_tiles = w.d_tiles + up(sizeof(float) * entries);
+  w.qdq = w.g_tiles + up(sizeof(bf16_t) * entries);
   w.kdk = w.qdq + up(sizeof(float) * tokens * d->n_heads);
   w.dg_part = w.kdk + up(sizeof(float) * tokens * d->n_heads);
   w.total = w.dg_part + up(sizeof(float) * (size_t)d->n_seqs * d->n_heads);
@@ -452,7 +500,8 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   const GlaBwdWorkspace w = gla_bwd_layout(d);
   if (!workspace || workspace_bytes < w.total) return PAL_E_WORKSPACE;
   char* ws = (char*)workspace;
-  float* g_tiles = (float*)(ws + w.g_tiles);
+  float* d_tiles = (float*)(ws + w.d_tiles);
+  bf16_t* g_tiles = (bf16_t*)(ws + w.g_tiles);
   float* qdq = (float*)(ws + w.qdq);
   float* kdk = (float*)(ws + w.kdk);
   float* dg_part = (float*)(ws + w.dg_part);
@@ -464,18 +513,18 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   // D_c = sum_t F_t dO_t q_t^T per tile, then the reverse scan over the tiles of each sequence
   {
     ChunkArgs b = a;
-    b.k = t->q; b.v = gr->d_o; b.chunk_mu = g_tiles; b.flags |= kFlagDecayFromStart;
+    b.k = t->q; b.v = gr->d_o; b.chunk_mu = d_tiles; b.flags |= kFlagDecayFromStart;
     if (int rc = launch_tile_delta(b, d->dtype, false, s)) return rc;
     const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk) / 256);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
-    PAL_TIMED_LAUNCH(kKernGlaBwdScan, s, gla_bwd_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, g_tiles,
-                     gr->d_init_mu);
+    PAL_TIMED_LAUNCH(kKernGlaBwdScan, s, gla_bwd_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, d_tiles,
+                     g_tiles, gr->d_init_mu);
     PAL_HIP_LAUNCH_CHECK();
   }
   GlaTileArgs A{};
   A.c = a;
   // dq: X = dO, Y = v, Z = k, tile-start states read transposed; q . dq on the side
-  A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = t->chunk_mu; A.out = gr->dq; A.W = t->q; A.dot = qdq;
+  A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = (const bf16_t*)t->chunk_I; A.out = gr->dq; A.W = t->q; A.dot = qdq;
   A.dc = d->dv; A.de = d->dk;
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDq, s)) return rc;
   // dv: X = k, Y = q, Z = dO, tile-end state gradients
@@ -501,13 +550,14 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
 extern "C" int pal_gla_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
   using namespace pal;
   if (int rc = check_gla(d, t)) return rc;
+  if (!t->chunk_mu) return PAL_E_NULL;
   ChunkArgs a;
   fill_gla_args(a, d, t);
   hipStream_t s = (hipStream_t)stream;
   if (int rc = launch_tile_states(a, d->dtype, false, s)) return rc;
   GlaTileArgs A{};
   A.c = a;
-  A.X = t->q; A.Y = t->k; A.Z = t->v; A.St = t->chunk_mu; A.out = t->o;
+  A.X = t->q; A.Y = t->k; A.Z = t->v; A.St = (const bf16_t*)t->chunk_I; A.out = t->o;
   A.dc = d->dk; A.de = d->dv;
   return launch_gla_tile_dt(A, d->dtype, kGlaOut, s);
 }

@@ -84,7 +84,9 @@ class ChunkSimpleGLA(torch.autograd.Function):
         if p.init_mu is not None:
             flags |= L.PAL_FLAG_HAS_INIT
         o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
-        tile_S = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+        # per-tile contributions (fp32, only needed inside the call) and tile-start states (bf16, kept for the backward)
+        scratch = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
+        tile_S = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.bfloat16, device=dev)
         final = None
         if output_final_state:
             final = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
@@ -92,7 +94,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(p.q), k=pt(p.k), v=pt(p.v), gt=pt(p.gt), g=pt(p.g), o=pt(o), init_mu=pt(p.init_mu),
                                final_mu=pt(final), cu_seqlens=pt(p.cu_seqlens), chunk_table=pt(table),
-                               chunk_offsets=pt(offsets), chunk_mu=pt(tile_S))
+                               chunk_offsets=pt(offsets), chunk_mu=pt(scratch), chunk_I=pt(tile_S))
         with torch.cuda.device(dev):
             rc = L.load().pal_gla_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
         L.check(rc, "pal_gla_chunk_fwd")
@@ -130,7 +132,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
                          var_dtype=cm._pal_dtype(cd), flags=m["flags"], scale=m["scale"])
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), gt=pt(gt), g=pt(rate), o=pt(do), init_mu=pt(init),
-                               cu_seqlens=pt(cu), chunk_table=pt(table), chunk_offsets=pt(offsets), chunk_mu=pt(tile_S))
+                               cu_seqlens=pt(cu), chunk_table=pt(table), chunk_offsets=pt(offsets), chunk_I=pt(tile_S))
         grads = L.PalBwdTensors(d_o=pt(do), dq=pt(dq), dk=pt(dk), dv=pt(dv), dgt=pt(dg_tok), dg=pt(d_rate),
                                 d_init_mu=pt(d_init))
         lib = L.load()
