@@ -118,18 +118,16 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
           if (HAS_J) AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
         }
       }
+      // the products are taken transposed (K as the row operand) so that a lane ends up with four consecutive
+      // key columns of one value row: rows n = 16nb + 4g + r, column d = 16dt + i, one 16-byte store per lane
       f32x4 M = {0.f, 0.f, 0.f, 0.f}, J = {0.f, 0.f, 0.f, 0.f};
-      M = mfma16(AM[0], BK[0], M);
-      if (HAS_J) J = mfma16(AJ[0], BKK[0], J);
-      M = mfma16(AM[1], BK[1], M);
-      if (HAS_J) J = mfma16(AJ[1], BKK[1], J);
-      // accumulator layout: rows d = 16dt + 4g + r, column n = 16nb + i
-      const int64_t co = (((int64_t)cidx * H + h) * dv + 16 * dt + 4 * g) * dk + 16 * nb + i;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        a.chunk_mu[co + (int64_t)r * dk] = M[r];
-        if (HAS_J) a.chunk_I[co + (int64_t)r * dk] = J[r];
-      }
+      M = mfma16(BK[0], AM[0], M);
+      if (HAS_J) J = mfma16(BKK[0], AJ[0], J);
+      M = mfma16(BK[1], AM[1], M);
+      if (HAS_J) J = mfma16(BKK[1], AJ[1], J);
+      const int64_t co = (((int64_t)cidx * H + h) * dv + 16 * dt + i) * dk + 16 * nb + 4 * g;
+      *(f32x4*)&a.chunk_mu[co] = M;
+      if (HAS_J) *(f32x4*)&a.chunk_I[co] = J;
     }
   }
 }
@@ -217,17 +215,19 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t E = (int64_t)a.dv * a.dk;
-  const int nblk = (int)(E / 256);
+  const int nblk = (int)((E + 1023) / 1024);     // four consecutive entries per thread
   const int blk = blockIdx.x % nblk;
   const int nh = blockIdx.x / nblk;
   const int h = nh % a.H, n = nh / a.H;
-  const int64_t e = (int64_t)blk * 256 + tid;
+  const int64_t e = ((int64_t)blk * 256 + tid) * 4;
+  const bool on = e < E;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const int nchunks = (len + kC - 1) / kC;
   const float gh = a.g[h] * kLog2e;
   const int64_t so = (int64_t)nh * E + e;
-  float S = a.init_mu ? a.init_mu[so] : 0.f;
+  f32x4 S = {0.f, 0.f, 0.f, 0.f};
+  if (a.init_mu && on) S = *(const f32x4*)(a.init_mu + so);
   for (int c0 = 0; c0 < nchunks; c0 += kScanTiles) {
     const int cn = min(kScanTiles, nchunks - c0);
     __syncthreads();
@@ -238,25 +238,30 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
       if (lane == 0) sF[c] = fast_exp2(tot);
     }
     __syncthreads();
+    if (!on) continue;
     int c = 0;
-    for (; c + 8 <= cn; c += 8) {
-      float dS[8];
+    for (; c + 4 <= cn; c += 4) {
+      f32x4 dS[4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) dS[u] = a.chunk_mu[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e];
+      for (int u = 0; u < 4; ++u) dS[u] = *(const f32x4*)(a.chunk_mu + ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        tile_S[((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e] = (bf16_t)S;
-        S = fmaf(sF[c + u], S, dS[u]);
+      for (int u = 0; u < 4; ++u) {
+        store_vec<4>(tile_S + ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e, (const float*)&S);
+        const float F = sF[c + u];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) S[x] = fmaf(F, S[x], dS[u][x]);
       }
     }
     for (; c < cn; ++c) {
       const int64_t off = ((int64_t)(cbase + c0 + c) * a.H + h) * E + e;
-      const float dS = a.chunk_mu[off];
-      tile_S[off] = (bf16_t)S;
-      S = fmaf(sF[c], S, dS);
+      const f32x4 dS = *(const f32x4*)(a.chunk_mu + off);
+      store_vec<4>(tile_S + off, (const float*)&S);
+      const float F = sF[c];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) S[x] = fmaf(F, S[x], dS[x]);
     }
   }
-  if (a.final_mu) a.final_mu[so] = S;
+  if (a.final_mu && on) *(f32x4*)(a.final_mu + so) = S;
 }
 
 // ------------------------------------------------------------------ kernel 2
@@ -566,7 +571,8 @@ int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) 
 int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
   if (int rc = launch_tile_delta(a, dtype, has_j, s)) return rc;
   {
-    const int64_t blocks = (int64_t)a.n_seqs * a.H * (((int64_t)a.dv * a.dk) / 256);
+    const int64_t E = (int64_t)a.dv * a.dk;
+    const int64_t blocks = (int64_t)a.n_seqs * a.H * (has_j ? E / 256 : (E + 1023) / 1024);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
     if (has_j) PAL_TIMED_LAUNCH(kKernChunkScan, s, chunk_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
     else PAL_TIMED_LAUNCH(kKernChunkScan, s, gla_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);

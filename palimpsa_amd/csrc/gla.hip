@@ -345,16 +345,17 @@ __global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, const fl
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t E = (int64_t)a.dv * a.dk;
-  const int nblk = (int)(E / 256);
+  const int nblk = (int)((E + 1023) / 1024);     // four consecutive entries per thread
   const int blk = blockIdx.x % nblk;
   const int nh = blockIdx.x / nblk;
   const int h = nh % a.H, n = nh / a.H;
-  const int64_t e = (int64_t)blk * 256 + tid;
+  const int64_t e = ((int64_t)blk * 256 + tid) * 4;
+  const bool on = e < E;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const int nchunks = (len + kC - 1) / kC;
   const float gh = a.g[h] * kLog2e;
-  float G = 0.f;
+  f32x4 G = {0.f, 0.f, 0.f, 0.f};
   for (int c_hi = nchunks; c_hi > 0; c_hi -= kScanTiles) {
     const int c0 = max(0, c_hi - kScanTiles), cn = c_hi - c0;
     __syncthreads();
@@ -365,25 +366,33 @@ __global__ __launch_bounds__(256) void gla_bwd_scan_kernel(ChunkArgs a, const fl
       if (lane == 0) sF[c] = fast_exp2(tot);
     }
     __syncthreads();
+    if (!on) continue;
     int c = cn;
-    for (; c >= 8; c -= 8) {
-      float D[8];
+    for (; c >= 4; c -= 4) {
+      f32x4 D[4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) D[u] = buf[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e];
+      for (int u = 0; u < 4; ++u) D[u] = *(const f32x4*)(buf + ((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        g_tiles[((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e] = (bf16_t)G;
-        G = fmaf(sF[c - 1 - u], G, D[u]);
+      for (int u = 0; u < 4; ++u) {
+        store_vec<4>(g_tiles + ((int64_t)(cbase + c0 + c - 1 - u) * a.H + h) * E + e, (const float*)&G);
+        const float F = sF[c - 1 - u];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) G[x] = fmaf(F, G[x], D[u][x]);
       }
     }
     for (; c >= 1; --c) {
       const int64_t off = ((int64_t)(cbase + c0 + c - 1) * a.H + h) * E + e;
-      const float D = buf[off];
-      g_tiles[off] = (bf16_t)G;
-      G = fmaf(sF[c - 1], G, D);
+      const f32x4 D = *(const f32x4*)(buf + off);
+      store_vec<4>(g_tiles + off, (const float*)&G);
+      const float F = sF[c - 1];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) G[x] = fmaf(F, G[x], D[x]);
     }
   }
-  if (d_init) d_init[(int64_t)nh * E + e] = a.scale * G;
+  if (d_init && on) {
+    const f32x4 r = {a.scale * G[0], a.scale * G[1], a.scale * G[2], a.scale * G[3]};
+    *(f32x4*)(d_init + (int64_t)nh * E + e) = r;
+  }
 }
 
 // Gate gradients.  With C_t the running sum of the log decay l_t = -gt_t g over a sequence, q_t enters
@@ -515,7 +524,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
     ChunkArgs b = a;
     b.k = t->q; b.v = gr->d_o; b.chunk_mu = d_tiles; b.flags |= kFlagDecayFromStart;
     if (int rc = launch_tile_delta(b, d->dtype, false, s)) return rc;
-    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk) / 256);
+    const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk + 1023) / 1024);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
     PAL_TIMED_LAUNCH(kKernGlaBwdScan, s, gla_bwd_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, d_tiles,
                      g_tiles, gr->d_init_mu);

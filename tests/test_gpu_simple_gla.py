@@ -333,3 +333,40 @@ def test_recurrent_with_autograd_still_differentiates(gpu_device):
     _closed_form(*ref_leaves, 0.4)[0].sum().backward()
     for name, x, r in zip(("q", "k", "v", "g"), leaves, ref_leaves):
         assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
+
+
+def test_packed_batch_with_empty_documents(gpu_device):
+    """Documents of length zero (repeated cu_seqlens entries) take no tile; their final state is the initial one
+    and the gradients of the others are untouched."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    H, dk, dv = 2, 32, 32
+    cu = [0, 0, 70, 70, 135, 135]
+    q, k, v, g, _ = _inputs(1, cu[-1], H, dk, dv, 51)
+    gen = torch.Generator().manual_seed(52)
+    S0 = torch.randn(len(cu) - 1, H, dk, dv, generator=gen) * 0.2
+    do = torch.randn(1, cu[-1], H, dv, generator=gen)
+    dev = gpu_device
+    cu_d = torch.tensor(cu, device=dev)
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o, S = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], initial_state=leaves[4],
+                            output_final_state=True, cu_seqlens=cu_d)
+    (o.float() * do.to(dev)).sum().backward()
+    with torch.no_grad():
+        o_r, S_r = fused_recurrent_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), initial_state=S0.to(dev),
+                                              output_final_state=True, cu_seqlens=cu_d)
+    for j in range(len(cu) - 1):
+        sl = slice(cu[j], cu[j + 1])
+        if cu[j + 1] == cu[j]:
+            assert torch.equal(S[j].cpu(), S0[j]) and torch.equal(S_r[j].cpu(), S0[j])
+            assert torch.equal(leaves[4].grad[j].cpu(), torch.zeros(H, dk, dv))
+            continue
+        ref_leaves = [x[:, sl].double().clone().requires_grad_(True) for x in (q, k, v, g)]
+        S0_ref = S0[j:j + 1].double().clone().requires_grad_(True)
+        o_ref, S_ref = _closed_form(*ref_leaves, dk ** -0.5, S0_ref)
+        (o_ref * do[:, sl].double()).sum().backward()
+        assert hp.max_abs(o[:, sl].float(), o_ref.detach()) <= hp.BF16_OUT_ABS_TOL
+        assert hp.max_abs(o_r[:, sl].float(), o_ref.detach()) <= hp.BF16_OUT_ABS_TOL
+        assert hp.max_rel(S[j:j + 1], S_ref.detach()) <= 1e-2 and hp.max_rel(S_r[j:j + 1], S_ref.detach()) <= hp.FP32_REL_TOL
+        for name, x, r in zip(("q", "k", "v", "g"), leaves, ref_leaves):
+            assert hp.max_rel(x.grad[:, sl], r.grad) <= hp.BF16_GRAD_NORM_TOL, (j, name)
+        assert hp.max_rel(leaves[4].grad[j:j + 1], S0_ref.grad) <= hp.BF16_GRAD_NORM_TOL
