@@ -370,3 +370,38 @@ def test_packed_batch_with_empty_documents(gpu_device):
         for name, x, r in zip(("q", "k", "v", "g"), leaves, ref_leaves):
             assert hp.max_rel(x.grad[:, sl], r.grad) <= hp.BF16_GRAD_NORM_TOL, (j, name)
         assert hp.max_rel(leaves[4].grad[j:j + 1], S0_ref.grad) <= hp.BF16_GRAD_NORM_TOL
+
+
+def test_sequence_longer_than_one_scan_window(gpu_device):
+    """More than 1024 tiles in one sequence: the state scans (forward and reverse) and the gate suffix sums work in
+    windows.  Forward against the token-serial kernel, gradients against the Palimpsa kernels on b = 0, Ip = 1
+    (both independent code), bf16 gates."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    B, T, H, dk, dv = 1, 1031 * 64 + 7, 2, 16, 32
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 61)
+    g = (g * 0.2).bfloat16()
+    gen = torch.Generator().manual_seed(62)
+    do = torch.randn(B, T, H, dv, generator=gen).bfloat16()
+    dev = gpu_device
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o, S = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], initial_state=leaves[4],
+                            output_final_state=True)
+    o.backward(do.to(dev))
+    with torch.no_grad():
+        o_r, S_r = fused_recurrent_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), initial_state=S0.to(dev),
+                                              output_final_state=True)
+    assert hp.max_abs(o.float(), o_r.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_r) <= 1e-2
+    ref = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    mu0 = S0.transpose(-1, -2).contiguous().to(dev).requires_grad_(True)
+    ones = torch.ones(H, device=dev)
+    o_p = chunk_palimpsa(ref[0], ref[1], ref[2], torch.zeros_like(ref[2]), -ref[3].float(), ones, ones,
+                         initial_mu_state=mu0, initial_I_state=torch.ones_like(mu0))
+    o_p.backward(do.to(dev))
+    assert leaves[3].grad.dtype == torch.bfloat16
+    for name, x, r in zip(("q", "k", "v"), leaves, ref):
+        assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
+    # the gate gradient accumulates over up to 66 k tokens; bf16 output, compared where the reference is large
+    assert hp.max_rel(leaves[3].grad.float(), ref[3].grad.float()) <= 2 * hp.BF16_GRAD_NORM_TOL
+    assert hp.max_rel(leaves[4].grad, mu0.grad.transpose(-1, -2)) <= hp.BF16_GRAD_NORM_TOL
