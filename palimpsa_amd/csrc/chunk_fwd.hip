@@ -27,8 +27,8 @@ namespace pal {
 // MFMA operand is one contiguous run of tokens), then wave w produces the 16x16 blocks of the state
 // whose key columns are [16w, 16w+16) (+64, ...).  The result is parked in the tile's slot of
 // chunk_mu / chunk_I until the scan below replaces it.
-// Row stride (elements) of the transposed staging tiles: fp32 tiles while they fit in LDS, bf16 tiles (half the
-// size; the operands are rounded to bf16 anyway) for the largest head dims.
+// Row stride (elements) of the transposed staging tiles.  bf16 rows are staged as they are; fp32 rows in fp32
+// tiles while those fit in LDS, else rounded to bf16 (the operands built from them are bf16 anyway).
 template <typename TS>
 struct StageStride { static constexpr int value = sizeof(TS) == 4 ? 68 : 72; };
 
@@ -38,18 +38,39 @@ __device__ __forceinline__ void stage_transposed(const TIn* src, int64_t row_str
   // src: [64 tokens][width] rows -> dst[width][stride] (token index fastest), rows >= clen are zero
   constexpr int kTS = StageStride<TS>::value;
   const int groups = width >> 3;
-  for (int idx = tid; idx < kC * groups; idx += 256) {
-    const int s = idx & (kC - 1), c8 = idx >> 6;
-    float x[8];
-    if (s < clen) {
-      load_vec<4>(src + (int64_t)s * row_stride + 8 * c8, x);
-      load_vec<4>(src + (int64_t)s * row_stride + 8 * c8 + 4, x + 4);
-    } else {
+  if constexpr (sizeof(TS) == 2) {
+    // bf16 tiles: a work item is two consecutive tokens by eight columns, so that neighbouring lanes read
+    // neighbouring 16-byte pieces of a row and a pair of tokens goes to LDS as one 32-bit word per column
+    for (int idx = tid; idx < (kC / 2) * groups; idx += 256) {
+      const int sp = idx / groups, c8 = idx - sp * groups;
+      float x0[8], x1[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = 0.f;
+      for (int e = 0; e < 8; ++e) { x0[e] = 0.f; x1[e] = 0.f; }
+      if (2 * sp < clen) {
+        load_vec<4>(src + (int64_t)(2 * sp) * row_stride + 8 * c8, x0);
+        load_vec<4>(src + (int64_t)(2 * sp) * row_stride + 8 * c8 + 4, x0 + 4);
+      }
+      if (2 * sp + 1 < clen) {
+        load_vec<4>(src + (int64_t)(2 * sp + 1) * row_stride + 8 * c8, x1);
+        load_vec<4>(src + (int64_t)(2 * sp + 1) * row_stride + 8 * c8 + 4, x1 + 4);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *(bf16x2*)&dst[(8 * c8 + e) * kTS + 2 * sp] = pack2(x0[e], x1[e]);
     }
+  } else {
+    for (int idx = tid; idx < kC * groups; idx += 256) {
+      const int s = idx & (kC - 1), c8 = idx >> 6;
+      float x[8];
+      if (s < clen) {
+        load_vec<4>(src + (int64_t)s * row_stride + 8 * c8, x);
+        load_vec<4>(src + (int64_t)s * row_stride + 8 * c8 + 4, x + 4);
+      } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dst[(8 * c8 + e) * kTS + s] = from_f32<TS>(x[e]);
+        for (int e = 0; e < 8; ++e) x[e] = 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[(8 * c8 + e) * kTS + s] = x[e];
+    }
   }
 }
 
@@ -555,8 +576,10 @@ static int launch_tile_delta_t(const ChunkArgs& a, hipStream_t s) {
 
 template <typename TIn, bool HAS_J>
 static int launch_tile_delta_j(const ChunkArgs& a, hipStream_t s) {
-  const size_t lds_f32 = sizeof(float) * (kC + (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<float>::value);
-  if (lds_f32 <= kMaxLds) return launch_tile_delta_t<TIn, HAS_J, float>(a, s);
+  if constexpr (sizeof(TIn) == 4) {
+    const size_t lds_f32 = sizeof(float) * (kC + (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<float>::value);
+    if (lds_f32 <= kMaxLds) return launch_tile_delta_t<TIn, HAS_J, float>(a, s);
+  }
   return launch_tile_delta_t<TIn, HAS_J, bf16_t>(a, s);
 }
 

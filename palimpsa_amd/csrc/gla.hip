@@ -199,14 +199,20 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
   for (int el = 0; el < EB; ++el)
 #pragma unroll
     for (int xb = 0; xb < 4; ++xb) acc[el][xb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 Xn[4];
+#pragma unroll
+  for (int xb = 0; xb < 4; ++xb) Xn[xb] = x_operand(xb, 0);
   for (int ks = 0; ks < KS; ++ks) {
-    bf16x8 Sa[EB];
+    bf16x8 Sa[EB], Xo[4];
 #pragma unroll
     for (int el = 0; el < EB; ++el) Sa[el] = raw[el];
-    if (ks + 1 < KS) fetch_state(ks + 1);     // in flight while this step's products run
-    bf16x8 Xo[4];
 #pragma unroll
-    for (int xb = 0; xb < 4; ++xb) Xo[xb] = x_operand(xb, ks);
+    for (int xb = 0; xb < 4; ++xb) Xo[xb] = Xn[xb];
+    if (ks + 1 < KS) {                         // next step's operands in flight while this step's products run
+      fetch_state(ks + 1);
+#pragma unroll
+      for (int xb = 0; xb < 4; ++xb) Xn[xb] = x_operand(xb, ks + 1);
+    }
 #pragma unroll
     for (int el = 0; el < EB; ++el)
 #pragma unroll
@@ -237,18 +243,15 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
 #pragma unroll
       for (int p = 0; p < 2; ++p)
         if ((REVERSE ? 2 * p + 1 >= xb : 2 * p <= xb)) acc[el][xb] = mfma16(Za[p], P[xb][p], acc[el][xb]);
+      // finished block: scale, and take the dot product with W while the values are still fp32
       const int x = 16 * xb + i;
-      if (valid && x < clen) {
-        const float res[4] = {acc[el][xb][0] * scale, acc[el][xb][1] * scale, acc[el][xb][2] * scale,
-                              acc[el][xb][3] * scale};
-        const int64_t off = ((int64_t)(t0 + x) * H + h) * de + 16 * eb + 4 * g;
-        store_vec<4>((TIn*)A.out + off, res);
-        if (has_dot) {
-          float wv[4];
-          load_vec<4>((const TIn*)A.W + off, wv);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) dot[xb] = fmaf(wv[r], res[r], dot[xb]);
-        }
+      for (int r = 0; r < 4; ++r) acc[el][xb][r] *= scale;
+      if (has_dot && valid && x < clen) {
+        float wv[4];
+        load_vec<4>((const TIn*)A.W + ((int64_t)(t0 + x) * H + h) * de + 16 * eb + 4 * g, wv);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dot[xb] = fmaf(wv[r], acc[el][xb][r], dot[xb]);
       }
     }
   }
@@ -256,9 +259,32 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
     // rows g of a wave hold different output columns of the same token: sum them, then the four waves
     const float tot = rows4_sum_x4(dot[0], dot[1], dot[2], dot[3]);   // lanes of row g: token block g
     sDot[w * kC + lane] = tot;                                        // lane = 16 g + i = token
-    __syncthreads();
-    if (w == 0 && lane < clen)
-      A.dot[(int64_t)(t0 + lane) * H + h] = (sDot[lane] + sDot[kC + lane]) + (sDot[2 * kC + lane] + sDot[3 * kC + lane]);
+  }
+  // The results go out through LDS (the staging tiles are dead once every wave has its products): a lane holds
+  // four columns of one token, which would make 8-byte pieces of rows; from the tile in LDS each row is written
+  // as one contiguous run of 16-byte accesses.
+  __syncthreads();
+  TIn* sOut = (TIn*)sP;               // [64][de + 8 / sizeof-ratio] over the score, Y and Z tiles
+  const int ostride = de + (16 / (int)sizeof(TIn));
+#pragma unroll
+  for (int el = 0; el < EB; ++el) {
+    const int ebn = w * EB + el;
+    if (ebn < n_eb) {
+#pragma unroll
+      for (int xb = 0; xb < 4; ++xb) store_vec<4>(sOut + (16 * xb + i) * ostride + 16 * ebn + 4 * g, (const float*)&acc[el][xb]);
+    }
+  }
+  if (has_dot && w == 0 && lane < clen)
+    A.dot[(int64_t)(t0 + lane) * H + h] = (sDot[lane] + sDot[kC + lane]) + (sDot[2 * kC + lane] + sDot[3 * kC + lane]);
+  __syncthreads();
+  {
+    constexpr int VEC = 16 / (int)sizeof(TIn);   // elements per 16-byte access
+    const int per_row = de / VEC;
+    TIn* obase = (TIn*)A.out + ((int64_t)t0 * H + h) * de;
+    for (int idx = tid; idx < clen * per_row; idx += 256) {
+      const int x = idx / per_row, c = idx - x * per_row;
+      *(f32x4*)(obase + (int64_t)x * H * de + VEC * c) = *(const f32x4*)(sOut + x * ostride + VEC * c);
+    }
   }
 }
 
@@ -267,8 +293,10 @@ enum GlaRole { kGlaOut = 0, kGlaDq, kGlaDv, kGlaDk };
 template <typename TIn, int EB, bool REVERSE, bool STATE_T>
 static int launch_gla_tile_eb(const GlaTileArgs& A, int kern_id, hipStream_t s) {
   const int KS = (A.dc + 31) / 32;
-  const size_t lds = sizeof(float) * (kC + 4 * kC) + 16 * 4 * 2 * 64 +
-                     sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+  const size_t lds_head = sizeof(float) * (kC + 4 * kC);
+  const size_t lds_stage = 16 * 4 * 2 * 64 + sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+  const size_t lds_out = (size_t)kC * (A.de * sizeof(TIn) + 16);   // the output tile reuses the staging area
+  const size_t lds = lds_head + (lds_stage > lds_out ? lds_stage : lds_out);
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;
