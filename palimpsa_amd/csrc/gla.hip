@@ -56,14 +56,14 @@ struct GlaTileArgs {
 //   dk  : X = v,  Y = dO, Z = q,  St = G read transposed,                              reverse
 // One workgroup of 4 waves per (tile, head), two phases.
 //  (1) Scores: wave w owns the tokens x in [16w, 16w+16).
-//        P^T[y,x] = sum_c Y[y,c] X[x,c]        A = Y rows (LDS), B = the wave's X rows (global)
+//        P^T[y,x] = sum_c Y[y,c] X[x,c]        A = Y rows (LDS), B = the wave's X rows (LDS)
 //        P^T     *= L(x,y), masked             in the accumulator layout (column x per lane, 4 rows y)
 //      The accumulators of two neighbouring y blocks, rounded to bf16, ARE a B operand of the second
 //      product when its contraction index is mapped to tokens as slot (g, j) -> y = 32p + 16(j/4) + 4g + j%4;
 //      they are parked in LDS so that every wave can use the scores of all 64 tokens.
 //  (2) Output: wave w owns the blocks of 16 output columns [w EB, (w+1) EB) for all 64 tokens.
 //        out^T[e,x] = w_x sum_c St[e,c] X[x,c]  A = state rows (global, bf16), loaded once and used
-//                                               for the four token blocks, B = X rows (global, L1)
+//                                               for the four token blocks, B = X rows (LDS)
 //                   + sum_y Z^T[e,y] P^T[y,x]   A = Z^T rows (LDS, read with the token map above)
 //      so every state entry is read by exactly one wave of the workgroup.
 // EB = ceil(de / 64) column blocks per wave.
@@ -78,7 +78,8 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
   float* sDot = sC + kC;              // [4][64] partial dot products of the waves
   bf16x8* sP = (bf16x8*)(sDot + 4 * kC);   // [4 token blocks][2][64 lanes] score operands
   bf16_t* sY = (bf16_t*)(sP + 4 * 2 * 64); // [64][dcp]
-  bf16_t* sZT = sY + kC * dcp;        // [de][kVT]
+  bf16_t* sX = sY + kC * dcp;         // [64][dcp]
+  bf16_t* sZT = sX + kC * dcp;        // [de][kVT]
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
@@ -89,14 +90,8 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     sC[lane] = wave_inclusive_scan(-gt * gh, lane);
   }
-  const TIn* xbase = (const TIn*)A.X + ((int64_t)t0 * H + h) * dc + 8 * g;
-  // X rows of token block xb as a B operand (column x = 16 xb + i, contraction index c = 32 ks + 8 g + j)
-  auto x_operand = [&](int xb, int ks) {
-    bf16x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
-    const int x = 16 * xb + i;
-    if (x < clen && 32 * ks + 8 * g < dc) r = load_bf16x8(xbase + (int64_t)x * H * dc + 32 * ks);
-    return r;
-  };
+  // X rows of token block xb as a B operand (column x = 16 xb + i, contraction index c = 32 ks + 8 g + j), from LDS
+  auto x_operand = [&](int xb, int ks) { return *(const bf16x8*)(sX + (16 * xb + i) * dcp + 8 * g + 32 * ks); };
   // State operands of this wave: blocks of 16 output columns [w EB, (w+1) EB), rows e = 16 eb + i, contraction
   // index c = 32 ks + 8 g + j.  The first step is requested before the staging below so that its latency
   // overlaps the staging's, every further step one step ahead of its use.
@@ -132,9 +127,13 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
     const int groups = 4 * KS;
     for (int idx = tid; idx < kC * groups; idx += 256) {
       const int s = idx / groups, c8 = idx - s * groups;
-      bf16x8 yx = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (s < clen && 8 * c8 < dc) yx = load_bf16x8(yp + (int64_t)s * H * dc + 8 * c8);
+      bf16x8 yx = {0, 0, 0, 0, 0, 0, 0, 0}, xx = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (s < clen && 8 * c8 < dc) {
+        yx = load_bf16x8(yp + (int64_t)s * H * dc + 8 * c8);
+        xx = load_bf16x8((const TIn*)A.X + ((int64_t)(t0 + s) * H + h) * dc + 8 * c8);
+      }
       *(bf16x8*)&sY[s * dcp + 8 * c8] = yx;
+      *(bf16x8*)&sX[s * dcp + 8 * c8] = xx;
     }
     // Z transposed (token index fastest), zero beyond the tile's tokens.  A work item is two consecutive
     // tokens by eight columns: neighbouring lanes read neighbouring 16-byte pieces of a row, and a
@@ -294,7 +293,7 @@ template <typename TIn, int EB, bool REVERSE, bool STATE_T>
 static int launch_gla_tile_eb(const GlaTileArgs& A, int kern_id, hipStream_t s) {
   const int KS = (A.dc + 31) / 32;
   const size_t lds_head = sizeof(float) * (kC + 4 * kC);
-  const size_t lds_stage = 16 * 4 * 2 * 64 + sizeof(bf16_t) * ((size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+  const size_t lds_stage = 16 * 4 * 2 * 64 + sizeof(bf16_t) * (2 * (size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
   const size_t lds_out = (size_t)kC * (A.de * sizeof(TIn) + 16);   // the output tile reuses the staging area
   const size_t lds = lds_head + (lds_stage > lds_out ? lds_stage : lds_out);
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
