@@ -185,16 +185,19 @@ def bench_simple_gla(torch, dev, steps, warmup):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    L.profile_enable(True)
-    torch.cuda.synchronize()
+    # the step is timed without the per-launch events (they cost host time on a step this short) ...
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    # ... and the kernels in a second pass with them
+    L.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
     kern = L.profile_read()
     L.profile_enable(False)
-    ms = elapsed * 1e3 / steps
     # algorithmic bytes of one launch of the forward tile kernel: q, k, v rows in, tile-start state (bf16) in, o out, gates
     tiles = B * (T // CHUNK) * H
     bytes_out = tiles * (CHUNK * (2 * d + d) * 2 + d * d * 2 + CHUNK * d * 2 + CHUNK * 4)
@@ -270,16 +273,17 @@ def bench_layer_slice(torch, dev, steps, warmup):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    L.profile_enable(True)
-    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    L.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
     kern = L.profile_read()
     L.profile_enable(False)
-    ms = elapsed * 1e3 / steps
     rows = B * T * H
     # algorithmic bytes of the prologue backward: q_raw, k_raw, dq, dk, x, dv, b_raw, db in; dq_raw, dk_raw, dx, db_raw
     # out (bf16 rows), plus the per-(token, head) scalars dt_raw, bs_raw (bf16) and dgt (fp32) in, ddt_raw, dbs_raw out

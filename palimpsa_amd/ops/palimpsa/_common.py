@@ -140,7 +140,14 @@ def make_fwd_tensors(p: Prepared, o, o_var, final_mu, final_I, chunk_table=None,
         chunk_mu=_ptr(chunk_mu), chunk_I=_ptr(chunk_I))
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream_ptr(dev: torch.device):
+    """Handle of torch's current stream on ``dev`` for the C ABI (the raw accessor saves ~20 us of host time
+    per call over constructing a torch.cuda.Stream object)."""
+    if _raw_stream is not None:
+        return C.c_void_p(_raw_stream(dev.index if dev.index is not None else torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 

@@ -34,6 +34,18 @@ from ..palimpsa.chunk import _chunk_meta, _count_chunks
 __all__ = ["chunk_simple_gla", "fused_recurrent_simple_gla"]
 
 
+_RATE_CACHE: dict = {}
+
+
+def _minus_one_rate(H: int, dev: torch.device) -> torch.Tensor:
+    """fp32 [H] tensor of -1 (the kernels compute f_t = exp(-gt_t * rate) and take g itself as gt); kept per device."""
+    key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device(), H)
+    t = _RATE_CACHE.get(key)
+    if t is None:
+        t = _RATE_CACHE[key] = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
+    return t
+
+
 def _run(op, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, **kw):
     if g is None:
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
@@ -65,8 +77,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
     def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens):
         H = q.shape[2]
         dev = q.device
-        # f_t = exp(-gt_t * rate): the kernels take g itself as gt with a rate of -1
-        rate = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
+        rate = _minus_one_rate(H, dev)
         S0 = None
         if initial_state is not None:
             S0 = initial_state.float().transpose(-1, -2).contiguous()       # [N,H,dk,dv] -> [N,H,dv,dk]
@@ -184,7 +195,7 @@ def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
         scale = q.shape[-1] ** -0.5
     H = q.shape[2]
     dev = q.device
-    rate = torch.full((H,), -1.0, dtype=torch.float32, device=dev)    # f_t = exp(-g_t * rate)
+    rate = _minus_one_rate(H, dev)
     p = cm.prepare_inputs(q, k, v, v, g, rate, rate, None, None, cu_seqlens, recurrent=False)
     S0 = None
     if initial_state is not None:
