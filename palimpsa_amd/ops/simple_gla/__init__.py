@@ -42,7 +42,8 @@ def _minus_one_rate(H: int, dev: torch.device) -> torch.Tensor:
     key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device(), H)
     t = _RATE_CACHE.get(key)
     if t is None:
-        t = _RATE_CACHE[key] = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
+        with torch.inference_mode(False):     # a tensor made under inference mode could not be saved for a later backward
+            t = _RATE_CACHE[key] = torch.full((H,), -1.0, dtype=torch.float32, device=dev)
     return t
 
 
