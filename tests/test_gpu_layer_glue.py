@@ -160,3 +160,48 @@ def test_layer_slice_end_to_end(gpu_device):
     for n in NAMES:
         err = hp.max_rel(leaves[n].grad, refl[n].grad)
         assert err <= 2 * hp.BF16_GRAD_NORM_TOL, (n, err)
+
+
+def test_random_shape_sweep(gpu_device):
+    """Seeded random shapes of both glue kernels (head dims any multiple of 8 up to 256, odd token counts, repeated
+    q/k heads), forward and backward against the oracle."""
+    import random
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs, palimpsa_output_norm
+    rng = random.Random(4321)
+    dev = gpu_device
+    for case in range(12):
+        Hqk = rng.choice([1, 2, 3])
+        H = Hqk * rng.choice([1, 2, 4])
+        dk, dv = 8 * rng.randint(1, 32), 8 * rng.randint(1, 32)
+        lead = (rng.randint(1, 3), rng.randint(1, 90))
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float32])
+        a = _inputs(lead, Hqk, H, dk, dv, 3000 + case, dtype)
+        leaves = {n: a[n].to(dev).clone().requires_grad_(True) for n in NAMES}
+        outs = palimpsa_inputs(**leaves)
+        refl = {n: a[n].double().clone().requires_grad_(True) for n in NAMES}
+        refs = lo.prologue(**refl, model_dtype=dtype)
+        gen = torch.Generator().manual_seed(4000 + case)
+        loss = loss_ref = 0.0
+        out_tol, grad_tol = (hp.BF16_OUT_ABS_TOL, hp.BF16_GRAD_NORM_TOL) if dtype == torch.bfloat16 else (1e-4, 1e-4)
+        tag = (case, lead, Hqk, H, dk, dv, dtype)
+        for y, r in zip(outs, refs):
+            assert hp.max_abs(y.float(), r) <= out_tol * max(1.0, r.abs().max().item()), tag
+            wgt = torch.randn(r.shape, generator=gen).to(y.dtype)
+            loss = loss + (y.float() * wgt.to(dev).float()).sum()
+            loss_ref = loss_ref + (r * wgt.double()).sum()
+        loss.backward()
+        loss_ref.backward()
+        for n in NAMES:
+            assert hp.max_rel(leaves[n].grad, refl[n].grad) <= grad_tol, (n,) + tag
+        # epilogue on the same shape
+        o = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+        gate = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+        Dp, w = torch.randn(H, generator=gen), 1.0 + 0.2 * torch.randn(dv, generator=gen)
+        dy = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+        ts = [o, a["x"], Dp, gate, w]
+        lv = [t.to(dev).clone().requires_grad_(True) for t in ts]
+        palimpsa_output_norm(*lv, 1e-5).backward(dy.to(dev))
+        rv = [t.double().clone().requires_grad_(True) for t in ts]
+        lo.epilogue(*rv, 1e-5).backward(dy.double())
+        for name, t, r in zip(("o", "x", "D", "gate", "weight"), lv, rv):
+            assert hp.max_rel(t.grad, r.grad) <= grad_tol, (name,) + tag

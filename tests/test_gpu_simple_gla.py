@@ -405,3 +405,56 @@ def test_sequence_longer_than_one_scan_window(gpu_device):
     # the gate gradient accumulates over up to 66 k tokens; bf16 output, compared where the reference is large
     assert hp.max_rel(leaves[3].grad.float(), ref[3].grad.float()) <= 2 * hp.BF16_GRAD_NORM_TOL
     assert hp.max_rel(leaves[4].grad, mu0.grad.transpose(-1, -2)) <= hp.BF16_GRAD_NORM_TOL
+
+
+def test_random_shape_sweep(gpu_device):
+    """Seeded random shapes (head dims any multiple of 8 up to 256 through the host-side padding, ragged lengths,
+    packed or batched, with or without an initial state): forward and backward against the closed form."""
+    import random
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    rng = random.Random(1234)
+    dev = gpu_device
+    for case in range(14):
+        H = rng.choice([1, 2, 3, 5])
+        dk = 8 * rng.randint(1, 32)
+        dv = 8 * rng.randint(1, 32)
+        packed = rng.random() < 0.4
+        if packed:
+            lens = [rng.randint(1, 150) for _ in range(rng.randint(1, 4))]
+            B, T = 1, sum(lens)
+            cu = [0]
+            for ln in lens:
+                cu.append(cu[-1] + ln)
+        else:
+            B, T, cu = rng.choice([1, 2]), rng.randint(1, 200), None
+        with_state = rng.random() < 0.5
+        scale = rng.choice([1.0, 0.37, dk ** -0.5])
+        q, k, v, g, _ = _inputs(B, T, H, dk, dv, 1000 + case)
+        n_seq = len(cu) - 1 if cu else B
+        gen = torch.Generator().manual_seed(2000 + case)
+        S0 = torch.randn(n_seq, H, dk, dv, generator=gen) * 0.2 if with_state else None
+        do = torch.randn(B, T, H, dv, generator=gen)
+        tensors = [q, k, v, g] + ([S0] if with_state else [])
+        leaves = [x.to(dev).clone().requires_grad_(True) for x in tensors]
+        o, S = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], scale=scale,
+                                initial_state=leaves[4] if with_state else None, output_final_state=True,
+                                cu_seqlens=torch.tensor(cu, device=dev) if cu else None)
+        (o.float() * do.to(dev)).sum().backward()
+        ref = [x.double().clone().requires_grad_(True) for x in tensors]
+        if cu:
+            outs, states = [], []
+            for j in range(n_seq):
+                sl = slice(cu[j], cu[j + 1])
+                o_j, S_j = _closed_form(ref[0][:, sl], ref[1][:, sl], ref[2][:, sl], ref[3][:, sl], scale,
+                                        ref[4][j:j + 1] if with_state else None)
+                outs.append(o_j)
+                states.append(S_j)
+            o_ref, S_ref = torch.cat(outs, dim=1), torch.cat(states, dim=0)
+        else:
+            o_ref, S_ref = _closed_form(ref[0], ref[1], ref[2], ref[3], scale, ref[4] if with_state else None)
+        (o_ref * do.double()).sum().backward()
+        tag = (case, B, T, H, dk, dv, cu, with_state)
+        assert hp.max_abs(o.float(), o_ref.detach()) <= hp.BF16_OUT_ABS_TOL * max(1.0, o_ref.abs().max().item()), tag
+        assert hp.max_rel(S, S_ref.detach()) <= 1e-2, tag
+        for name, x, r in zip(("q", "k", "v", "g", "S0"), leaves, ref):
+            assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, (name,) + tag
