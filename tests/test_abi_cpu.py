@@ -163,3 +163,85 @@ def test_chunk_table_rejects_bad_cu_seqlens(L):
     out = (C.c_int32 * 8)()
     assert lib.pal_build_chunk_table(cu, 2, out, 2, None) == L.PAL_E_CAPACITY
     assert lib.pal_build_chunk_table(None, 2, None, 0, None) == L.PAL_E_NULL
+
+
+def test_simple_gla_entry_points_reject_bad_arguments(L):
+    """Host-side checks of the entry points without the precision state (no HIP call before they pass)."""
+    lib = L.load()
+    ok = dict(chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000))
+    for fn in (lib.pal_gla_chunk_fwd, lib.pal_gla_recurrent_fwd):
+        assert fn(None, None, None) == L.PAL_E_NULL
+        assert fn(_dims(L), None, None) == L.PAL_E_NULL
+        assert fn(_dims(L), _fwd_tensors(L, q=None, **ok), None) == L.PAL_E_NULL
+        assert fn(_dims(L, dv=40), _fwd_tensors(L, **ok), None) == L.PAL_E_HEADDIM
+        assert fn(_dims(L, flags=L.PAL_FLAG_HAS_VAR), _fwd_tensors(L, o_var=_fake(), **ok), None) == L.PAL_E_STATE
+        assert fn(_dims(L, flags=L.PAL_FLAG_HAS_INIT), _fwd_tensors(L, **ok), None) == L.PAL_E_STATE
+        assert fn(_dims(L), _fwd_tensors(L, final_mu=_fake(), **ok), None) == L.PAL_E_STATE
+        assert fn(_dims(L), _fwd_tensors(L, cu_seqlens=_fake(), **ok), None) == L.PAL_E_CU_SEQLENS
+        assert fn(_dims(L), _fwd_tensors(L, v=_fake(0x3008), **ok), None) == L.PAL_E_ALIGN
+    # the chunked form needs both tile buffers and a consistent tile count
+    assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_mu=_fake(0x9000)), None) == L.PAL_E_NULL
+    assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_I=_fake(0xa000)), None) == L.PAL_E_NULL
+    assert lib.pal_gla_chunk_fwd(_dims(L, total_chunks=3), _fwd_tensors(L, **ok), None) == L.PAL_E_CHUNK
+    assert lib.pal_gla_chunk_fwd(_dims(L, batch=1, n_seqs=2, seq_len=32, flags=L.PAL_FLAG_VARLEN),
+                                 _fwd_tensors(L, cu_seqlens=_fake(), **ok), None) == L.PAL_E_NULL      # chunk tables
+    # backward
+    gr = L.PalBwdTensors(**{n: _fake(0x1000 * (i + 20)) for i, n in enumerate(("d_o", "dq", "dk", "dv", "dgt", "dg"))})
+    assert lib.pal_gla_chunk_bwd(_dims(L), _fwd_tensors(L, **ok), None, None, 0, None) == L.PAL_E_NULL
+    assert lib.pal_gla_chunk_bwd(_dims(L), _fwd_tensors(L, **ok), gr, None, 0, None) == L.PAL_E_WORKSPACE
+    need = lib.pal_gla_chunk_bwd_workspace_bytes(_dims(L))
+    # D (fp32) and G (bf16) tiles, two rows of dot products, per-sequence shares of dg
+    assert need >= 2 * 2 * 32 * 32 * (4 + 2) + 2 * 2 * 16 * 2 * 4 + 2 * 2 * 4
+    assert lib.pal_gla_chunk_bwd(_dims(L), _fwd_tensors(L, **ok), gr, _fake(0x100000), need - 1, None) == L.PAL_E_WORKSPACE
+    gr2 = L.PalBwdTensors(**{n: _fake(0x1000 * (i + 20)) for i, n in enumerate(("d_o", "dq", "dk", "dv", "dgt", "dg", "d_init_mu"))})
+    assert lib.pal_gla_chunk_bwd(_dims(L), _fwd_tensors(L, **ok), gr2, _fake(0x100000), need, None) == L.PAL_E_STATE
+    assert lib.pal_gla_chunk_bwd_workspace_bytes(_dims(L, dk=5)) == 0
+
+
+def test_layer_glue_entry_points_reject_bad_arguments(L):
+    lib = L.load()
+
+    def gd(**kw):
+        d = dict(tokens=10, n_heads=4, n_qk_heads=2, dk=32, dv=64, dtype=L.PAL_DTYPE_BF16, eps=1e-6)
+        d.update(kw)
+        return L.PalGlueDims(**d)
+
+    names = ("q_raw", "k_raw", "x", "dt_raw", "bs_raw", "b_raw", "dt_bias", "b_scale", "q", "k", "v", "b", "gt")
+
+    def pt(**kw):
+        t = {n: _fake(0x1000 * (i + 1)) for i, n in enumerate(names)}
+        t.update(kw)
+        return L.PalPrologueTensors(**t)
+
+    assert lib.pal_prologue_fwd(None, None, None) == L.PAL_E_NULL
+    assert lib.pal_prologue_fwd(gd(), None, None) == L.PAL_E_NULL
+    assert lib.pal_prologue_fwd(gd(tokens=0), pt(), None) == L.PAL_E_DIM
+    assert lib.pal_prologue_fwd(gd(n_qk_heads=3), pt(), None) == L.PAL_E_DIM           # 4 heads not a multiple of 3
+    assert lib.pal_prologue_fwd(gd(dk=12), pt(), None) == L.PAL_E_HEADDIM
+    assert lib.pal_prologue_fwd(gd(dv=264), pt(), None) == L.PAL_E_HEADDIM
+    assert lib.pal_prologue_fwd(gd(dtype=7), pt(), None) == L.PAL_E_DTYPE
+    assert lib.pal_prologue_fwd(gd(), pt(x=None), None) == L.PAL_E_NULL
+    assert lib.pal_prologue_fwd(gd(), pt(b=None), None) == L.PAL_E_STATE                # b_raw without b
+    assert lib.pal_prologue_fwd(gd(), pt(b_scale=None), None) == L.PAL_E_NULL
+    assert lib.pal_prologue_fwd(gd(), pt(q=_fake(0x9004)), None) == L.PAL_E_ALIGN
+    assert lib.pal_prologue_bwd(gd(), pt(), None, None, 0, None) == L.PAL_E_NULL
+    gnames = ("dq", "dk", "dv", "db", "dgt", "dq_raw", "dk_raw", "dx", "db_raw", "ddt_raw", "dbs_raw", "ddt_bias", "db_scale")
+    gr = L.PalPrologueGrads(**{n: _fake(0x1000 * (i + 30)) for i, n in enumerate(gnames)})
+    assert lib.pal_prologue_bwd(gd(), pt(), gr, None, 0, None) == L.PAL_E_WORKSPACE
+    assert lib.pal_prologue_bwd_workspace_bytes(gd()) > 0 and lib.pal_prologue_bwd_workspace_bytes(gd(dk=3)) == 0
+
+    def et(**kw):
+        t = {n: _fake(0x1000 * (i + 1)) for i, n in enumerate(("o", "x", "D", "gate", "weight", "y", "rstd"))}
+        t.update(kw)
+        return L.PalEpilogueTensors(**t)
+
+    assert lib.pal_epilogue_fwd(gd(), None, None) == L.PAL_E_NULL
+    assert lib.pal_epilogue_fwd(gd(), et(weight=None), None) == L.PAL_E_NULL
+    assert lib.pal_epilogue_fwd(gd(), et(D=None), None) == L.PAL_E_NULL                  # x without D
+    assert lib.pal_epilogue_fwd(gd(), et(o=_fake(0x1008)), None) == L.PAL_E_ALIGN
+    eg = L.PalEpilogueGrads(**{n: _fake(0x1000 * (i + 40)) for i, n in enumerate(("dy", "d_o", "dx", "dgate", "dD", "dweight"))})
+    assert lib.pal_epilogue_bwd(gd(), et(), None, None, 0, None) == L.PAL_E_NULL
+    assert lib.pal_epilogue_bwd(gd(), et(), L.PalEpilogueGrads(dy=_fake(), d_o=_fake(0x2000), dweight=_fake(0x3000)), None, 0,
+                                None) == L.PAL_E_NULL                                    # dx / dD / dgate missing
+    assert lib.pal_epilogue_bwd(gd(), et(), eg, None, 0, None) == L.PAL_E_WORKSPACE
+    assert lib.pal_epilogue_bwd_workspace_bytes(gd()) > 0
