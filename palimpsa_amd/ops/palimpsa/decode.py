@@ -25,10 +25,12 @@ class DecodeStep:
 
     ``rows_dtype`` is the dtype of q, k, v, b (bf16 or fp32); gt, g, Ip and the states are fp32.
     ``dk`` must be one of the head dims the token-serial kernel is compiled for and ``dv`` a
-    multiple of 16 (no padding here: a server lays its state out once)."""
+    multiple of 16 (no padding here: a server lays its state out once).  ``tokens`` > 1 makes a step
+    consume that many tokens per sequence (blocked or speculative decode): the state stays in registers
+    over the block and is read and written once."""
 
     def __init__(self, B: int, H: int, dk: int, dv: int, device, rows_dtype=torch.bfloat16,
-                 scale: Optional[float] = None, output_uncertainty: bool = False):
+                 scale: Optional[float] = None, output_uncertainty: bool = False, tokens: int = 1):
         dev = torch.device(device)
         if dev.type != "cuda":
             raise RuntimeError("palimpsa_amd runs on an AMD GPU only; there is no CPU fallback")
@@ -38,16 +40,19 @@ class DecodeStep:
             raise ValueError(f"dk must be one of {L.RECURRENT_DK} and dv a multiple of 16; got dk={dk}, dv={dv}")
         if rows_dtype not in (torch.bfloat16, torch.float32):
             raise ValueError("rows_dtype must be torch.bfloat16 or torch.float32")
+        if not isinstance(tokens, int) or tokens < 1:
+            raise ValueError(f"tokens must be a positive int, got {tokens!r}")
+        self.tokens = tokens
         self.B, self.H, self.dk, self.dv, self.device, self.rows_dtype = B, H, dk, dv, dev, rows_dtype
-        self.o = torch.empty(B, 1, H, dv, dtype=rows_dtype, device=dev)
-        self.o_var = torch.empty(B, 1, H, dv, dtype=torch.float32, device=dev) if output_uncertainty else None
+        self.o = torch.empty(B, tokens, H, dv, dtype=rows_dtype, device=dev)
+        self.o_var = torch.empty(B, tokens, H, dv, dtype=torch.float32, device=dev) if output_uncertainty else None
         flags = L.PAL_FLAG_HAS_INIT | L.PAL_FLAG_STORE_FINAL | (L.PAL_FLAG_HAS_VAR if output_uncertainty else 0)
-        self._dims = L.PalDims(batch=B, seq_len=1, n_seqs=B, n_heads=H, dk=dk, dv=dv, total_chunks=0,
+        self._dims = L.PalDims(batch=B, seq_len=tokens, n_seqs=B, n_heads=H, dk=dk, dv=dv, total_chunks=0,
                                dtype=cm._pal_dtype(rows_dtype), gate_dtype=L.PAL_DTYPE_F32, var_dtype=L.PAL_DTYPE_F32,
                                flags=flags, scale=float(dk ** -0.5 if scale is None else scale))
         self._tens = L.PalFwdTensors(o=cm._ptr(self.o), o_var=cm._ptr(self.o_var))
         self._fn = L.load().pal_recurrent_fwd
-        self._row_shape = (B, 1, H)
+        self._row_shape = (B, tokens, H)
 
     def _check(self, name, x, shape, dtype):
         if tuple(x.shape) != shape or x.dtype != dtype or x.device != self.device or not x.is_contiguous():
@@ -76,11 +81,12 @@ class DecodeStep:
         return self
 
     def step(self, stream: Optional[int] = None) -> torch.Tensor:
-        """One token for every sequence from the bound tensors; returns the (reused) output buffer
-        ``[B,1,H,dv]``.  ``stream`` is a raw HIP stream handle; default: torch's current stream."""
+        """One token (``tokens`` of them) for every sequence from the bound tensors; returns the (reused) output
+        buffer ``[B,tokens,H,dv]``.  ``stream`` is a raw HIP stream handle; default: torch's current stream."""
         if stream is None:
-            stream = torch.cuda.current_stream(self.device).cuda_stream
-        rc = self._fn(self._dims, self._tens, C.c_void_p(stream))
+            rc = self._fn(self._dims, self._tens, cm.current_stream_ptr(self.device))
+        else:
+            rc = self._fn(self._dims, self._tens, C.c_void_p(stream))
         if rc:
             L.check(rc, "pal_recurrent_fwd")
         return self.o

@@ -277,3 +277,39 @@ def test_bound_decode_step_matches_entry_point_and_replays_in_a_graph(gpu_device
         dec.bind(buf["q"].float(), buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"], mu_b, I_b)
     with pytest.raises(ValueError):
         DecodeStep(B, H, 40, dv, dev)
+
+
+def test_bound_decode_step_with_several_tokens_per_step(gpu_device):
+    """A bound step over blocks of 3 tokens equals the same tokens one at a time (state in place)."""
+    from palimpsa_amd.ops.palimpsa import DecodeStep
+    B, H, dk, dv, blocks, k = 4, 2, 32, 48, 3, 3
+    dev = gpu_device
+    inp = hp.rounded(po.make_inputs(B, blocks * k, H, dk, dv, seed=71), torch.bfloat16)
+    d = hp.to_device(inp, dev)
+    gen = torch.Generator().manual_seed(72)
+    mu0 = (torch.randn(B, H, dv, dk, generator=gen) * 0.1).to(dev)
+    I0 = (1.0 + torch.rand(B, H, dv, dk, generator=gen)).to(dev)
+
+    def run(tokens):
+        dec = DecodeStep(B, H, dk, dv, dev, torch.bfloat16, tokens=tokens)
+        buf = {n: torch.empty_like(d[n][:, :tokens].contiguous()) for n in ("q", "k", "v", "b", "gt")}
+        mu, I = mu0.clone(), I0.clone()
+        dec.bind(buf["q"], buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"], mu, I)
+        outs = []
+        for t in range(0, blocks * k, tokens):
+            for n in buf:
+                buf[n].copy_(d[n][:, t:t + tokens])
+            outs.append(dec.step().clone())
+        return torch.cat(outs, dim=1), mu, I
+
+    o1, mu1, I1 = run(1)
+    o3, mu3, I3 = run(k)
+    assert o3.shape == (B, blocks * k, H, dv)
+    # inside a block the state stays in registers as (M, J); between single steps it crosses as (mu, I)
+    assert hp.max_abs(o3.float(), o1.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu3, mu1) <= 1e-5 and hp.max_rel(I3, I1) <= 1e-5
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0.cpu(), I0=I0.cpu())
+    assert hp.max_abs(o3.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu3, mu_ref) <= hp.FP32_REL_TOL and hp.max_rel(I3, I_ref) <= hp.FP32_REL_TOL
+    with pytest.raises(ValueError):
+        DecodeStep(B, H, dk, dv, dev, tokens=0)
