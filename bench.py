@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla] [--no-layer-slice]
 
 Headline workload (the metric's own configuration): chunked forward+backward at
-B=8, T=2048, H=12, dk=dv=64, bf16 rows, fp32 gates/states, 64-token tiles,
+B=8, T=2048, H=12, dk=dv=64, bf16 rows and gates (--gates fp32: fp32 gates), fp32 states, 64-token tiles,
 synthetic seeded inputs, timed through the public entry point
 (palimpsa_amd.ops.palimpsa.chunk_palimpsa + autograd), inputs resident in HBM.
 One JSON line is printed; it also carries
@@ -50,12 +50,14 @@ def make_inputs(torch, B, T, H, dk, dv, seed, dtype):
                 g=torch.ones(H), Ip=torch.ones(H))
 
 
-def bench_chunk(torch, dev, steps, warmup):
+def bench_chunk(torch, dev, steps, warmup, gates="bf16"):
     from palimpsa_amd import _lib as L
     from palimpsa_amd.ops.palimpsa import chunk_palimpsa
 
     B, T, H, d = 8, 2048, 12, 64
     inp = make_inputs(torch, B, T, H, d, d, 0, torch.bfloat16)
+    if gates == "bf16":     # the benchmark configuration stores the per-token gates in bf16 like the rows
+        inp["gt"] = inp["gt"].to(torch.bfloat16)
     leaves = {n: inp[n].to(dev).requires_grad_(True) for n in ("q", "k", "v", "b", "gt", "g", "Ip")}
     do = torch.randn(B, T, H, d, generator=torch.Generator().manual_seed(1)).to(dev, torch.bfloat16)
 
@@ -114,7 +116,7 @@ def bench_chunk(torch, dev, steps, warmup):
     kernels = {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()}
     return dict(value=tokens / (ms_per_step * 1e-3), ms_per_step=ms_per_step, ms_per_step_no_events=ms_plain,
                 roofline=roofline, kernels=kernels,
-                config={"workload": "c1: chunked fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates C=64",
+                config={"workload": f"c1: chunked fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows {gates} gates fp32 states C=64",
                         "B": B, "T": T, "H": H, "dk": d, "dv": d, "chunk": CHUNK})
 
 
@@ -330,6 +332,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--decode-steps", type=int, default=1024)
+    ap.add_argument("--gates", choices=("bf16", "fp32"), default="bf16",
+                    help="element type of the per-token gate tensor gt of the headline workload (the reference layer "
+                         "passes fp32; the benchmark configuration says bf16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-simple-gla", action="store_true")
@@ -356,7 +361,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    res = bench_chunk(torch, dev, args.steps, args.warmup)
+    res = bench_chunk(torch, dev, args.steps, args.warmup, args.gates)
     extra = {"kernels": res["kernels"], "ms_per_step_no_events": res["ms_per_step_no_events"]}
     if not args.no_decode:
         extra["decode"] = bench_decode(torch, dev, args.decode_steps)
