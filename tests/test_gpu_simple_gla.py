@@ -458,3 +458,24 @@ def test_random_shape_sweep(gpu_device):
         assert hp.max_rel(S, S_ref.detach()) <= 1e-2, tag
         for name, x, r in zip(("q", "k", "v", "g", "S0"), leaves, ref):
             assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, (name,) + tag
+
+
+def test_prefill_then_decode(gpu_device):
+    """Serving flow: chunked prefill returns the state in the cache's [N,H,dk,dv] layout, single-token decode steps
+    continue from it; the outputs equal those of one pass over the whole sequence."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    B, T0, T1, H, dk, dv = 2, 150, 6, 2, 64, 96
+    q, k, v, g, _ = _inputs(B, T0 + T1, H, dk, dv, 71)
+    dev = gpu_device
+    qd, kd, vd, gd = (x.to(dev) for x in (q, k, v, g))
+    with torch.no_grad():
+        o0, S = chunk_simple_gla(q=qd[:, :T0], k=kd[:, :T0], v=vd[:, :T0], g=gd[:, :T0], output_final_state=True)
+        outs = [o0]
+        for t in range(T0, T0 + T1):
+            o, S = fused_recurrent_simple_gla(q=qd[:, t:t + 1], k=kd[:, t:t + 1], v=vd[:, t:t + 1], g=gd[:, t:t + 1],
+                                              initial_state=S, output_final_state=True)
+            outs.append(o)
+    o_all = torch.cat(outs, dim=1)
+    o_ref, S_ref = _closed_form(q, k, v, g, dk ** -0.5)
+    assert hp.max_abs(o_all.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_ref) <= 1e-2
