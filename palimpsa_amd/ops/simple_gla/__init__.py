@@ -31,7 +31,7 @@ from ..palimpsa import _common as cm
 from ..palimpsa import chunk_palimpsa, fused_recurrent_palimpsa
 from ..palimpsa.chunk import _chunk_meta, _count_chunks
 
-__all__ = ["chunk_simple_gla", "fused_recurrent_simple_gla"]
+__all__ = ["chunk_simple_gla", "fused_recurrent_simple_gla", "ChunkSimpleGLA", "SimpleGlaDecodeStep"]
 
 
 _RATE_CACHE: dict = {}
@@ -221,3 +221,62 @@ def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
     if final is not None and (p.dk_p != p.dk or p.dv_p != p.dv):
         final = final[:, :, :p.dk, :p.dv].contiguous()
     return o, final
+
+
+class SimpleGlaDecodeStep:
+    """Bound decode step of the path without the precision state (the counterpart of
+    ``palimpsa_amd.ops.palimpsa.DecodeStep``): shapes and dtypes are checked once in ``bind``, ``step`` only issues
+    ``pal_gla_recurrent_fwd`` on the current stream.  The state ``S`` ``[B, H, dk, dv]`` fp32 is updated in place, the
+    output buffer is reused and nothing is allocated per step, so a step can be recorded into a HIP graph.
+    ``dk`` and ``dv`` must be multiples of 16; ``tokens`` > 1 takes that many tokens per sequence and step."""
+
+    def __init__(self, B: int, H: int, dk: int, dv: int, device, rows_dtype=torch.bfloat16,
+                 scale: Optional[float] = None, tokens: int = 1):
+        dev = torch.device(device)
+        if dev.type != "cuda":
+            raise RuntimeError("palimpsa_amd runs on an AMD GPU only; there is no CPU fallback")
+        if dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        if dk % 16 or dv % 16 or not (16 <= dk <= 256 and 16 <= dv <= 256):
+            raise ValueError(f"dk and dv must be multiples of 16 in [16, 256]; got dk={dk}, dv={dv}")
+        if rows_dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("rows_dtype must be torch.bfloat16 or torch.float32")
+        if not isinstance(tokens, int) or tokens < 1:
+            raise ValueError(f"tokens must be a positive int, got {tokens!r}")
+        self.B, self.H, self.dk, self.dv, self.device, self.rows_dtype, self.tokens = B, H, dk, dv, dev, rows_dtype, tokens
+        self.o = torch.empty(B, tokens, H, dv, dtype=rows_dtype, device=dev)
+        self._rate = _minus_one_rate(H, dev)
+        self._dims = L.PalDims(batch=B, seq_len=tokens, n_seqs=B, n_heads=H, dk=dk, dv=dv, total_chunks=0,
+                               dtype=cm._pal_dtype(rows_dtype), gate_dtype=L.PAL_DTYPE_F32, var_dtype=L.PAL_DTYPE_F32,
+                               flags=L.PAL_FLAG_HAS_INIT | L.PAL_FLAG_STORE_FINAL,
+                               scale=float(dk ** -0.5 if scale is None else scale))
+        self._tens = L.PalFwdTensors(o=cm._ptr(self.o), g=cm._ptr(self._rate))
+        self._fn = L.load().pal_gla_recurrent_fwd
+
+    def _check(self, name, x, shape, dtype):
+        if tuple(x.shape) != shape or x.dtype != dtype or x.device != self.device or not x.is_contiguous():
+            raise ValueError(f"{name}: expected contiguous {dtype} {shape} on {self.device}, "
+                             f"got {x.dtype} {tuple(x.shape)} on {x.device}")
+
+    def bind(self, q, k, v, g, S) -> "SimpleGlaDecodeStep":
+        """Check the tensors once and remember their addresses (q, k ``[B,tokens,H,dk]``, v ``[B,tokens,H,dv]``, g fp32
+        ``[B,tokens,H]``, S fp32 ``[B,H,dk,dv]``); write the next tokens' rows into the same tensors before each step."""
+        rs = (self.B, self.tokens, self.H)
+        self._check("q", q, rs + (self.dk,), self.rows_dtype)
+        self._check("k", k, rs + (self.dk,), self.rows_dtype)
+        self._check("v", v, rs + (self.dv,), self.rows_dtype)
+        self._check("g", g, rs, torch.float32)
+        self._check("S", S, (self.B, self.H, self.dk, self.dv), torch.float32)
+        t = self._tens
+        t.q, t.k, t.v, t.gt = q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr()
+        t.init_mu = t.final_mu = S.data_ptr()
+        self._keep = (q, k, v, g, S)
+        return self
+
+    def step(self, stream: Optional[int] = None) -> torch.Tensor:
+        """Advance every sequence by ``tokens`` tokens; returns the (reused) output buffer ``[B,tokens,H,dv]``."""
+        sp = cm.current_stream_ptr(self.device) if stream is None else C.c_void_p(stream)
+        rc = self._fn(self._dims, self._tens, sp)
+        if rc:
+            L.check(rc, "pal_gla_recurrent_fwd")
+        return self.o

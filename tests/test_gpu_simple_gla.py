@@ -479,3 +479,65 @@ def test_prefill_then_decode(gpu_device):
     o_ref, S_ref = _closed_form(q, k, v, g, dk ** -0.5)
     assert hp.max_abs(o_all.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_rel(S, S_ref) <= 1e-2
+
+
+def test_bound_decode_step_and_graph_replay(gpu_device):
+    """SimpleGlaDecodeStep: same kernel as fused_recurrent_simple_gla, so results agree exactly; recorded into a HIP
+    graph, every replay (with eager work in between) agrees with the eager result too."""
+    from palimpsa_amd.ops.simple_gla import SimpleGlaDecodeStep, fused_recurrent_simple_gla
+    B, H, dk, dv, steps = 5, 3, 64, 48, 6
+    q, k, v, g, S0 = _inputs(B, steps, H, dk, dv, 81)
+    dev = gpu_device
+    qd, kd, vd, gd = (x.to(dev) for x in (q, k, v, g))
+    S = S0.to(dev)
+    outs = []
+    with torch.no_grad():
+        for t in range(steps):
+            o, S = fused_recurrent_simple_gla(q=qd[:, t:t + 1], k=kd[:, t:t + 1], v=vd[:, t:t + 1], g=gd[:, t:t + 1],
+                                              initial_state=S, output_final_state=True)
+            outs.append(o)
+    dec = SimpleGlaDecodeStep(B, H, dk, dv, dev)
+    buf = [torch.empty_like(x[:, :1].contiguous()) for x in (qd, kd, vd, gd)]
+    Sb = S0.to(dev).clone()
+    dec.bind(buf[0], buf[1], buf[2], buf[3], Sb)
+    for t in range(steps):
+        for b_, x in zip(buf, (qd, kd, vd, gd)):
+            b_.copy_(x[:, t:t + 1])
+        assert torch.equal(dec.step(), outs[t])
+    assert torch.equal(Sb, S)
+    # graph
+    Sb.copy_(S0.to(dev))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        dec.step()
+        Sb.copy_(S0.to(dev))
+        with torch.cuda.graph(graph, stream=side):
+            dec.step()
+    torch.cuda.current_stream().wait_stream(side)
+    for t in range(steps):
+        for b_, x in zip(buf, (qd, kd, vd, gd)):
+            b_.copy_(x[:, t:t + 1])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dec.o, outs[t]), t
+    assert torch.equal(Sb, S)
+    # blocks of three tokens against the closed form
+    dec3 = SimpleGlaDecodeStep(B, H, dk, dv, dev, tokens=3)
+    buf3 = [torch.empty_like(x[:, :3].contiguous()) for x in (qd, kd, vd, gd)]
+    S3 = S0.to(dev).clone()
+    dec3.bind(buf3[0], buf3[1], buf3[2], buf3[3], S3)
+    o3 = []
+    for t in range(0, steps, 3):
+        for b_, x in zip(buf3, (qd, kd, vd, gd)):
+            b_.copy_(x[:, t:t + 3])
+        o3.append(dec3.step().clone())
+    o_ref, S_ref = _closed_form(q, k, v, g, dk ** -0.5, S0)
+    assert hp.max_abs(torch.cat(o3, dim=1).float(), o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S3, S_ref) <= hp.FP32_REL_TOL
+    with pytest.raises(ValueError):
+        dec.bind(buf[0].float(), buf[1], buf[2], buf[3], Sb)
+    with pytest.raises(ValueError):
+        SimpleGlaDecodeStep(B, H, 40, dv, dev)
