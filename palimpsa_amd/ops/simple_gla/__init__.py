@@ -167,6 +167,7 @@ def _check_chunk_args(q, g, cu_seqlens):
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
     if g.shape != q.shape[:3]:
         raise ValueError(f"g must have shape {tuple(q.shape[:3])}, got {tuple(g.shape)}")
+    cm._require_gpu(q, g)
     if cu_seqlens is not None and q.shape[0] != 1:
         raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
 

@@ -125,3 +125,24 @@ def test_simple_gla_wrappers_keep_the_layer_call_site_keywords():
             fn(q=x, k=x, v=x, g=None)
         with pytest.raises(ValueError):
             fn(q=x, k=x, v=x, g=torch.zeros(1, 4, 3))
+
+
+def test_no_cpu_fallback_anywhere():
+    """Every entry point of the package refuses CPU tensors instead of computing something on the host."""
+    import pytest
+    import torch
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs, palimpsa_output_norm
+    from palimpsa_amd.ops.palimpsa import DecodeStep
+    from palimpsa_amd.ops.simple_gla import SimpleGlaDecodeStep, chunk_simple_gla, fused_recurrent_simple_gla
+    x = torch.zeros(1, 4, 2, 16)
+    g = torch.zeros(1, 4, 2)
+    for fn in (chunk_simple_gla, fused_recurrent_simple_gla):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            fn(q=x, k=x, v=x, g=g)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        palimpsa_inputs(x, x, x, g, torch.zeros(2), g, x, torch.zeros(2))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        palimpsa_output_norm(x, x, torch.zeros(2), x, torch.ones(16), 1e-6)
+    for cls in (DecodeStep, SimpleGlaDecodeStep):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            cls(1, 2, 16, 16, "cpu")
