@@ -245,3 +245,12 @@ def test_layer_glue_entry_points_reject_bad_arguments(L):
                                 None) == L.PAL_E_NULL                                    # dx / dD / dgate missing
     assert lib.pal_epilogue_bwd(gd(), et(), eg, None, 0, None) == L.PAL_E_WORKSPACE
     assert lib.pal_epilogue_bwd_workspace_bytes(gd()) > 0
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    """Without the built library the package raises ImportError with the build instruction; nothing is computed."""
+    from palimpsa_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libpalimpsa_hip.so"))
+    with pytest.raises(ImportError, match="palimpsa_amd.build"):
+        _lib.load()
