@@ -205,3 +205,41 @@ def test_random_shape_sweep(gpu_device):
         lo.epilogue(*rv, 1e-5).backward(dy.double())
         for name, t, r in zip(("o", "x", "D", "gate", "weight"), lv, rv):
             assert hp.max_rel(t.grad, r.grad) <= grad_tol, (name,) + tag
+
+
+def test_full_size_headline_shape(gpu_device):
+    """Both glue kernels at the headline shape (B=8, T=2048, H=12, d=64, bf16), forward and backward against the
+    oracle; the per-head and per-column sums of the backward run over 16384 tokens per head."""
+    from palimpsa_amd.ops.layer_glue import palimpsa_inputs, palimpsa_output_norm
+    lead, H, d = (8, 2048), 12, 64
+    a = _inputs(lead, H, H, d, d, 7, torch.bfloat16)
+    dev = gpu_device
+    leaves = {n: a[n].to(dev).clone().requires_grad_(True) for n in NAMES}
+    outs = palimpsa_inputs(**leaves)
+    refl = {n: a[n].double().clone().requires_grad_(True) for n in NAMES}
+    refs = lo.prologue(**refl, model_dtype=torch.bfloat16)
+    gen = torch.Generator().manual_seed(8)
+    loss = loss_ref = 0.0
+    for y, r in zip(outs, refs):
+        assert hp.max_abs(y.float(), r) <= hp.BF16_OUT_ABS_TOL * max(1.0, r.abs().max().item())
+        wgt = torch.randn(r.shape, generator=gen).to(y.dtype)
+        loss = loss + (y.float() * wgt.to(dev).float()).sum()
+        loss_ref = loss_ref + (r * wgt.double()).sum()
+    loss.backward()
+    loss_ref.backward()
+    for n in NAMES:
+        assert hp.max_rel(leaves[n].grad, refl[n].grad) <= hp.BF16_GRAD_NORM_TOL, n
+    o = torch.randn(*lead, H, d, generator=gen).bfloat16()
+    gate = torch.randn(*lead, H, d, generator=gen).bfloat16()
+    Dp, w = torch.randn(H, generator=gen), 1.0 + 0.2 * torch.randn(d, generator=gen)
+    dy = torch.randn(*lead, H, d, generator=gen).bfloat16()
+    ts = [o, a["x"], Dp, gate, w]
+    lv = [t.to(dev).clone().requires_grad_(True) for t in ts]
+    y = palimpsa_output_norm(*lv, 1e-6)
+    y.backward(dy.to(dev))
+    rv = [t.double().clone().requires_grad_(True) for t in ts]
+    y_ref = lo.epilogue(*rv, 1e-6)
+    y_ref.backward(dy.double())
+    assert hp.max_abs(y.float(), y_ref.detach()) <= hp.BF16_OUT_ABS_TOL * max(1.0, y_ref.abs().max().item())
+    for name, t, r in zip(("o", "x", "D", "gate", "weight"), lv, rv):
+        assert hp.max_rel(t.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
