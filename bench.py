@@ -35,7 +35,9 @@ CHUNK = 64
 # HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
 # from inside this process, so the figures are carried here and are stale once those kernels change.
-MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 506.3e6, "recurrent_fwd_kernel": 1111.9e6}
+MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 506.3e6, "recurrent_fwd_kernel": 1111.9e6,
+                          # profiles/bench_simple_gla__layer_slice.hbm_traffic_pmc.txt
+                          "gla_out_kernel": 141.5e6, "gla_recurrent_fwd_kernel": 543.4e6, "prologue_bwd_kernel": 304.6e6}
 
 
 def make_inputs(torch, B, T, H, dk, dv, seed, dtype):
@@ -231,13 +233,14 @@ def bench_simple_gla(torch, dev, steps, warmup):
     decode = {"workload": "fused_recurrent_simple_gla B=256 H=16 dk=dv=128, single-token steps, state fed back",
               "tokens_per_s": Bd * dsteps / d_elapsed, "ms_per_step": d_elapsed * 1e3 / dsteps,
               "roofline": {"bound": "hbm", "kernel": "gla_recurrent_fwd_kernel", "achieved": dec_gbs, "peak": PEAK_HBM_GBS,
-                           "unit": "GB/s", "frac": dec_gbs / PEAK_HBM_GBS, "traffic": None,
+                           "unit": "GB/s", "frac": dec_gbs / PEAK_HBM_GBS,
+                           "traffic": MEASURED_TRAFFIC_BYTES["gla_recurrent_fwd_kernel"],
                            "algorithmic_bytes_per_launch": bytes_dec, "avg_launch_ms": dk_ms / max(dk_n, 1)}}
     return {"workload": "chunk_simple_gla fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates", "decode": decode,
             "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms, "kernel_ms_per_step": sum(v[0] for v in kern.values()) / steps,
             "kernels": kernels,
             "roofline": {"bound": "hbm", "kernel": "gla_out_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
-                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES["gla_out_kernel"],
                          "algorithmic_bytes_per_launch": bytes_out, "avg_launch_ms": avg_out_ms}}
 
 
@@ -299,7 +302,8 @@ def bench_layer_slice(torch, dev, steps, warmup):
             "glue_kernel_ms_per_step": sum(kern[k][0] for k in glue if k in kern) / steps,
             "kernels": {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()},
             "roofline": {"bound": "hbm", "kernel": "prologue_bwd_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
-                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                         "traffic": MEASURED_TRAFFIC_BYTES["prologue_bwd_kernel"],
                          "algorithmic_bytes_per_launch": bytes_pb, "avg_launch_ms": avg_pb}}
 
 
