@@ -41,7 +41,8 @@ struct GlaTileArgs {
   const bf16_t* St;       // per-tile states [tile][H][dv][dk], bf16
   void* out;              // rows [token][H][de]
   const void* W;          // optional rows [token][H][de]: dot[token] = sum_e W out (fp32, before rounding)
-  float* dot;             // [token][H] or null
+  float* dot;             // [H][tokens] (head-major, so that the gate kernel reads contiguous rows) or null
+  int64_t n_tokens;       // tokens in the batch (row length of dot)
   int32_t dc, de;         // contraction width of the scores, width of the output rows
 };
 
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
     }
   }
   if (has_dot && w == 0 && lane < clen)
-    A.dot[(int64_t)(t0 + lane) * H + h] = (sDot[lane] + sDot[kC + lane]) + (sDot[2 * kC + lane] + sDot[3 * kC + lane]);
+    A.dot[(int64_t)h * A.n_tokens + t0 + lane] = (sDot[lane] + sDot[kC + lane]) + (sDot[2 * kC + lane] + sDot[3 * kC + lane]);
   __syncthreads();
   {
     constexpr int VEC = 16 / (int)sizeof(TIn);   // elements per 16-byte access
@@ -433,7 +434,7 @@ constexpr int kGateTok = 4;                    // consecutive tokens per thread
 constexpr int kGatePiece = 256 * kGateTok;     // tokens per step of a workgroup
 
 __global__ __launch_bounds__(256) void gla_bwd_gate_kernel(ChunkArgs a, const float* qdq, const float* kdk, float* dgt,
-                                                           float* dg_part) {
+                                                           float* dg_part, int64_t n_tokens) {
   __shared__ float sTot[2][4];
   __shared__ float sAcc[4];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -448,7 +449,7 @@ __global__ __launch_bounds__(256) void gla_bwd_gate_kernel(ChunkArgs a, const fl
     float x[kGateTok];
 #pragma unroll
     for (int j = 0; j < kGateTok; ++j) {
-      const int64_t off = (int64_t)(bos + tf + j) * a.H + h;
+      const int64_t off = (int64_t)h * n_tokens + bos + tf + j;      // the dot products are stored head-major
       x[j] = (tf + j < len) ? qdq[off] - kdk[off] : 0.f;
     }
     // suffix sums inside the thread, then over the lanes of the wave (exclusive of the thread itself)
@@ -559,6 +560,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   }
   GlaTileArgs A{};
   A.c = a;
+  A.n_tokens = (int64_t)d->batch * d->seq_len;
   // dq: X = dO, Y = v, Z = k, tile-start states read transposed; q . dq on the side
   A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = (const bf16_t*)t->chunk_I; A.out = gr->dq; A.W = t->q; A.dot = qdq;
   A.dc = d->dv; A.de = d->dk;
@@ -574,7 +576,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   {
     const int64_t blocks = (int64_t)d->n_seqs * d->n_heads;
     PAL_TIMED_LAUNCH(kKernGlaBwdGate, s, gla_bwd_gate_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, qdq, kdk, gr->dgt,
-                     dg_part);
+                     dg_part, (int64_t)d->batch * d->seq_len);
     PAL_HIP_LAUNCH_CHECK();
     hipLaunchKernelGGL(gla_bwd_head_reduce_kernel, dim3((d->n_heads + 63) / 64), dim3(64), 0, s, dg_part, gr->dg,
                        d->n_seqs, d->n_heads);
