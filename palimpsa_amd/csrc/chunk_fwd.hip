@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
 
 // ------------------------------------------------------------------ kernel 1b
 // Serial part of the forward: S_c = F_c S_{c-1} + Delta_c per state entry, fp32, pure streaming.
-// One thread per (sequence, head, state entry), 256 consecutive entries per block.  Each slot of
+// One thread per four consecutive state entries of a (sequence, head), 1024 entries per block.  Each slot of
 // chunk_mu / chunk_I is overwritten with the state at the START of its tile in (mu, I) form
 // (what the reference stores as intermediate_*_state, chunk_palimpsa_forgetting_scalar.py:187-188);
 // the state after the last tile goes to final_mu / final_I (:214-218).
@@ -163,23 +163,37 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
   __shared__ float sF[kScanTiles];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t E = (int64_t)a.dv * a.dk;
-  const int nblk = (int)(E / 256);
+  const int nblk = (int)((E + 1023) / 1024);     // four consecutive entries per thread
   const int blk = blockIdx.x % nblk;
   const int nh = blockIdx.x / nblk;
   const int h = nh % a.H, n = nh / a.H;
-  const int64_t e = (int64_t)blk * 256 + tid;
+  const int64_t e = ((int64_t)blk * 256 + tid) * 4;
+  const bool on = e < E;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const int nchunks = (len + kC - 1) / kC;
   const float Ip = a.Ip[h];
   const float gh = a.g[h] * kLog2e;
-  float SM = 0.f, SJ = 0.f;
+  f32x4 SM = {0.f, 0.f, 0.f, 0.f}, SJ = {0.f, 0.f, 0.f, 0.f};
   const int64_t so = (int64_t)nh * E + e;
-  if (a.init_mu) {
-    const float mu = a.init_mu[so], I = a.init_I[so];
-    SM = mu * I;
-    SJ = I - Ip;
+  if (a.init_mu && on) {
+    const f32x4 mu = *(const f32x4*)(a.init_mu + so), I = *(const f32x4*)(a.init_I + so);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) { SM[x] = mu[x] * I[x]; SJ[x] = I[x] - Ip; }
   }
+  // the slot of a tile: its Delta is read, the state at its start (mu, I) written, the state advanced
+  auto advance = [&](int64_t off, const f32x4& dM, const f32x4& dJ, float F) {
+    f32x4 mu, I;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      I[x] = SJ[x] + Ip;
+      mu[x] = SM[x] * fast_rcp(I[x]);
+      SM[x] = fmaf(F, SM[x], dM[x]);
+      SJ[x] = fmaf(F, SJ[x], dJ[x]);
+    }
+    *(f32x4*)(a.chunk_mu + off) = mu;
+    *(f32x4*)(a.chunk_I + off) = I;
+  };
   for (int c0 = 0; c0 < nchunks; c0 += kScanTiles) {
     const int cn = min(kScanTiles, nchunks - c0);
     __syncthreads();
@@ -190,41 +204,31 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(ChunkArgs a) {
       if (lane == 0) sF[c] = fast_exp2(tot);
     }
     __syncthreads();
+    if (!on) continue;
     int c = 0;
     for (; c + 4 <= cn; c += 4) {
-      float dM[4], dJ[4];
+      f32x4 dM[4], dJ[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t off = ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e;
-        dM[u] = a.chunk_mu[off];
-        dJ[u] = a.chunk_I[off];
+        dM[u] = *(const f32x4*)(a.chunk_mu + off);
+        dJ[u] = *(const f32x4*)(a.chunk_I + off);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int64_t off = ((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e;
-        const float I = SJ + Ip;
-        a.chunk_mu[off] = SM * fast_rcp(I);
-        a.chunk_I[off] = I;
-        const float F = sF[c + u];
-        SM = fmaf(F, SM, dM[u]);
-        SJ = fmaf(F, SJ, dJ[u]);
-      }
+      for (int u = 0; u < 4; ++u) advance(((int64_t)(cbase + c0 + c + u) * a.H + h) * E + e, dM[u], dJ[u], sF[c + u]);
     }
     for (; c < cn; ++c) {
       const int64_t off = ((int64_t)(cbase + c0 + c) * a.H + h) * E + e;
-      const float dM = a.chunk_mu[off], dJ = a.chunk_I[off];
-      const float I = SJ + Ip;
-      a.chunk_mu[off] = SM * fast_rcp(I);
-      a.chunk_I[off] = I;
-      const float F = sF[c];
-      SM = fmaf(F, SM, dM);
-      SJ = fmaf(F, SJ, dJ);
+      const f32x4 dM = *(const f32x4*)(a.chunk_mu + off), dJ = *(const f32x4*)(a.chunk_I + off);
+      advance(off, dM, dJ, sF[c]);
     }
   }
-  if (a.final_mu) {
-    const float I = SJ + Ip;
-    a.final_mu[so] = SM * fast_rcp(I);
-    a.final_I[so] = I;
+  if (a.final_mu && on) {
+    f32x4 mu, I;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) { I[x] = SJ[x] + Ip; mu[x] = SM[x] * fast_rcp(I[x]); }
+    *(f32x4*)(a.final_mu + so) = mu;
+    *(f32x4*)(a.final_I + so) = I;
   }
 }
 
@@ -595,7 +599,7 @@ int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s)
   if (int rc = launch_tile_delta(a, dtype, has_j, s)) return rc;
   {
     const int64_t E = (int64_t)a.dv * a.dk;
-    const int64_t blocks = (int64_t)a.n_seqs * a.H * (has_j ? E / 256 : (E + 1023) / 1024);
+    const int64_t blocks = (int64_t)a.n_seqs * a.H * ((E + 1023) / 1024);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
     if (has_j) PAL_TIMED_LAUNCH(kKernChunkScan, s, chunk_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
     else PAL_TIMED_LAUNCH(kKernChunkScan, s, gla_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
