@@ -541,3 +541,32 @@ def test_bound_decode_step_and_graph_replay(gpu_device):
         dec.bind(buf[0].float(), buf[1], buf[2], buf[3], Sb)
     with pytest.raises(ValueError):
         SimpleGlaDecodeStep(B, H, 40, dv, dev)
+
+
+def test_packed_pretraining_batch_full_size(gpu_device):
+    """The packed-batch benchmark shape (32768 tokens in 23 documents, H=16, d=96) on the path without the precision
+    state: forward against the token-serial kernel, gradients against the Palimpsa kernels on b = 0, Ip = 1."""
+    from oracle import palimpsa_oracle as po
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    cu = po.make_varlen_lengths(32768, seed=0)
+    T, H, d = cu[-1], 16, 96
+    q, k, v, g, _ = _inputs(1, T, H, d, d, 91)
+    gen = torch.Generator().manual_seed(92)
+    do = torch.randn(1, T, H, d, generator=gen).bfloat16()
+    dev = gpu_device
+    cu_d = torch.tensor(cu, device=dev, dtype=torch.int32)
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    o, S = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], output_final_state=True, cu_seqlens=cu_d)
+    o.backward(do.to(dev))
+    with torch.no_grad():
+        o_r, S_r = fused_recurrent_simple_gla(q=q.to(dev), k=k.to(dev), v=v.to(dev), g=g.to(dev), output_final_state=True,
+                                              cu_seqlens=cu_d)
+    assert hp.max_abs(o.float(), o_r.float()) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(S, S_r) <= 1e-2
+    ref = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    ones = torch.ones(H, device=dev)
+    o_p = chunk_palimpsa(ref[0], ref[1], ref[2], torch.zeros_like(ref[2]), -ref[3], ones, ones, cu_seqlens=cu_d)
+    o_p.backward(do.to(dev))
+    for name, x, r in zip(("q", "k", "v", "g"), leaves, ref):
+        assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
