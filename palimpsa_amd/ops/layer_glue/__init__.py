@@ -192,6 +192,7 @@ class PalimpsaOutputNorm(torch.autograd.Function):
                 None if dgate is None else dgate.to(dt[3]), dw.reshape(m["w_shape"]).to(dt[4]), None)
 
 
+@cm.no_compile
 def palimpsa_inputs(q_raw: torch.Tensor, k_raw: torch.Tensor, x: torch.Tensor, dt_raw: torch.Tensor,
                     dt_bias: torch.Tensor, bs_raw: torch.Tensor, b_raw: Optional[torch.Tensor] = None,
                     b_scale: Optional[torch.Tensor] = None, eps: float = 1e-12):
@@ -206,6 +207,7 @@ def palimpsa_inputs(q_raw: torch.Tensor, k_raw: torch.Tensor, x: torch.Tensor, d
     return PalimpsaInputs.apply(q_raw, k_raw, x, dt_raw, dt_bias, bs_raw, b_raw, b_scale, eps)
 
 
+@cm.no_compile
 def palimpsa_output_norm(o: torch.Tensor, x: Optional[torch.Tensor], D: Optional[torch.Tensor],
                          gate: Optional[torch.Tensor], weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
     """Residual and output norm of the layer (layers/palimpsa.py:337-343): ``rmsnorm(o + x * D) * weight``,

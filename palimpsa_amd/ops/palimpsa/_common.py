@@ -13,6 +13,13 @@ import torch.nn.functional as F
 from ... import _lib as L
 
 
+def no_compile(fn):
+    """Keep torch.compile from tracing into an entry point: the work happens in ctypes calls that a tracer cannot
+    follow, so the call is left as an opaque eager region (a graph break) instead of being probed and warned about."""
+    disable = getattr(getattr(torch, "compiler", None), "disable", None)
+    return disable(fn) if disable is not None else fn
+
+
 def _require_gpu(*tensors) -> torch.device:
     dev = tensors[0].device
     if dev.type != "cuda":

@@ -229,6 +229,7 @@ class ChunkPalimpsa(torch.autograd.Function):
                 None, None, None, None, None, None, None, None)
 
 
+@cm.no_compile
 def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state=None, scale=None,
                    chunk_size=16, output_final_state=False, output_uncertainty=False, cu_seqlens=None):
     """Chunked Palimpsa attention; calling convention of chunk_palimpsa in the reference

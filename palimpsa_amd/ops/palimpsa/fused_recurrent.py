@@ -129,6 +129,7 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
                 dIp.reshape(m["Ip_shape"]).to(dts[6]), None, d_init_mu, d_init_I, None, None, None)
 
 
+@cm.no_compile
 def fused_recurrent_palimpsa(
     q: torch.Tensor,
     k: torch.Tensor,

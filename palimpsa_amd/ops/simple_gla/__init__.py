@@ -172,6 +172,7 @@ def _check_chunk_args(q, g, cu_seqlens):
         raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
 
 
+@cm.no_compile
 def chunk_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optional[torch.Tensor] = None,
                      scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                      output_final_state: bool = False, cu_seqlens: Optional[torch.Tensor] = None):
@@ -182,6 +183,7 @@ def chunk_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optio
     return ChunkSimpleGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
 
 
+@cm.no_compile
 def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optional[torch.Tensor] = None,
                                scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                                output_final_state: bool = False, cu_seqlens: Optional[torch.Tensor] = None):

@@ -176,3 +176,25 @@ def test_largest_head_dims_forward(gpu_device, dk, dv):
     assert hp.max_abs(o.float(), o_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_abs(ov.float(), ov_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
+def test_entry_point_under_torch_compile(gpu_device):
+    """A compiled function that calls the operator runs it as an opaque eager region (the reference was written with
+    torch.compile in mind): same results and gradients as eager."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    inp = hp.rounded(po.make_inputs(1, 100, 2, 32, 32, seed=8), torch.bfloat16)
+    dev = gpu_device
+
+    def f(q, k, v, b, gt, g, Ip):
+        return (chunk_palimpsa(q * 1.0, k, v, b, gt, g, Ip, chunk_size=64).float() ** 2).sum()
+
+    def run(fn):
+        leaves = [inp[n].to(dev).clone().requires_grad_(n in ("q", "v")) for n in ("q", "k", "v", "b", "gt", "g", "Ip")]
+        out = fn(*leaves)
+        out.backward()
+        return out.detach(), leaves[0].grad, leaves[2].grad
+
+    eager = run(f)
+    compiled = run(torch.compile(f))
+    for a, b_ in zip(eager, compiled):
+        assert hp.max_rel(b_, a) <= 1e-6
