@@ -232,3 +232,31 @@ def test_head_dim_envelope_of_the_backward(gpu_device, dk, dv, ok):
     for n in ("q", "k", "v", "b", "gt", "g", "Ip"):
         err = hp.max_rel(leaves[n].grad, ref[n])
         assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)
+
+
+def test_runs_on_the_callers_stream(gpu_device):
+    """The kernels are enqueued on torch's current stream: the same call on a side stream gives bitwise the same
+    results, and work queued behind it on that stream sees them."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    inp = hp.rounded(po.make_inputs(2, 200, 2, 32, 32, seed=9), torch.bfloat16)
+    dev = gpu_device
+    names = ("q", "k", "v", "b", "gt", "g", "Ip")
+
+    def run():
+        leaves = [inp[n].to(dev).clone().requires_grad_(True) for n in names]
+        o = chunk_palimpsa(*leaves, chunk_size=64)
+        o.float().sum().backward()
+        return [o.detach()] + [x.grad for x in leaves]
+
+    ref = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = run()
+        total = sum(x.float().abs().sum() for x in got)     # queued behind the kernels on the side stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for a, b_ in zip(ref, got):
+        assert torch.equal(a, b_)
+    assert torch.isfinite(total)
