@@ -24,12 +24,29 @@ __device__ __forceinline__ void store8(T* p, const float* x) {
   store_vec<4>(p, x);
   store_vec<4>(p + 4, x + 4);
 }
-// sum over the GL lanes of a row group (GL a power of two <= 32); every lane of the group gets it
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+// sum over the GL lanes of a row group (GL a power of two <= 32, the same for the whole wave, groups
+// aligned to multiples of GL); every lane of the group gets it.  Lane exchanges inside a row of 16
+// lanes are data-parallel moves: neighbours in a quad, quads, then the mirrored half rows and rows
+// (by then every lane of the smaller group holds the same partial sum, so a mirror pairs as an xor does).
 __device__ __forceinline__ float group_sum(float x, int GL) {
-  for (int m = 1; m < GL; m <<= 1) x += __shfl_xor(x, m);
+  if (GL > 1) x += dpp_move<0xB1>(x);    // quad_perm [1,0,3,2]
+  if (GL > 2) x += dpp_move<0x4E>(x);    // quad_perm [2,3,0,1]
+  if (GL > 4) x += dpp_move<0x141>(x);   // row_half_mirror
+  if (GL > 8) x += dpp_move<0x140>(x);   // row_mirror
+  if (GL > 16) {
+    float a = x, b = x;
+    swap_rows(a, b);
+    x = a + b;
+  }
   return x;
 }
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+// reciprocal to 1 ulp (one instruction; an IEEE division is ten)
+__device__ __forceinline__ float rcpf_(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float sigmoidf_(float x) { return rcpf_(1.f + __expf(-x)); }
 // softplus as torch computes it (threshold 20)
 __device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
 template <typename T>
@@ -78,7 +95,7 @@ __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
       ss = group_sum(ss, GL);
-      const float inv = 1.f / fmaxf(sqrtf(ss), A.eps);
+      const float inv = rcpf_(fmaxf(__builtin_amdgcn_sqrtf(ss), A.eps));
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] *= inv;
       if (on)
@@ -143,9 +160,9 @@ __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
       for (int e = 0; e < 8; ++e) { ss = fmaf(x[e], x[e], ss); xs = fmaf(x[e], s[e], xs); }
       ss = group_sum(ss, GL);
       xs = group_sum(xs, GL);
-      const float nrm = sqrtf(ss);
+      const float nrm = __builtin_amdgcn_sqrtf(ss);
       const bool clamped = nrm < A.eps;
-      const float inv = 1.f / fmaxf(nrm, A.eps);
+      const float inv = rcpf_(fmaxf(nrm, A.eps));
       const float c = clamped ? 0.f : xs * inv * inv * inv;   // (y . s) / n^2 * ... folded: dx = s/n - x (x.s)/n^3
       float out[8];
 #pragma unroll
