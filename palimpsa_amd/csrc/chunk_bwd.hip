@@ -555,7 +555,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
 // One workgroup of 4 waves per (tile, head); wave w owns tokens [16w, 16w+16).  The four products
 // run on the matrix cores (bf16 operands, fp32 accumulate); their results are parked in LDS and then
 // added to the tile-local gradients with 16-byte loads/stores that are contiguous along the head dim.
-template <typename TIn>
+// KSMAX = operand registers per product (32 contraction indices each: head dims up to 32 KSMAX).  With
+// SEQ the dv and db products take turns in one result buffer: less LDS, so that more workgroups share
+// a compute unit (the kernel is a chain of dependent load, product and store phases, and it is the
+// number of resident workgroups that hides them).
+template <typename TIn, int KSMAX, bool SEQ>
 __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
@@ -565,11 +569,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   float* sW4 = sAs + kC;                   // [8]
   float* sBt = sW4 + 8;                    // [64][dv/8] beta of the carry terms, one slot per work item
   float* sO1 = sBt + kC * (dv >> 3);       // [64][OS] dk^carry, later dv^carry
-  float* sO2 = sO1 + kC * (dmax + 4);      // [64][OS] db^carry
+  float* sO2 = SEQ ? sO1 : sO1 + kC * (dmax + 4);   // [64][OS] db^carry (SEQ: after dv^carry has been applied)
   // [2][dk][dv + 8] R_M^T, R_J^T in bf16, operand source of all four products.  When both do not fit the LDS
   // (large head dims) the bf16 copy shares its bytes with db^carry and the dv/db products read the fp32
   // carries from global memory instead.
-  const bool alias = A.apply_alias != 0;
+  const bool alias = !SEQ && A.apply_alias != 0;
   bf16_t* sRT = (bf16_t*)(alias ? sO2 : sO2 + kC * (dmax + 4));
   const int RS = dv + 8;
   const int OS = dmax + 4;
@@ -603,9 +607,13 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     const float* sI = a.chunk_I + ((int64_t)cidx * H + h) * E;
     const float Ipb = a.Ip[h];
     float acc = 0.f;
-    const int ngrp = dk >> 2;
-    for (int idx = tid; idx < dv * ngrp; idx += 256) {
-      const int d = idx % dv, c4 = idx / dv;
+    // a wave instruction covers 16 value rows x 64 bytes, and a wave walks along the rows before it
+    // moves to other rows, so that both halves of a 128-byte line are used while it is still in L1
+    const int nc = dk >> 4, nblk = (dv >> 4) * nc, per = (nblk + 3) >> 2;
+    for (int j = 0; j < per; ++j) {
+      const int blk = w * per + j;
+      if (blk >= nblk) break;
+      const int d = 16 * (blk / nc) + i, c4 = 4 * (blk % nc) + g;
       const int64_t e = (int64_t)d * dk + 4 * c4;
       const f32x4 rm = *(const f32x4*)(RM + e), rj = *(const f32x4*)(RJ + e);
       const f32x4 mu = *(const f32x4*)(smu + e), I = *(const f32x4*)(sI + e);
@@ -632,11 +640,11 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
   {
     const int KS = (dv + 31) / 32;
-    bf16x8 A3[8], A4[8];
+    bf16x8 A3[KSMAX], A4[KSMAX];
     const TIn* vp = (const TIn*)a.v + tokA * dv;
     const TIn* bp = (const TIn*)a.b + tokA * dv;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
+    for (int ks = 0; ks < KSMAX; ++ks) {
       if (ks < KS) {
         const int d0 = 8 * g + 32 * ks;
         float vv[8], bb[8];
@@ -670,7 +678,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       if (nbk + 1 < NBK) load_k4(nbk + 1, knext);
       f32x4 accM = {0.f, 0.f, 0.f, 0.f}, accJ = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
+      for (int ks = 0; ks < KSMAX; ++ks) {
         if (ks < KS) {
           const int d0 = 8 * g + 32 * ks;
           bf16x8 B3, B4;
@@ -715,10 +723,10 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
   {
     const int KS = (dk + 31) / 32;
-    bf16x8 A1[8], A2[8];
+    bf16x8 A1[KSMAX], A2[KSMAX];
     const TIn* kp = (const TIn*)a.k + tokA * dk;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
+    for (int ks = 0; ks < KSMAX; ++ks) {
       if (ks < KS) {
         const int n0 = 8 * g + 32 * ks;
         float kv[8];
@@ -736,79 +744,91 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         }
       }
     }
-    for (int db_ = 0; db_ < dv / 16; ++db_) {
-      f32x4 accV = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        if (ks < KS) {
-          const int n0 = 8 * g + 32 * ks;
-          bf16x8 B1, B2;
-          if (n0 < dk && !alias) {
-            // 8 consecutive key columns of value row d = 16db_ + i: a column walk through the transposed
-            // bf16 copy in LDS (the fp32 carries in global memory would miss L2 on this second read)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              B1[j] = sRT[(n0 + j) * RS + 16 * db_ + i];
-              B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i];
-            }
-          } else if (n0 < dk) {
-            const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
-            const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
-            const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
-            const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
-              B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { B1[j] = (bf16_t)0.f; B2[j] = (bf16_t)0.f; }
-          }
-          accV = mfma16(A1[ks], B1, accV);
-          accB = mfma16(A2[ks], B2, accB);
-        }
-      }
-      // accumulator layout: rows s = 16w + 4g + r, column d = 16db_ + i
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        sO1[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accV[r];
-        sO2[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accB[r];
-      }
-    }
-  }
-  __syncthreads();
-  {
-    // add to the tile-local dv, db; beta_s = <v_s, dv^carry_s> + <b_s, db^carry_s>
     const int groups = dv >> 3;   // work item = (token, 8 value rows); the items of a token sit in adjacent lanes
     const TIn* vin = (const TIn*)a.v + tok0 * dv;
     const TIn* bin = (const TIn*)a.b + tok0 * dv;
     TIn* dvo = (TIn*)A.dv + tok0 * dv;
     TIn* dbo = (TIn*)A.db + tok0 * dv;
-    for (int idx = tid; idx < kC * groups; idx += 256) {
-      const int c8 = idx % groups, s = idx / groups;
-      float beta = 0.f;
-      if (s < clen) {
-        const int64_t off = (int64_t)s * H * dv + 8 * c8;
-        float xv[8], xb[8], gv[8], gb[8];
-        load_vec<4>(vin + off, xv); load_vec<4>(vin + off + 4, xv + 4);
-        load_vec<4>(bin + off, xb); load_vec<4>(bin + off + 4, xb + 4);
-        load_vec<4>(dvo + off, gv); load_vec<4>(dvo + off + 4, gv + 4);
-        load_vec<4>(dbo + off, gb); load_vec<4>(dbo + off + 4, gb + 4);
+    constexpr int NPASS = SEQ ? 2 : 1;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float cv = sO1[s * OS + 8 * c8 + e], cb = sO2[s * OS + 8 * c8 + e];
-          beta = fmaf(xv[e], cv, beta);
-          beta = fmaf(xb[e], cb, beta);
-          gv[e] += cv;
-          gb[e] += cb;
+    for (int pass = 0; pass < NPASS; ++pass) {
+      const bool doV = !SEQ || pass == 0, doB = !SEQ || pass == 1;
+      for (int db_ = 0; db_ < dv / 16; ++db_) {
+        f32x4 accV = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSMAX; ++ks) {
+          if (ks < KS) {
+            const int n0 = 8 * g + 32 * ks;
+            bf16x8 B1, B2;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { B1[j] = (bf16_t)0.f; B2[j] = (bf16_t)0.f; }
+            if (n0 < dk && !alias) {
+              // 8 consecutive key columns of value row d = 16db_ + i: a column walk through the transposed
+              // bf16 copy in LDS (the fp32 carries in global memory would miss L2 on this second read)
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                if (doV) B1[j] = sRT[(n0 + j) * RS + 16 * db_ + i];
+                if (doB) B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i];
+              }
+            } else if (n0 < dk) {
+              const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
+              const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
+              const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
+              const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
+                B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
+              }
+            }
+            if (doV) accV = mfma16(A1[ks], B1, accV);
+            if (doB) accB = mfma16(A2[ks], B2, accB);
+          }
         }
-        store_vec<4>(dvo + off, gv); store_vec<4>(dvo + off + 4, gv + 4);
-        store_vec<4>(dbo + off, gb); store_vec<4>(dbo + off + 4, gb + 4);
+        // accumulator layout: rows s = 16w + 4g + r, column d = 16db_ + i
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (doV) sO1[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accV[r];
+          if (doB) sO2[(16 * w + 4 * g + r) * OS + 16 * db_ + i] = accB[r];
+        }
       }
-      sBt[idx] = beta;
+      __syncthreads();
+      // add to the tile-local dv, db; beta_s = <v_s, dv^carry_s> + <b_s, db^carry_s>
+      for (int idx = tid; idx < kC * groups; idx += 256) {
+        const int c8 = idx % groups, s = idx / groups;
+        float beta = 0.f;
+        if (s < clen) {
+          const int64_t off = (int64_t)s * H * dv + 8 * c8;
+          if (doV) {
+            float xv[8], gv[8];
+            load_vec<4>(vin + off, xv); load_vec<4>(vin + off + 4, xv + 4);
+            load_vec<4>(dvo + off, gv); load_vec<4>(dvo + off + 4, gv + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float cv = sO1[s * OS + 8 * c8 + e];
+              beta = fmaf(xv[e], cv, beta);
+              gv[e] += cv;
+            }
+            store_vec<4>(dvo + off, gv); store_vec<4>(dvo + off + 4, gv + 4);
+          }
+          if (doB) {
+            float xb[8], gb[8];
+            load_vec<4>(bin + off, xb); load_vec<4>(bin + off + 4, xb + 4);
+            load_vec<4>(dbo + off, gb); load_vec<4>(dbo + off + 4, gb + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float cb = sO2[s * OS + 8 * c8 + e];
+              beta = fmaf(xb[e], cb, beta);
+              gb[e] += cb;
+            }
+            store_vec<4>(dbo + off, gb); store_vec<4>(dbo + off + 4, gb + 4);
+          }
+        }
+        // the second pass of SEQ adds to the share the same thread left in the first
+        sBt[idx] = (SEQ && pass == 1) ? sBt[idx] + beta : beta;
+      }
+      __syncthreads();   // SEQ: the result buffer is free for the next pass; last pass: sBt is complete
     }
-    __syncthreads();
     if (tid < clen) {
       float bsum = 0.f;
       for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[tid * groups + c8];   // fixed order
@@ -942,6 +962,20 @@ static int launch_local(const BwdArgs& A, hipStream_t s) {
   }
 }
 
+template <typename TIn, int KSMAX, bool SEQ>
+static int launch_carry_apply_t(const BwdArgs& A, unsigned blocks, size_t lds, hipStream_t s) {
+  if (int rc = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ>), dim3(blocks), dim3(256), lds, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+template <typename TIn>
+static int launch_carry_apply(const BwdArgs& A, int ksmax, bool seq, unsigned blocks, size_t lds, hipStream_t s) {
+  if (ksmax == 2) return seq ? launch_carry_apply_t<TIn, 2, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 2, false>(A, blocks, lds, s);
+  if (ksmax == 4) return seq ? launch_carry_apply_t<TIn, 4, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 4, false>(A, blocks, lds, s);
+  return seq ? launch_carry_apply_t<TIn, 8, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 8, false>(A, blocks, lds, s);
+}
+
 }  // namespace pal
 
 extern "C" size_t pal_chunk_bwd_workspace_bytes(const PalDims* d) {
@@ -1000,14 +1034,14 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
       A.apply_alias = 1;
       lds = lds_fixed + (rt_bytes > o_bytes ? rt_bytes : o_bytes);
     }
+    // one result buffer used twice when that lets more workgroups share a compute unit
+    const size_t lds_seq = lds_fixed + rt_bytes;
+    const bool seq = lds_seq <= kMaxLds && kMaxLds / lds_seq > (lds > kMaxLds ? 0 : kMaxLds / lds);
+    if (seq) { lds = lds_seq; A.apply_alias = 0; }
     if (lds > kMaxLds) return PAL_E_HEADDIM;
-    if (bf) {
-      if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<bf16_t>, lds)) return rc2;
-      PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<bf16_t>), dim3(blocks), dim3(256), lds, s, A);
-    } else {
-      if (int rc2 = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<float>, lds)) return rc2;
-      PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<float>), dim3(blocks), dim3(256), lds, s, A);
-    }
+    const int ksmax = dmax <= 64 ? 2 : dmax <= 128 ? 4 : 8;
+    rc = bf ? launch_carry_apply<bf16_t>(A, ksmax, seq, blocks, lds, s) : launch_carry_apply<float>(A, ksmax, seq, blocks, lds, s);
+    if (rc) return rc;
     PAL_HIP_LAUNCH_CHECK();
   }
   PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads)), dim3(256), 0, s, A);
