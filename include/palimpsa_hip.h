@@ -270,6 +270,18 @@ size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims *dims);
 int pal_epilogue_bwd(const PalGlueDims *dims, const PalEpilogueTensors *t, const PalEpilogueGrads *gr,
                      void *workspace, size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------------------ tuning knob */
+
+/* How the chunked entry points (pal_chunk_fwd, pal_gla_chunk_fwd, pal_gla_chunk_bwd) build the
+ * states at the start of every tile; no counterpart in the reference, results agree to rounding.
+ *   0 (default): chosen by shape;
+ *   1: per-tile contributions by all tiles in parallel, then a scan over the tiles
+ *      (any shape and dtype);
+ *   2: one pass per (sequence, head) that keeps the running state in registers, wherever it
+ *      applies (bf16 rows).
+ * Process-global; meant for tests and measurements. */
+void pal_set_state_pass_mode(int mode);
+
 /* ------------------------------------------------------------ measurement */
 
 /* Per-kernel timing aid; no counterpart in the reference.  While enabled, every

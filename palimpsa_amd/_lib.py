@@ -121,6 +121,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_size_t
         fn.argtypes = [P(PalGlueDims)]
+    lib.pal_set_state_pass_mode.restype = None
+    lib.pal_set_state_pass_mode.argtypes = [C.c_int]
     lib.pal_profile_enable.restype = C.c_int
     lib.pal_profile_enable.argtypes = [C.c_int]
     lib.pal_profile_kernel_count.restype = C.c_int
@@ -131,6 +133,9 @@ def load() -> C.CDLL:
     lib.pal_profile_read.argtypes = [C.c_int, P(C.c_double), P(C.c_int64)]
     if lib.pal_abi_version() != PAL_ABI_VERSION:
         raise ImportError(f"{LIB_PATH}: ABI version {lib.pal_abi_version()} != expected {PAL_ABI_VERSION}; rebuild")
+    mode = os.environ.get("PALIMPSA_STATE_PASS_MODE")
+    if mode is not None:
+        lib.pal_set_state_pass_mode(int(mode))
     _lib = lib
     return lib
 

@@ -107,14 +107,22 @@ __device__ __forceinline__ int tile_block_exponent(const TIn* kt, const TIn* vt,
   return (m > 4096.f) ? min(15, ilogbf(m) - 12) : 0;
 }
 
-// inclusive prefix sum over the 64 lanes of a wave
+// inclusive prefix sum over the 64 lanes of a wave: four shifted adds inside each row of 16 lanes (DPP
+// row_shr with zero fill), then the totals of the rows before (lane 15 of each, read as scalars)
+template <int N>
+__device__ __forceinline__ float row_shr_zero(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + N, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float wave_inclusive_scan(float x, int lane) {
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    float y = __shfl_up(x, off);
-    if (lane >= off) x += y;
-  }
-  return x;
+  x += row_shr_zero<1>(x);
+  x += row_shr_zero<2>(x);
+  x += row_shr_zero<4>(x);
+  x += row_shr_zero<8>(x);
+  const float t0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 15));
+  const float t1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 31));
+  const float t2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 47));
+  const int row = lane >> 4;
+  return x + (row == 0 ? 0.f : row == 1 ? t0 : row == 2 ? t0 + t1 : (t0 + t1) + t2);
 }
 
 }  // namespace pal

@@ -565,6 +565,12 @@ void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
 
 namespace pal {
 
+// the one-pass form of chunk_states.hip
+bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j);
+int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tiles_b, const float* init_a,
+                      const float* init_b, float* fin_a, float* fin_b, bool reverse, float fin_scale, int kern_id,
+                      hipStream_t s);
+
 // Local contribution of every tile to the state, into chunk_mu (and chunk_I when has_j).
 template <typename TIn, bool HAS_J, typename TS>
 static int launch_tile_delta_t(const ChunkArgs& a, hipStream_t s) {
@@ -596,6 +602,9 @@ int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) 
 // Tile-start states: local contributions, then the serial scan over the tiles of each sequence.
 // has_j = false leaves the precision state out (b, Ip, chunk_I, init_I, final_I are not touched).
 int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {
+  if (state_pass_applies(a, dtype, has_j))
+    return launch_state_pass(a, has_j, has_j ? (void*)a.chunk_mu : (void*)a.chunk_I, has_j ? a.chunk_I : nullptr, a.init_mu,
+                             a.init_I, a.final_mu, a.final_I, false, 1.f, kKernChunkStates, s);
   if (int rc = launch_tile_delta(a, dtype, has_j, s)) return rc;
   {
     const int64_t E = (int64_t)a.dv * a.dk;

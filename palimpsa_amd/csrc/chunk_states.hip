@@ -1,0 +1,384 @@
+// Tile-start states of the chunked algorithm in one pass (bf16 rows):
+//     S_c = F_c S_{c-1} + Delta_c ,  Delta_c = sum_s a_s v_s k_s^T  (and sum_s a_s b_s (k_s*k_s)^T for the
+//     precision state)
+// computed by a workgroup that walks the tiles of one sequence in order with the running state in the
+// accumulators of the matrix cores, so that the per-tile contributions Delta_c never go to memory (the
+// two-kernel form, chunk_delta_kernel + a scan kernel, writes them in fp32 and reads them back: three times
+// the bytes of the states themselves).  What the reference keeps as intermediate_*_state
+// (chunk_palimpsa_forgetting_scalar.py:187-188) is written at the start of every tile, the state after
+// the last tile at the end (:214-218).
+//
+// One workgroup of 12 waves per (sequence, head, slice of ds value rows): four hold the state (the slice times
+// dk is at most 4096 entries = 16 blocks of 16x16, up to four per wave), two groups of four stage the rows for them.  The rows of a tile are staged transposed in LDS
+// (token index fastest, two tokens per 32-bit word) as in chunk_delta_kernel.  The serial chain over the tiles
+// is hidden by fetching ahead: rows are fetched into registers three steps before they go to LDS, two LDS
+// buffers hold the current and the next tile, one barrier per tile.
+// The same kernel walks a sequence backwards for the gradient of the scalar-gated path (weights from the
+// start of the tile, G_{c-1} = F_c G_c + D_c, the value left after the first tile is the gradient of the
+// initial state).
+#include "chunk_common.h"
+#include "pal_host.h"
+#include "pal_profile.h"
+
+namespace pal {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kStTS = 72;          // tokens (bf16) per staged row: 64 + 8 keeps 16-byte reads conflict-free
+constexpr int kStMaxBlocks = 4;    // 16x16 state blocks per wave
+
+struct StatePassArgs {
+  ChunkArgs c;
+  void* tiles_a;          // scalar-gated: bf16 tile states; Palimpsa: fp32 mu at the start of every tile
+  float* tiles_b;         // Palimpsa: fp32 I at the start of every tile
+  const float *init_a, *init_b;
+  float *fin_a, *fin_b;
+  int32_t ds, nsplit, reverse, per_xcd, total;
+  float fin_scale;
+};
+
+template <int NIK>
+struct StageRegs {
+  u32x4 k[NIK][2];
+  u32x4 v[2], b[2];
+  uint32_t gt;   // gate of token `lane` as loaded: fp32 bits or a bf16 in the low half (last wave)
+};
+
+template <bool HAS_J, int NIK>
+__global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
+  const ChunkArgs& a = A.c;
+  extern __shared__ float smem[];
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = a.H, dk = a.dk, dv = a.dv, ds = A.ds;
+  // consecutive workgroup ids go to different XCDs: give the slices of one (sequence, head) to the same one,
+  // they read the same key rows
+  const int m = ((int)blockIdx.x & 7) * A.per_xcd + ((int)blockIdx.x >> 3);
+  if (m >= A.total) return;
+  const int nh = m / A.nsplit, d0 = (m % A.nsplit) * ds;
+  const int h = nh % H, n = nh / H;
+  int bos, len, cbase;
+  seq_lookup(a, n, bos, len, cbase);
+  const int nchunks = (len + kC - 1) / kC;
+
+  float* sA = smem;                                   // [3][64] weight of token s in its tile (ring over tiles)
+  float* sF = sA + 3 * kC;                            // [3] decay over the whole tile (+1 pad)
+  uint32_t* sKT = (uint32_t*)(sF + 4);                // [2][dk][36] words = [dk][72] bf16
+  uint32_t* sVT = sKT + 2 * dk * (kStTS / 2);         // [2][ds][36]
+  uint32_t* sBT = sVT + 2 * ds * (kStTS / 2);         // [2][ds][36] (HAS_J)
+  const int kbuf = dk * (kStTS / 2), vbuf = ds * (kStTS / 2);
+  auto tile_len = [&](int p) {
+    const int c = A.reverse ? nchunks - 1 - p : p;
+    return p < nchunks ? min(kC, len - c * kC) : 0;
+  };
+
+  // Waves 0-3 own the state (a 16x16 block per wave and slot), waves 4-11 feed them: a single wave issues an
+  // instruction every five to eight cycles, so the kinds of work sit on different waves of each SIMD instead
+  // of following one another.  The feeding waves form two groups of four, one for the even tiles (LDS buffer
+  // 0) and one for the odd tiles (buffer 1): a group works out the weights of a tile and fetches ahead in one
+  // step, and puts the tile's rows into its buffer in the next, while the other group does the opposite.
+  // All roles pass the same barriers, one per step; steps -2 and -1 fill the pipeline.
+  if (w >= 4) {
+    // ---------------------------------------------------------------- staging role
+    // Items of a thread: (token pair, 8 columns).  The key items start at staging thread 0, the value items at
+    // thread 64, the items of b at thread 128 (both wrap around) and the last wave turns the gates of a tile
+    // into its weights.  Byte offsets of the two tokens from the first row of a tile and word offsets in the
+    // staging tiles do not change from tile to tile.
+    const int grp = (w - 4) >> 2;           // parity of the tiles this group stages
+    const int wg = (w - 4) & 3;             // wave in the group
+    const int st = tid - 256 - 256 * grp;
+    const int gk = dk >> 3, gv = ds >> 3;
+    int ksp[NIK];
+    uint32_t koff[NIK][2], kdst[NIK];
+    bool kval[NIK];
+#pragma unroll
+    for (int j = 0; j < NIK; ++j) {
+      const int idx = st + 256 * j;
+      kval[j] = idx < 32 * gk;
+      ksp[j] = idx / gk;
+      const int c8 = idx - ksp[j] * gk;
+      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * H * dk + 8 * c8) * 2) : 0u;
+      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * H * dk + 8 * c8) * 2) : 0u;
+      kdst[j] = (uint32_t)(8 * c8 * (kStTS / 2) + ksp[j]);
+    }
+    const int vtid = (st + 192) & 255, btid = (st + 128) & 255;
+    const bool vval = vtid < 32 * gv, bval = HAS_J && btid < 32 * gv;
+    const int vsp = vtid / gv, vc8 = vtid - vsp * gv, bsp = btid / gv, bc8 = btid - bsp * gv;
+    uint32_t voff[2], boff[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      voff[u] = vval ? (uint32_t)(((2 * vsp + u) * H * dv + 8 * vc8) * 2) : 0u;
+      boff[u] = bval ? (uint32_t)(((2 * bsp + u) * H * dv + 8 * bc8) * 2) : 0u;
+    }
+    const uint32_t vdst = (uint32_t)(8 * vc8 * (kStTS / 2) + vsp), bdst = (uint32_t)(8 * bc8 * (kStTS / 2) + bsp);
+    const char* kbase = (const char*)((const bf16_t*)a.k + ((int64_t)bos * H + h) * dk);
+    const char* vbase = (const char*)((const bf16_t*)a.v + ((int64_t)bos * H + h) * dv + d0);
+    const char* bbase = HAS_J ? (const char*)((const bf16_t*)a.b + ((int64_t)bos * H + h) * dv + d0) : nullptr;
+    const float gh = a.g[h] * kLog2e;
+    const bool from_start = (a.flags & kFlagDecayFromStart) != 0;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+    // Fetches are issued without a branch and without touching the result: a row beyond the end of a tile is
+    // fetched from the tile's first row (a tile past the end of the sequence: from the start of the tensor) and
+    // zeroed when the registers go to LDS.  Any use of a fetched value here would make the wave wait for
+    // everything it has in flight, which is what fetching ahead is meant to avoid.
+    auto load_stage = [&](StageRegs<NIK>& R, int p) {
+      const int c = A.reverse ? nchunks - 1 - p : p;
+      const int clen = tile_len(p);
+      const bool live = clen > 0, full = clen == kC;
+      const int64_t tb = live ? (int64_t)c * kC : 0;
+      const char* kt = live ? kbase + tb * H * dk * 2 : (const char*)a.k;
+      const char* vt = live ? vbase + tb * H * dv * 2 : (const char*)a.v;
+      const char* bt = live ? bbase + tb * H * dv * 2 : (const char*)a.b;
+#pragma unroll
+      for (int j = 0; j < NIK; ++j) {
+        R.k[j][0] = *(const u32x4*)(kt + ((full || 2 * ksp[j] < clen) ? koff[j][0] : 0u));
+        R.k[j][1] = *(const u32x4*)(kt + ((full || 2 * ksp[j] + 1 < clen) ? koff[j][1] : 0u));
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        R.v[u] = *(const u32x4*)(vt + ((full || 2 * vsp + u < clen) ? voff[u] : 0u));
+        if (HAS_J) R.b[u] = *(const u32x4*)(bt + ((full || 2 * bsp + u < clen) ? boff[u] : 0u));
+      }
+      if (wg == 3) {
+        const int64_t gi = (lane < clen) ? (bos + tb + lane) * H + h : 0;
+        R.gt = a.gate_bf16 ? (uint32_t)((const uint16_t*)a.gt)[gi] : ((const uint32_t*)a.gt)[gi];   // raw; widened below
+      }
+    };
+    // eight columns of two tokens -> one word (token pair) per column
+    auto put = [&](uint32_t* dst, u32x4 x0, u32x4 x1, int sp, int clen) {
+      if (clen < kC) {   // same for the whole workgroup
+        if (2 * sp >= clen) x0 = zero4;
+        if (2 * sp + 1 >= clen) x1 = zero4;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+        dst[e * (kStTS / 2)] = __builtin_amdgcn_perm(x1[e >> 1], x0[e >> 1], sel);
+      }
+    };
+    // the same for rows of v and b, which are staged times the weight of their token (the operand the matrix
+    // cores take is a_s v_s, rounded to bf16 once)
+    auto put_weighted = [&](uint32_t* dst, u32x4 x0, u32x4 x1, int sp, int clen, const float* wts) {
+      if (clen < kC) {
+        if (2 * sp >= clen) x0 = zero4;
+        if (2 * sp + 1 >= clen) x1 = zero4;
+      }
+      const f32x2 a2 = *(const f32x2*)&wts[2 * sp];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t w0 = x0[e >> 1], w1 = x1[e >> 1];
+        const float f0 = __builtin_bit_cast(float, (e & 1) ? (w0 & 0xffff0000u) : (w0 << 16));
+        const float f1 = __builtin_bit_cast(float, (e & 1) ? (w1 & 0xffff0000u) : (w1 << 16));
+        *(bf16x2*)&dst[e * (kStTS / 2)] = pack2(f0 * a2[0], f1 * a2[1]);
+      }
+    };
+    auto store_stage = [&](const StageRegs<NIK>& R, int buf, int p) {
+      const int clen = tile_len(p);
+#pragma unroll
+      for (int j = 0; j < NIK; ++j)
+        if (kval[j]) put(sKT + buf * kbuf + kdst[j], R.k[j][0], R.k[j][1], ksp[j], clen);
+      const float* wts = sA + (p % 3) * kC;
+      if (vval) put_weighted(sVT + buf * vbuf + vdst, R.v[0], R.v[1], vsp, clen, wts);
+      if (HAS_J && bval) put_weighted(sBT + buf * vbuf + bdst, R.b[0], R.b[1], bsp, clen, wts);
+    };
+    // weights of the tokens of tile p and the decay over the whole tile, one step before its rows are staged
+    auto scan_stage = [&](const StageRegs<NIK>& R, int p) {
+      if (wg == 3) {
+        const int clen = tile_len(p);
+        const float gt = (lane < clen) ? __builtin_bit_cast(float, a.gate_bf16 ? R.gt << 16 : R.gt) : 0.f;
+        const float cs = wave_inclusive_scan(-gt * gh, lane);
+        const float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cs), 63));
+        sA[(p % 3) * kC + lane] = fast_exp2(from_start ? cs : tot - cs);
+        if (lane == 0) sF[p % 3] = fast_exp2(tot);
+      }
+    };
+
+    // Two register sets per group: the tile being staged and the group's next one (two tiles later), which is
+    // fetched three steps before its rows go to LDS.  In step p the group of parity (p + 1) & 1 stages tile p + 1,
+    // the other one handles tile p + 2: weights from its gates (set (p + 2) / 2 % 2), then the fetch of tile p + 4
+    // into the set that was staged a step ago.
+    StageRegs<NIK> R[2];
+    load_stage(R[0], grp);
+    for (int p0 = -2; p0 < nchunks; p0 += 4) {
+#pragma unroll
+      for (int ph = 0; ph < 4; ++ph) {
+        const int p = p0 + ph;           // p + 2 = ph (mod 4)
+        if ((ph & 1) == grp) {
+          scan_stage(R[(ph >> 1) & 1], p + 2);
+          load_stage(R[1 - ((ph >> 1) & 1)], p + 4);
+        } else if (p + 1 >= 0) {
+          store_stage(R[(((ph + 3) & 3) >> 1) & 1], grp, p + 1);
+        }
+        __syncthreads();
+      }
+    }
+    return;
+  }
+
+  // ------------------------------------------------------------------ state role
+  // state blocks of this wave: block sb = w + 4 jj -> (value rows 16 db.., key columns 16 nb..)
+  const int NB = dk >> 4, NSB = (ds >> 4) * NB;
+  int ldk[kStMaxBlocks], ldv[kStMaxBlocks], goff[kStMaxBlocks];   // operand rows in the staging tiles, entry in a state
+  bool sval[kStMaxBlocks];
+  f32x4 accM[kStMaxBlocks], accJ[kStMaxBlocks];
+  const int64_t E = (int64_t)dv * dk;
+  const float Ip = HAS_J ? a.Ip[h] : 0.f;
+#pragma unroll
+  for (int jj = 0; jj < kStMaxBlocks; ++jj) {
+    const int sb = w + 4 * jj;
+    sval[jj] = sb < NSB;
+    const int db = sb / NB, nb = sb - db * NB;
+    // rows n = 16 nb + 4 g + r (four consecutive key columns), column d = d0 + 16 db + i
+    ldk[jj] = (16 * nb + i) * kStTS + 8 * g;
+    ldv[jj] = (16 * db + i) * kStTS + 8 * g;
+    goff[jj] = (d0 + 16 * db + i) * dk + 16 * nb + 4 * g;
+    accM[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    accJ[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (sval[jj] && A.init_a) {
+      const int64_t off = (int64_t)nh * E + goff[jj];
+      const f32x4 x = *(const f32x4*)(A.init_a + off);
+      if (HAS_J) {
+        const f32x4 I = *(const f32x4*)(A.init_b + off);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { accM[jj][r] = x[r] * I[r]; accJ[jj][r] = I[r] - Ip; }
+      } else {
+        accM[jj] = x;
+      }
+    }
+  }
+  __syncthreads();   // steps -2 and -1 of the feeding waves
+  __syncthreads();
+  for (int p = 0; p < nchunks; ++p) {
+    const int buf = p & 1;
+    const int c = A.reverse ? nchunks - 1 - p : p;
+    const int64_t slot = ((int64_t)(cbase + c) * H + h) * E;
+    const float F = sF[p % 3];
+    const bf16_t* kt = (const bf16_t*)(sKT + buf * kbuf);
+    const bf16_t* vt = (const bf16_t*)(sVT + buf * vbuf);
+    const bf16_t* bt = (const bf16_t*)(sBT + buf * vbuf);
+#pragma unroll
+    for (int jj = 0; jj < kStMaxBlocks; ++jj) {
+      if (!sval[jj]) continue;
+      const int64_t off = slot + goff[jj];
+      if (HAS_J) {
+        f32x4 mu, I;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { I[r] = accJ[jj][r] + Ip; mu[r] = accM[jj][r] * fast_rcp(I[r]); }
+        *(f32x4*)((float*)A.tiles_a + off) = mu;
+        *(f32x4*)(A.tiles_b + off) = I;
+      } else {
+        store_vec<4>((bf16_t*)A.tiles_a + off, (const float*)&accM[jj]);
+      }
+      f32x4 M = accM[jj] * F, J = accJ[jj] * F;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const bf16x8 BK = *(const bf16x8*)&kt[ldk[jj] + 32 * ks];
+        const bf16x8 AM = *(const bf16x8*)&vt[ldv[jj] + 32 * ks];
+        M = mfma16(BK, AM, M);
+        if (HAS_J) {
+          const bf16x8 AJ = *(const bf16x8*)&bt[ldv[jj] + 32 * ks];
+          bf16x8 BKK;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float kf = (float)BK[j];
+            BKK[j] = (bf16_t)(kf * kf);
+          }
+          J = mfma16(BKK, AJ, J);
+        }
+      }
+      accM[jj] = M;
+      accJ[jj] = J;
+    }
+    __syncthreads();
+  }
+  // the feeding waves take their steps in groups of four, starting at -2
+  for (int p = nchunks; ((p + 2) & 3) != 0; ++p) __syncthreads();
+
+  if (A.fin_a) {
+#pragma unroll
+    for (int jj = 0; jj < kStMaxBlocks; ++jj) {
+      if (!sval[jj]) continue;
+      const int64_t off = (int64_t)nh * E + goff[jj];
+      if (HAS_J) {
+        f32x4 mu, I;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { I[r] = accJ[jj][r] + Ip; mu[r] = accM[jj][r] * fast_rcp(I[r]); }
+        *(f32x4*)(A.fin_a + off) = mu;
+        *(f32x4*)(A.fin_b + off) = I;
+      } else {
+        *(f32x4*)(A.fin_a + off) = accM[jj] * A.fin_scale;
+      }
+    }
+  }
+}
+
+static int g_state_pass_mode = 0;   // 0: by shape, 1: always the two-kernel form, 2: the one-pass form where it applies
+
+template <bool HAS_J, int NIK>
+static int launch_state_pass_t(const StatePassArgs& A, int kern_id, unsigned grid, size_t lds, hipStream_t s) {
+  if (int rc = allow_lds((const void*)&chunk_states_kernel<HAS_J, NIK>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kern_id, s, (chunk_states_kernel<HAS_J, NIK>), dim3(grid), dim3(768), lds, s, A);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
+template <bool HAS_J>
+static int launch_state_pass_j(const StatePassArgs& A, int kern_id, unsigned grid, size_t lds, hipStream_t s) {
+  switch ((A.c.dk + 63) / 64) {
+    case 1: return launch_state_pass_t<HAS_J, 1>(A, kern_id, grid, lds, s);
+    case 2: return launch_state_pass_t<HAS_J, 2>(A, kern_id, grid, lds, s);
+    case 3: return launch_state_pass_t<HAS_J, 3>(A, kern_id, grid, lds, s);
+    case 4: return launch_state_pass_t<HAS_J, 4>(A, kern_id, grid, lds, s);
+    default: return PAL_E_HEADDIM;
+  }
+}
+
+// Whether the one-pass form serves this call: bf16 rows, and enough (sequence, head, slice) workgroups that
+// the serial walk over the tiles does not leave most of the GPU idle.
+bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j) {
+  if (dtype != PAL_DTYPE_BF16 || g_state_pass_mode == 1) return false;
+  if (a.dk < 16 || a.dk > 256 || a.dk % 16 || a.dv % 16) return false;
+  if (g_state_pass_mode == 2) return true;
+  // Measured on MI355X: a workgroup needs about 0.8 us per tile whatever the head dims, so the one-pass form
+  // pays where the per-tile contributions are large (their fp32 round trip is what it saves) and a few
+  // hundred workgroups exist; with the precision state and 64x64 heads the two-kernel form is as fast.
+  if ((int64_t)a.n_seqs * a.H * (a.dv / 16) < 192) return false;
+  return !has_j || (int64_t)a.dk * a.dv >= 8192;
+}
+
+// tiles_a / tiles_b, init_*, fin_*: see StatePassArgs.  reverse walks every sequence from its last tile.
+int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tiles_b, const float* init_a,
+                      const float* init_b, float* fin_a, float* fin_b, bool reverse, float fin_scale, int kern_id,
+                      hipStream_t s) {
+  StatePassArgs A;
+  A.c = a;
+  A.tiles_a = tiles_a; A.tiles_b = tiles_b;
+  A.init_a = init_a; A.init_b = init_b; A.fin_a = fin_a; A.fin_b = fin_b;
+  A.reverse = reverse ? 1 : 0;
+  A.fin_scale = fin_scale;
+  // value rows per workgroup: the largest slice that still gives the GPU a few hundred workgroups
+  int ds = 16;
+  const int cand[3] = {64, 48, 32};
+  for (int c : cand) {
+    if (a.dv % c || c * a.dk > 4096) continue;
+    if ((int64_t)a.n_seqs * a.H * (a.dv / c) >= 512) { ds = c; break; }
+  }
+  A.ds = ds;
+  A.nsplit = a.dv / ds;
+  const int64_t total = (int64_t)a.n_seqs * a.H * A.nsplit;
+  if (total <= 0) return PAL_OK;
+  int64_t per_xcd = (total + 7) / 8;
+  per_xcd = (per_xcd + A.nsplit - 1) / A.nsplit * A.nsplit;
+  if (per_xcd * 8 > 0x7fffffff) return PAL_E_DIM;
+  A.total = (int32_t)total;
+  A.per_xcd = (int32_t)per_xcd;
+  const size_t lds = sizeof(float) * (3 * kC + 4) + (size_t)2 * 2 * kStTS * (a.dk + ds * (has_j ? 2 : 1));
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  const unsigned grid = (unsigned)(per_xcd * 8);
+  return has_j ? launch_state_pass_j<true>(A, kern_id, grid, lds, s) : launch_state_pass_j<false>(A, kern_id, grid, lds, s);
+}
+
+}  // namespace pal
+
+extern "C" void pal_set_state_pass_mode(int mode) { pal::g_state_pass_mode = (mode >= 0 && mode <= 2) ? mode : 0; }

@@ -17,6 +17,10 @@ namespace pal {
 void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t);
 int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
 int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
+bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j);
+int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tiles_b, const float* init_a,
+                      const float* init_b, float* fin_a, float* fin_b, bool reverse, float fin_scale, int kern_id,
+                      hipStream_t s);
 
 constexpr int kVT = 72;  // row stride (bf16) of the transposed value tile
 
@@ -551,12 +555,18 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   {
     ChunkArgs b = a;
     b.k = t->q; b.v = gr->d_o; b.chunk_mu = d_tiles; b.flags |= kFlagDecayFromStart;
+    if (state_pass_applies(b, d->dtype, false)) {
+      if (int rc = launch_state_pass(b, false, g_tiles, nullptr, nullptr, nullptr, gr->d_init_mu, nullptr, true, a.scale,
+                                     kKernGlaBwdStates, s))
+        return rc;
+    } else {
     if (int rc = launch_tile_delta(b, d->dtype, false, s)) return rc;
     const int64_t blocks = (int64_t)d->n_seqs * d->n_heads * (((int64_t)d->dv * d->dk + 1023) / 1024);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
     PAL_TIMED_LAUNCH(kKernGlaBwdScan, s, gla_bwd_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, d_tiles,
                      g_tiles, gr->d_init_mu);
     PAL_HIP_LAUNCH_CHECK();
+    }
   }
   GlaTileArgs A{};
   A.c = a;

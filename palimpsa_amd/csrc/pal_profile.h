@@ -27,6 +27,8 @@ enum KernelId {
   kKernEpilogueFwd,
   kKernEpilogueBwd,
   kKernGlaRecurrentFwd,
+  kKernChunkStates,
+  kKernGlaBwdStates,
   kKernCount
 };
 
