@@ -9,13 +9,15 @@
 // the last tile at the end (:214-218).
 //
 // One workgroup of 12 waves per (sequence, head, slice of ds value rows): four hold the state (the slice times
-// dk is at most 4096 entries = 16 blocks of 16x16, up to four per wave), two groups of four stage the rows for them.  The rows of a tile are staged transposed in LDS
+// dk is at most 6144 entries = 24 blocks of 16x16, up to six per wave), two groups of four stage the rows for them.  The rows of a tile are staged transposed in LDS
 // (token index fastest, two tokens per 32-bit word) as in chunk_delta_kernel.  The serial chain over the tiles
 // is hidden by fetching ahead: rows are fetched into registers three steps before they go to LDS, two LDS
 // buffers hold the current and the next tile, one barrier per tile.
 // The same kernel walks a sequence backwards for the gradient of the scalar-gated path (weights from the
 // start of the tile, G_{c-1} = F_c G_c + D_c, the value left after the first tile is the gradient of the
 // initial state).
+#include <type_traits>
+
 #include "chunk_common.h"
 #include "pal_host.h"
 #include "pal_profile.h"
@@ -25,7 +27,7 @@ namespace pal {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kStTS = 72;          // tokens (bf16) per staged row: 64 + 8 keeps 16-byte reads conflict-free
-constexpr int kStMaxBlocks = 4;    // 16x16 state blocks per wave
+constexpr int kStMaxBlocks = 6;    // 16x16 state blocks per wave
 
 struct StatePassArgs {
   ChunkArgs c;
@@ -67,10 +69,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
   uint32_t* sVT = sKT + 2 * dk * (kStTS / 2);         // [2][ds][36]
   uint32_t* sBT = sVT + 2 * ds * (kStTS / 2);         // [2][ds][36] (HAS_J)
   const int kbuf = dk * (kStTS / 2), vbuf = ds * (kStTS / 2);
-  auto tile_len = [&](int p) {
-    const int c = A.reverse ? nchunks - 1 - p : p;
-    return p < nchunks ? min(kC, len - c * kC) : 0;
-  };
+
 
   // Waves 0-3 own the state (a 16x16 block per wave and slot), waves 4-11 feed them: a single wave issues an
   // instruction every five to eight cycles, so the kinds of work sit on different waves of each SIMD instead
@@ -80,9 +79,9 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
   // All roles pass the same barriers, one per step; steps -2 and -1 fill the pipeline.
   if (w >= 4) {
     // ---------------------------------------------------------------- staging role
-    // Items of a thread: (token pair, 8 columns).  The key items start at staging thread 0, the value items at
-    // thread 64, the items of b at thread 128 (both wrap around) and the last wave turns the gates of a tile
-    // into its weights.  Byte offsets of the two tokens from the first row of a tile and word offsets in the
+    // Items of a thread: (token pair, 8 columns).  The key and the value items start at thread 0 of the group,
+    // the items of b follow those of v (wrapping around), and the last wave turns the gates of a tile into its
+    // weights (in the step in which the group stages nothing).  Byte offsets of the two tokens from the first row of a tile and word offsets in the
     // staging tiles do not change from tile to tile.
     const int grp = (w - 4) >> 2;           // parity of the tiles this group stages
     const int wg = (w - 4) & 3;             // wave in the group
@@ -97,60 +96,65 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
       kval[j] = idx < 32 * gk;
       ksp[j] = idx / gk;
       const int c8 = idx - ksp[j] * gk;
-      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * H * dk + 8 * c8) * 2) : 0u;
-      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * H * dk + 8 * c8) * 2) : 0u;
+      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * H * dk + 8 * c8) * 2) : 0x80000000u;
+      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * H * dk + 8 * c8) * 2) : 0x80000000u;
       kdst[j] = (uint32_t)(8 * c8 * (kStTS / 2) + ksp[j]);
     }
-    const int vtid = (st + 192) & 255, btid = (st + 128) & 255;
+    const int vtid = st, btid = (st + 256 - 32 * gv) & 255;
     const bool vval = vtid < 32 * gv, bval = HAS_J && btid < 32 * gv;
     const int vsp = vtid / gv, vc8 = vtid - vsp * gv, bsp = btid / gv, bc8 = btid - bsp * gv;
     uint32_t voff[2], boff[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      voff[u] = vval ? (uint32_t)(((2 * vsp + u) * H * dv + 8 * vc8) * 2) : 0u;
-      boff[u] = bval ? (uint32_t)(((2 * bsp + u) * H * dv + 8 * bc8) * 2) : 0u;
+      voff[u] = vval ? (uint32_t)(((2 * vsp + u) * H * dv + 8 * vc8) * 2) : 0x80000000u;
+      boff[u] = bval ? (uint32_t)(((2 * bsp + u) * H * dv + 8 * bc8) * 2) : 0x80000000u;
     }
     const uint32_t vdst = (uint32_t)(8 * vc8 * (kStTS / 2) + vsp), bdst = (uint32_t)(8 * bc8 * (kStTS / 2) + bsp);
-    const char* kbase = (const char*)((const bf16_t*)a.k + ((int64_t)bos * H + h) * dk);
-    const char* vbase = (const char*)((const bf16_t*)a.v + ((int64_t)bos * H + h) * dv + d0);
-    const char* bbase = HAS_J ? (const char*)((const bf16_t*)a.b + ((int64_t)bos * H + h) * dv + d0) : nullptr;
+    // Rows are fetched through buffer descriptors that end with the last row of the sequence: the byte offset
+    // of a row piece is a per-thread constant plus the offset of the tile, rows beyond the end of the sequence
+    // (the tail of its last tile, tiles past its end) are out of range and read as zero, so no fetch needs a
+    // branch or a select.  Nothing touches a fetched value before it goes to LDS: any use here would make the
+    // wave wait for everything it has in flight, which is what fetching ahead is meant to avoid.
+    const bf16_t* kbase = (const bf16_t*)a.k + ((int64_t)bos * H + h) * dk;
+    const bf16_t* vbase = (const bf16_t*)a.v + ((int64_t)bos * H + h) * dv + d0;
+    const int esz = a.gate_bf16 ? 2 : 4;
+    const uint32_t kbytes = len > 0 ? (uint32_t)(((len - 1) * H * dk + dk) * 2) : 0u;
+    const uint32_t vbytes = len > 0 ? (uint32_t)(((len - 1) * H * dv + ds) * 2) : 0u;
+    const uint32_t gbytes = len > 0 ? (uint32_t)(((len - 1) * H + 1) * esz) : 0u;
+    const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, kbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, vbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+        HAS_J ? (void*)((const bf16_t*)a.b + ((int64_t)bos * H + h) * dv + d0) : (void*)vbase, 0, vbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t grs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const char*)a.gt + ((int64_t)bos * H + h) * esz), 0, gbytes, 0x00020000);
+    const uint32_t goff = (uint32_t)(lane * H * esz);
     const float gh = a.g[h] * kLog2e;
     const bool from_start = (a.flags & kFlagDecayFromStart) != 0;
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
-    // Fetches are issued without a branch and without touching the result: a row beyond the end of a tile is
-    // fetched from the tile's first row (a tile past the end of the sequence: from the start of the tensor) and
-    // zeroed when the registers go to LDS.  Any use of a fetched value here would make the wave wait for
-    // everything it has in flight, which is what fetching ahead is meant to avoid.
     auto load_stage = [&](StageRegs<NIK>& R, int p) {
       const int c = A.reverse ? nchunks - 1 - p : p;
-      const int clen = tile_len(p);
-      const bool live = clen > 0, full = clen == kC;
-      const int64_t tb = live ? (int64_t)c * kC : 0;
-      const char* kt = live ? kbase + tb * H * dk * 2 : (const char*)a.k;
-      const char* vt = live ? vbase + tb * H * dv * 2 : (const char*)a.v;
-      const char* bt = live ? bbase + tb * H * dv * 2 : (const char*)a.b;
+      const bool live = p < nchunks;
+      // a tile past the end: every offset out of range
+      const uint32_t tk = live ? (uint32_t)(c * kC * H * dk * 2) : 0x80000000u;
+      const uint32_t tv = live ? (uint32_t)(c * kC * H * dv * 2) : 0x80000000u;
 #pragma unroll
       for (int j = 0; j < NIK; ++j) {
-        R.k[j][0] = *(const u32x4*)(kt + ((full || 2 * ksp[j] < clen) ? koff[j][0] : 0u));
-        R.k[j][1] = *(const u32x4*)(kt + ((full || 2 * ksp[j] + 1 < clen) ? koff[j][1] : 0u));
+        R.k[j][0] = __builtin_amdgcn_raw_buffer_load_b128(krs, koff[j][0] + tk, 0, 0);
+        R.k[j][1] = __builtin_amdgcn_raw_buffer_load_b128(krs, koff[j][1] + tk, 0, 0);
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        R.v[u] = *(const u32x4*)(vt + ((full || 2 * vsp + u < clen) ? voff[u] : 0u));
-        if (HAS_J) R.b[u] = *(const u32x4*)(bt + ((full || 2 * bsp + u < clen) ? boff[u] : 0u));
+        R.v[u] = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff[u] + tv, 0, 0);
+        if (HAS_J) R.b[u] = __builtin_amdgcn_raw_buffer_load_b128(brs, boff[u] + tv, 0, 0);
       }
       if (wg == 3) {
-        const int64_t gi = (lane < clen) ? (bos + tb + lane) * H + h : 0;
-        R.gt = a.gate_bf16 ? (uint32_t)((const uint16_t*)a.gt)[gi] : ((const uint32_t*)a.gt)[gi];   // raw; widened below
+        const uint32_t tg = live ? (uint32_t)(c * kC * H * esz) : 0x80000000u;
+        R.gt = a.gate_bf16 ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(grs, goff + tg, 0, 0)
+                           : __builtin_amdgcn_raw_buffer_load_b32(grs, goff + tg, 0, 0);   // raw; widened below
       }
     };
     // eight columns of two tokens -> one word (token pair) per column
-    auto put = [&](uint32_t* dst, u32x4 x0, u32x4 x1, int sp, int clen) {
-      if (clen < kC) {   // same for the whole workgroup
-        if (2 * sp >= clen) x0 = zero4;
-        if (2 * sp + 1 >= clen) x1 = zero4;
-      }
+    auto put = [&](uint32_t* dst, const u32x4& x0, const u32x4& x1) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
@@ -159,11 +163,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
     };
     // the same for rows of v and b, which are staged times the weight of their token (the operand the matrix
     // cores take is a_s v_s, rounded to bf16 once)
-    auto put_weighted = [&](uint32_t* dst, u32x4 x0, u32x4 x1, int sp, int clen, const float* wts) {
-      if (clen < kC) {
-        if (2 * sp >= clen) x0 = zero4;
-        if (2 * sp + 1 >= clen) x1 = zero4;
-      }
+    auto put_weighted = [&](uint32_t* dst, const u32x4& x0, const u32x4& x1, int sp, const float* wts) {
       const f32x2 a2 = *(const f32x2*)&wts[2 * sp];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -174,19 +174,17 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
       }
     };
     auto store_stage = [&](const StageRegs<NIK>& R, int buf, int p) {
-      const int clen = tile_len(p);
 #pragma unroll
       for (int j = 0; j < NIK; ++j)
-        if (kval[j]) put(sKT + buf * kbuf + kdst[j], R.k[j][0], R.k[j][1], ksp[j], clen);
+        if (kval[j]) put(sKT + buf * kbuf + kdst[j], R.k[j][0], R.k[j][1]);
       const float* wts = sA + (p % 3) * kC;
-      if (vval) put_weighted(sVT + buf * vbuf + vdst, R.v[0], R.v[1], vsp, clen, wts);
-      if (HAS_J && bval) put_weighted(sBT + buf * vbuf + bdst, R.b[0], R.b[1], bsp, clen, wts);
+      if (vval) put_weighted(sVT + buf * vbuf + vdst, R.v[0], R.v[1], vsp, wts);
+      if (HAS_J && bval) put_weighted(sBT + buf * vbuf + bdst, R.b[0], R.b[1], bsp, wts);
     };
     // weights of the tokens of tile p and the decay over the whole tile, one step before its rows are staged
     auto scan_stage = [&](const StageRegs<NIK>& R, int p) {
       if (wg == 3) {
-        const int clen = tile_len(p);
-        const float gt = (lane < clen) ? __builtin_bit_cast(float, a.gate_bf16 ? R.gt << 16 : R.gt) : 0.f;
+        const float gt = __builtin_bit_cast(float, a.gate_bf16 ? R.gt << 16 : R.gt);   // zero beyond the sequence
         const float cs = wave_inclusive_scan(-gt * gh, lane);
         const float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cs), 63));
         sA[(p % 3) * kC + lane] = fast_exp2(from_start ? cs : tot - cs);
@@ -198,21 +196,29 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
     // fetched three steps before its rows go to LDS.  In step p the group of parity (p + 1) & 1 stages tile p + 1,
     // the other one handles tile p + 2: weights from its gates (set (p + 2) / 2 % 2), then the fetch of tile p + 4
     // into the set that was staged a step ago.
-    StageRegs<NIK> R[2];
-    load_stage(R[0], grp);
-    for (int p0 = -2; p0 < nchunks; p0 += 4) {
+    // (One copy of the loop per group: with the group a compile-time constant the order of fetches and uses is
+    // static, and the compiler can count how many younger fetches may still be in flight when a set is used;
+    // with a run-time test it has to wait for all of them, which throws the fetching ahead away.)
+    auto run = [&](auto parity) {
+      constexpr int G = decltype(parity)::value;
+      StageRegs<NIK> R[2];
+      load_stage(R[0], G);
+      for (int p0 = -2; p0 < nchunks; p0 += 4) {
 #pragma unroll
-      for (int ph = 0; ph < 4; ++ph) {
-        const int p = p0 + ph;           // p + 2 = ph (mod 4)
-        if ((ph & 1) == grp) {
-          scan_stage(R[(ph >> 1) & 1], p + 2);
-          load_stage(R[1 - ((ph >> 1) & 1)], p + 4);
-        } else if (p + 1 >= 0) {
-          store_stage(R[(((ph + 3) & 3) >> 1) & 1], grp, p + 1);
+        for (int ph = 0; ph < 4; ++ph) {
+          const int p = p0 + ph;           // p + 2 = ph (mod 4)
+          if ((ph & 1) == G) {   // folds once the loop is unrolled
+            scan_stage(R[(ph >> 1) & 1], p + 2);
+            load_stage(R[1 - ((ph >> 1) & 1)], p + 4);
+          } else {
+            if (p + 1 >= 0) store_stage(R[(((ph + 3) & 3) >> 1) & 1], G, p + 1);
+          }
+          __syncthreads();
         }
-        __syncthreads();
       }
-    }
+    };
+    if (grp == 0) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
     return;
   }
 
@@ -339,12 +345,12 @@ static int launch_state_pass_j(const StatePassArgs& A, int kern_id, unsigned gri
 bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j) {
   if (dtype != PAL_DTYPE_BF16 || g_state_pass_mode == 1) return false;
   if (a.dk < 16 || a.dk > 256 || a.dk % 16 || a.dv % 16) return false;
+  // rows are addressed with 32-bit byte offsets from the first row of a sequence
+  if ((int64_t)a.T * a.H * (a.dk > a.dv ? a.dk : a.dv) * 2 >= 0x7fffffffLL) return false;
   if (g_state_pass_mode == 2) return true;
-  // Measured on MI355X: a workgroup needs about 0.8 us per tile whatever the head dims, so the one-pass form
-  // pays where the per-tile contributions are large (their fp32 round trip is what it saves) and a few
-  // hundred workgroups exist; with the precision state and 64x64 heads the two-kernel form is as fast.
-  if ((int64_t)a.n_seqs * a.H * (a.dv / 16) < 192) return false;
-  return !has_j || (int64_t)a.dk * a.dv >= 8192;
+  // The walk over the tiles is serial per workgroup (0.4-0.7 us per tile): with fewer workgroups than this the
+  // two-kernel form, which spreads the tiles over the whole GPU, is faster.
+  return (int64_t)a.n_seqs * a.H * (a.dv / 16) >= 192;
 }
 
 // tiles_a / tiles_b, init_*, fin_*: see StatePassArgs.  reverse walks every sequence from its last tile.
@@ -357,12 +363,14 @@ int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tile
   A.init_a = init_a; A.init_b = init_b; A.fin_a = fin_a; A.fin_b = fin_b;
   A.reverse = reverse ? 1 : 0;
   A.fin_scale = fin_scale;
-  // value rows per workgroup: the largest slice that still gives the GPU a few hundred workgroups
+  // value rows per workgroup: the largest slice that still gives three quarters of the compute units a
+  // workgroup (measured: wider slices stage the key rows for more state at the same cost per tile; with
+  // fewer workgroups than that the idle units cost more)
   int ds = 16;
   const int cand[3] = {64, 48, 32};
   for (int c : cand) {
-    if (a.dv % c || c * a.dk > 4096) continue;
-    if ((int64_t)a.n_seqs * a.H * (a.dv / c) >= 512) { ds = c; break; }
+    if (a.dv % c || c * a.dk > 256 * 4 * kStMaxBlocks) continue;
+    if ((int64_t)a.n_seqs * a.H * (a.dv / c) >= 192) { ds = c; break; }
   }
   A.ds = ds;
   A.nsplit = a.dv / ds;
