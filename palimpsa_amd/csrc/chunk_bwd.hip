@@ -43,7 +43,7 @@ struct BwdArgs {
   const void *d_o, *d_o_var;
   void *dq, *dk, *dv, *db;
   float *dgt, *dg, *dIp, *d_init_mu, *d_init_I;
-  float *wDM, *wDJ;       // [total_chunks,H,dv,dk] local carries, then incoming carries
+  void *wDM, *wDJ;        // [total_chunks,H,dv,dk] local carries, then incoming carries, in the dtype of the rows
   float* wFtot;           // [total_chunks,H] log2 of the total decay of a tile
   float* wSig;            // [total_chunks,H] sum over the tile of dJloc
   float* wBnd;            // [total_chunks,H] F_C <carry, state at the start of the tile>
@@ -389,8 +389,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
       }
     }
     const float f_first = fast_exp2(sC[0]);
-    float* wDM = A.wDM + tile_off + 16 * nb;
-    float* wDJ = A.wDJ + tile_off + 16 * nb;
+    // the carries between tiles are kept in the dtype of the rows: bf16 rows feed them to the matrix cores in bf16
+    // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers
+    TIn* wDM = (TIn*)A.wDM + tile_off + 16 * nb;
+    TIn* wDJ = (TIn*)A.wDJ + tile_off + 16 * nb;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
     float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
 
@@ -451,8 +453,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             // carry handed to the previous tile: f_first * dM^loc at the first token
             const f32x4 rm = {f_first * aM[0], f_first * aM[1], f_first * aM[2], f_first * aM[3]};
             const f32x4 rj = {f_first * aJ[0], f_first * aJ[1], f_first * aJ[2], f_first * aJ[3]};
-            *(f32x4*)&(wDM + (int64_t)d * dk)[4 * g] = rm;
-            *(f32x4*)&(wDJ + (int64_t)d * dk)[4 * g] = rj;
+            store_vec<4>(wDM + (int64_t)d * dk + 4 * g, (const float*)&rm);
+            store_vec<4>(wDJ + (int64_t)d * dk + 4 * g, (const float*)&rj);
           }
         }
         pw[dd * kC] = rows4_sum_x4(dvp[0], dvp[1], dbp[0], dbp[1]);
@@ -512,38 +514,72 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 }
 
 // ----------------------------------------------------------------- carry scan
-// one thread per (sequence, head, state entry); 256 consecutive entries per block
+// R_{c-1} = R_loc,c + F_c R_c backwards over the tiles of a sequence: one thread per four consecutive state
+// entries of a (sequence, head), 1024 entries per block; the running sums stay in fp32 registers, the slot of a
+// tile is read (its local carry) and overwritten (the carry coming in from the later tiles) in the row dtype.
+__host__ __device__ inline int carry_scan_blocks(int64_t E) { return (int)((E + 1023) / 1024); }
+
+template <typename TC>
 __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   __shared__ float sW[4];
   const int64_t E = (int64_t)a.dv * a.dk;
-  const int nblk = (int)(E / 256);
+  const int nblk = carry_scan_blocks(E);
   const int blk = blockIdx.x % nblk;
   const int nh = blockIdx.x / nblk;
   const int h = nh % a.H, n = nh / a.H;
-  const int64_t e = (int64_t)blk * 256 + threadIdx.x;
+  const int64_t e = ((int64_t)blk * 256 + threadIdx.x) * 4;
+  const bool on = e < E;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const int nchunks = (len + kC - 1) / kC;
-  float RM = 0.f, RJ = 0.f;
-  for (int c = nchunks - 1; c >= 0; --c) {
-    const int64_t off = ((int64_t)(cbase + c) * a.H + h) * E + e;
-    const float DM = A.wDM[off], DJ = A.wDJ[off];
-    const float Ft = fast_exp2(A.wFtot[(int64_t)(cbase + c) * a.H + h]);
-    A.wDM[off] = RM;
-    A.wDJ[off] = RJ;
-    RM = fmaf(Ft, RM, DM);
-    RJ = fmaf(Ft, RJ, DJ);
+  TC* wDM = (TC*)A.wDM;
+  TC* wDJ = (TC*)A.wDJ;
+  float RM[4] = {0.f, 0.f, 0.f, 0.f}, RJ[4] = {0.f, 0.f, 0.f, 0.f};
+  if (on) {
+    auto advance = [&](int64_t off, const float* DM, const float* DJ, float Ft) {
+      store_vec<4>(wDM + off, RM);
+      store_vec<4>(wDJ + off, RJ);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        RM[x] = fmaf(Ft, RM[x], DM[x]);
+        RJ[x] = fmaf(Ft, RJ[x], DJ[x]);
+      }
+    };
+    int c = nchunks - 1;
+    for (; c >= 3; c -= 4) {   // four tiles' loads in flight at a time
+      float DM[4][4], DJ[4][4], Ft[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t off = ((int64_t)(cbase + c - u) * a.H + h) * E + e;
+        load_vec<4>(wDM + off, DM[u]);
+        load_vec<4>(wDJ + off, DJ[u]);
+        Ft[u] = A.wFtot[(int64_t)(cbase + c - u) * a.H + h];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        advance(((int64_t)(cbase + c - u) * a.H + h) * E + e, DM[u], DJ[u], fast_exp2(Ft[u]));
+    }
+    for (; c >= 0; --c) {
+      const int64_t off = ((int64_t)(cbase + c) * a.H + h) * E + e;
+      float DM[4], DJ[4];
+      load_vec<4>(wDM + off, DM);
+      load_vec<4>(wDJ + off, DJ);
+      advance(off, DM, DJ, fast_exp2(A.wFtot[(int64_t)(cbase + c) * a.H + h]));
+    }
   }
   if (a.init_mu) {
     const int64_t so = (int64_t)nh * E + e;
-    if (A.d_init_mu) {
-      const float mu0 = a.init_mu[so], I0 = a.init_I[so];
-      A.d_init_mu[so] = RM * I0;
-      A.d_init_I[so] = fmaf(RM, mu0, RJ);
+    if (A.d_init_mu && on) {
+      const f32x4 mu0 = *(const f32x4*)(a.init_mu + so), I0 = *(const f32x4*)(a.init_I + so);
+      const f32x4 dmu = {RM[0] * I0[0], RM[1] * I0[1], RM[2] * I0[2], RM[3] * I0[3]};
+      const f32x4 dI = {fmaf(RM[0], mu0[0], RJ[0]), fmaf(RM[1], mu0[1], RJ[1]), fmaf(RM[2], mu0[2], RJ[2]),
+                        fmaf(RM[3], mu0[3], RJ[3])};
+      *(f32x4*)(A.d_init_mu + so) = dmu;
+      *(f32x4*)(A.d_init_I + so) = dI;
     }
     // J_0 = I_0 - Ip: the prior also receives -sum dJ_0
-    float s = wave_sum(RJ);
+    float s = wave_sum((RJ[0] + RJ[1]) + (RJ[2] + RJ[3]));
     if ((threadIdx.x & 63) == 0) sW[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) A.wInitPart[(int64_t)nh * nblk + blk] = sW[0] + sW[1] + sW[2] + sW[3];
@@ -598,8 +634,8 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     if (lane == 0) sW4[4] = fast_exp2(tot);
   }
   const int64_t E = (int64_t)dv * dk;
-  const float* RM = A.wDM + ((int64_t)cidx * H + h) * E;
-  const float* RJ = A.wDJ + ((int64_t)cidx * H + h) * E;
+  const TIn* RM = (const TIn*)A.wDM + ((int64_t)cidx * H + h) * E;
+  const TIn* RJ = (const TIn*)A.wDJ + ((int64_t)cidx * H + h) * E;
   {
     // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile; the same
     // pass leaves R^T in LDS for the products that contract over the value rows
@@ -615,7 +651,9 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       if (blk >= nblk) break;
       const int d = 16 * (blk / nc) + i, c4 = 4 * (blk % nc) + g;
       const int64_t e = (int64_t)d * dk + 4 * c4;
-      const f32x4 rm = *(const f32x4*)(RM + e), rj = *(const f32x4*)(RJ + e);
+      float rm[4], rj[4];
+      load_vec<4>(RM + e, rm);
+      load_vec<4>(RJ + e, rj);
       const f32x4 mu = *(const f32x4*)(smu + e), I = *(const f32x4*)(sI + e);
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
@@ -771,14 +809,15 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
                 if (doB) B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i];
               }
             } else if (n0 < dk) {
-              const float* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
-              const float* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
-              const f32x4 x0 = *(const f32x4*)r1, x1 = *(const f32x4*)(r1 + 4);
-              const f32x4 y0 = *(const f32x4*)r2, y1 = *(const f32x4*)(r2 + 4);
+              const TIn* r1 = RM + (int64_t)(16 * db_ + i) * dk + n0;
+              const TIn* r2 = RJ + (int64_t)(16 * db_ + i) * dk + n0;
+              float x[8], y[8];
+              load_vec<4>(r1, x); load_vec<4>(r1 + 4, x + 4);
+              load_vec<4>(r2, y); load_vec<4>(r2 + 4, y + 4);
 #pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                B1[j] = (bf16_t)x0[j]; B1[j + 4] = (bf16_t)x1[j];
-                B2[j] = (bf16_t)y0[j]; B2[j + 4] = (bf16_t)y1[j];
+              for (int j = 0; j < 8; ++j) {
+                B1[j] = (bf16_t)x[j];
+                B2[j] = (bf16_t)y[j];
               }
             }
             if (doV) accV = mfma16(A1[ks], B1, accV);
@@ -872,7 +911,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_gate_kernel(BwdArgs A) {
     double s = 0.0;
     for (int c = 0; c < nchunks; ++c) s += (double)A.wSig[(int64_t)(cbase + c) * a.H + h];
     if (a.init_mu) {
-      const int nblk = (int)(((int64_t)a.dv * a.dk) / 256);
+      const int nblk = carry_scan_blocks((int64_t)a.dv * a.dk);
       for (int b2 = 0; b2 < nblk; ++b2) s -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
     }
     A.wDIpPart[(int64_t)n * a.H + h] = s;
@@ -1008,7 +1047,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   A.dgt = gr->dgt; A.dg = gr->dg; A.dIp = gr->dIp;
   A.d_init_mu = gr->d_init_mu; A.d_init_I = gr->d_init_I;
   char* ws = (char*)workspace;
-  A.wDM = (float*)(ws + L.oDM); A.wDJ = (float*)(ws + L.oDJ);
+  A.wDM = ws + L.oDM; A.wDJ = ws + L.oDJ;
   A.wFtot = (float*)(ws + L.oFtot); A.wSig = (float*)(ws + L.oSig); A.wBnd = (float*)(ws + L.oBnd);
   A.wE = (float*)(ws + L.oE); A.wBc = (float*)(ws + L.oBc); A.wInitPart = (float*)(ws + L.oInit);
   A.wDgPart = (double*)(ws + L.oDg); A.wDIpPart = (double*)(ws + L.oDIp);
@@ -1018,9 +1057,10 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   rc = bf ? launch_local<bf16_t>(A, s) : launch_local<float>(A, s);
   if (rc) return rc;
   {
-    const int64_t blocks = (int64_t)dd.n_seqs * dd.n_heads * (((int64_t)dd.dv * dd.dk) / 256);
+    const int64_t blocks = (int64_t)dd.n_seqs * dd.n_heads * carry_scan_blocks((int64_t)dd.dv * dd.dk);
     if (blocks > 0x7fffffff) return PAL_E_DIM;
-    PAL_TIMED_LAUNCH(kKernBwdCarryScan, s, chunk_bwd_carry_scan_kernel, dim3((unsigned)blocks), dim3(256), 0, s, A);
+    if (bf) PAL_TIMED_LAUNCH(kKernBwdCarryScan, s, chunk_bwd_carry_scan_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, s, A);
+    else PAL_TIMED_LAUNCH(kKernBwdCarryScan, s, chunk_bwd_carry_scan_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, A);
     PAL_HIP_LAUNCH_CHECK();
   }
   {
