@@ -296,16 +296,21 @@ constexpr int kDG = 16;  // value rows per staging group
 // index of the L operand for (tb, ks): tb0,tb1 -> one K step; tb2,tb3 -> two
 __device__ __forceinline__ constexpr int lidx(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
 
-template <typename TIn, int NB, bool HAS_VAR>
-__global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
+// RS > 1 splits the value rows of a group among RS waves per column block (wave = (column block, rows dd = rs mod RS)).
+// The hardware puts wave i of a workgroup on SIMD i mod 4, so a workgroup of 5, 6 or 7 waves loads the SIMDs 2:1:1:1 or
+// 2:2:1:1 and this kernel, which is bound by vector issue, then runs at the pace of the busiest SIMD (measured: the same
+// time for 5, 6, 7 and 8 column blocks).  With two waves per column block the waves spread evenly.
+template <typename TIn, int NB, bool HAS_VAR, int RS>
+__global__ __launch_bounds__(NB * RS * 64) void chunk_out_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
   float* sC = smem;                       // [64] running log2-decay inside the tile
   f16_t* sV = (f16_t*)(sC + kC);          // [2][16][kVH] v^T 2^-E of the current and the next value-row group, f16
   f16_t* sB = sV + 2 * kDG * kVH;         // [2][16][kVH] b^T 2^-E
   float* sO = (float*)(sB + 2 * kDG * kVH);   // [NB][16][64] per-wave partial outputs
   float* sOv = sO + NB * kDG * kC;        // same for o_var
-  constexpr int NT = NB * 64;
-  const int tid = threadIdx.x, lane = tid & 63, nb = tid >> 6, i = lane & 15, g = lane >> 4;
+  constexpr int NT = NB * RS * 64;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int nb = (tid >> 6) % NB, rs = (tid >> 6) / NB;
   const int H = a.H, dk = a.dk, dv = a.dv;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
@@ -313,7 +318,7 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
   const float Ip = a.Ip[h];
   const float gh = a.g[h] * kLog2e;
 
-  if (nb == 0) {
+  if (tid < 64) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     sC[lane] = wave_inclusive_scan(-gt * gh, lane);
   }
@@ -420,20 +425,20 @@ __global__ __launch_bounds__(NB * 64) void chunk_out_kernel(ChunkArgs a) {
   const float* cI = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
 
   // tile-start state of the next value row is fetched one iteration ahead
-  f32x4 mu0_n = *(const f32x4*)cmu, I0_n = *(const f32x4*)cI;
+  f32x4 mu0_n = *(const f32x4*)(cmu + (int64_t)rs * dk), I0_n = *(const f32x4*)(cI + (int64_t)rs * dk);
   const int n_groups = dv / kDG;
   for (int dg = 0; dg < n_groups; ++dg) {
     const int buf = dg & 1;
-    for (int dd = 0; dd < kDG; ++dd) {
+    for (int dd = rs; dd < kDG; dd += RS) {
       const int d = dg * kDG + dd;
-      if (dd == kDG / 2 && dg + 1 < n_groups) {
+      if (dd - rs == kDG / 2 && dg + 1 < n_groups) {
         // rows of the next group go to the other buffer mid-group (read only after the barriers below)
         stage_load(dg + 1);
         stage_store(buf ^ 1);
       }
       const f32x4 mu0 = mu0_n, I0 = I0_n;
       {
-        const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
+        const int64_t dn = (int64_t)min(d + RS, dv - 1) * dk;
         mu0_n = *(const f32x4*)(cmu + dn);
         I0_n = *(const f32x4*)(cI + dn);
       }
@@ -509,12 +514,15 @@ static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;
+  // waves per column block, see chunk_out_kernel (7 blocks x 2 would need 128 VGPRs per wave and spills; with 1-3
+  // blocks several workgroups share a compute unit and the repeated per-wave set-up costs more than the balance gains)
+  constexpr int RS = (NB == 5 || NB == 6) ? 2 : 1;
   if (var) {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true, RS>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true, RS>), dim3((unsigned)blocks), dim3(NB * RS * 64), lds, s, a);
   } else {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false>), dim3((unsigned)blocks), dim3(NB * 64), lds, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false, RS>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false, RS>), dim3((unsigned)blocks), dim3(NB * RS * 64), lds, s, a);
   }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
