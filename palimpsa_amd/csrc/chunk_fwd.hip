@@ -310,7 +310,7 @@ __global__ __launch_bounds__(NB * RS * 64) void chunk_out_kernel(ChunkArgs a) {
   float* sOv = sO + NB * kDG * kC;        // same for o_var
   constexpr int NT = NB * RS * 64;
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
-  const int nb = (tid >> 6) % NB, rs = (tid >> 6) / NB;
+  const int nb = RS == 1 ? (tid >> 6) : (tid >> 6) % NB, rs = RS == 1 ? 0 : (tid >> 6) / NB;
   const int H = a.H, dk = a.dk, dv = a.dv;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
