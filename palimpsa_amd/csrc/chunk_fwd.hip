@@ -300,19 +300,28 @@ __device__ __forceinline__ constexpr int lidx(int tb, int ks) { return tb < 2 ? 
 // The hardware puts wave i of a workgroup on SIMD i mod 4, so a workgroup of 5, 6 or 7 waves loads the SIMDs 2:1:1:1 or
 // 2:2:1:1 and this kernel, which is bound by vector issue, then runs at the pace of the busiest SIMD (measured: the same
 // time for 5, 6, 7 and 8 column blocks).  With two waves per column block the waves spread evenly.
-template <typename TIn, int NB, bool HAS_VAR, int RS>
-__global__ __launch_bounds__(NB * RS * 64) void chunk_out_kernel(ChunkArgs a) {
+// TS > 1 gives a workgroup TS (tile, head) pairs, each with its own NB * RS waves and its own piece of LDS (they only
+// share the barriers), so that a workgroup of two waves becomes one of four and covers all four SIMDs.
+template <typename TIn, int NB, bool HAS_VAR, int RS, int TS>
+__global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
-  float* sC = smem;                       // [64] running log2-decay inside the tile
+  constexpr int NT = NB * RS * 64;        // threads per (tile, head)
+  constexpr int kTileFloats = kC + (HAS_VAR ? 2 : 1) * NB * kDG * kC + (4 * kDG * kVH) / 2;
+  const int sub = TS == 1 ? 0 : (int)threadIdx.x / NT;
+  const int tid = (int)threadIdx.x - sub * NT;
+  const int64_t n_items = (int64_t)a.total_chunks * a.H;
+  const int64_t item_raw = (int64_t)blockIdx.x * TS + sub;
+  const bool valid = item_raw < n_items;          // a spare group of the last workgroup repeats the last item, unstored
+  const int64_t item = valid ? item_raw : n_items - 1;
+  float* sC = smem + sub * kTileFloats;   // [64] running log2-decay inside the tile
   f16_t* sV = (f16_t*)(sC + kC);          // [2][16][kVH] v^T 2^-E of the current and the next value-row group, f16
   f16_t* sB = sV + 2 * kDG * kVH;         // [2][16][kVH] b^T 2^-E
   float* sO = (float*)(sB + 2 * kDG * kVH);   // [NB][16][64] per-wave partial outputs
   float* sOv = sO + NB * kDG * kC;        // same for o_var
-  constexpr int NT = NB * RS * 64;
-  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int nb = RS == 1 ? (tid >> 6) : (tid >> 6) % NB, rs = RS == 1 ? 0 : (tid >> 6) / NB;
   const int H = a.H, dk = a.dk, dv = a.dv;
-  const int cidx = blockIdx.x / H, h = blockIdx.x % H;
+  const int cidx = (int)(item / H), h = (int)(item % H);
   int seq, t0, clen, cis;
   chunk_lookup(a, cidx, seq, t0, clen, cis);
   const float Ip = a.Ip[h];
@@ -484,7 +493,7 @@ __global__ __launch_bounds__(NB * RS * 64) void chunk_out_kernel(ChunkArgs a) {
     // flush the group's outputs: work item = (token t, 4 value rows)
     for (int idx = tid; idx < kC * kDG / 4; idx += NT) {
       const int t = idx >> 2, dq = idx & 3;
-      if (t < clen) {
+      if (t < clen && valid) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f}, accv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < NB; ++w)
@@ -517,12 +526,16 @@ static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
   // waves per column block, see chunk_out_kernel (7 blocks x 2 would need 128 VGPRs per wave and spills; with 1-3
   // blocks several workgroups share a compute unit and the repeated per-wave set-up costs more than the balance gains)
   constexpr int RS = (NB == 5 || NB == 6) ? 2 : 1;
+  // (tile, head) pairs per workgroup, see chunk_out_kernel (measured: +9 % at two column blocks, nothing at one or three)
+  constexpr int TS = NB == 2 ? 2 : 1;
+  const size_t lds_all = lds * TS;
+  const unsigned grid = (unsigned)((blocks + TS - 1) / TS);
   if (var) {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true, RS>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true, RS>), dim3((unsigned)blocks), dim3(NB * RS * 64), lds, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true, RS, TS>, lds_all)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true, RS, TS>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
   } else {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false, RS>, lds)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false, RS>), dim3((unsigned)blocks), dim3(NB * RS * 64), lds, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false, RS, TS>, lds_all)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false, RS, TS>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
   }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
