@@ -198,3 +198,18 @@ def test_entry_point_under_torch_compile(gpu_device):
     compiled = run(torch.compile(f, backend="eager"))     # the tracer only: no code generation involved
     for a, b_ in zip(eager, compiled):
         assert hp.max_rel(b_, a) <= 1e-6
+
+
+@pytest.mark.parametrize("dk,dv", [(96, 64), (80, 48), (32, 32)])
+def test_output_kernel_wave_layouts_with_uncertainty(gpu_device, dk, dv):
+    """Head dims whose forward output kernel runs two waves per column block (dk = 80, 96) or two (tile, head) pairs
+    per workgroup (dk = 32; 3 tiles x 3 heads = an odd number of pairs, so the last workgroup has a spare group)."""
+    ck, _ = _ops()
+    B, T, H = 1, 150, 3
+    inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=dk + dv), torch.bfloat16)
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, want_var=True)
+    d = hp.to_device(inp, gpu_device)
+    (o, ov), mu, I = _call(ck, d, output_final_state=True, output_uncertainty=True)
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_abs(ov, ov_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
