@@ -50,7 +50,7 @@ struct BwdArgs {
   float* wE;              // [H, tokens]  local part of d log f
   float* wBc;             // [H, tokens]  beta_r of the carry terms
   float* wInitPart;       // [n_seqs,H,dv*dk/256] partial sums of dJ_0
-  double *wDgPart, *wDIpPart;  // [n_seqs,H]
+  double *wDgPart, *wDIpPart;  // [n_seqs,H,pieces of the gate pass], [n_seqs,H]
   int32_t tokens;
   int32_t apply_alias;     // carry apply: db^carry shares LDS with the bf16 carries (large head dims)
 };
@@ -877,19 +877,24 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
 }
 
 // ----------------------------------------------------------------- gate pass
-// one block per (sequence, head); a wave per tile: local part + prefix of the carry terms + boundary term
+// one block per (sequence, head, piece of kGateTokens tokens); a wave per tile: local part + prefix of the carry
+// terms + boundary term.  The pieces only share the sums dg and dIp, which leave as per-block shares.
+constexpr int kGateTokens = 512;
+__host__ __device__ inline int gate_pieces(int max_len) { return (max_len + kGateTokens - 1) / kGateTokens; }
+
 __global__ __launch_bounds__(256) void chunk_bwd_gate_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   __shared__ double sG[4];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int h = blockIdx.x % a.H, n = blockIdx.x / a.H;
+  const int piece = blockIdx.y, n_pieces = gridDim.y;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const float gh = a.g[h];
   double dg_acc = 0.0;
   const int nchunks = (len + kC - 1) / kC;
-  const int nseg = (len + 255) / 256;
-  for (int seg = 0; seg < nseg; ++seg) {
+  const int seg0 = piece * (kGateTokens / 256), seg1 = min((len + 255) / 256, seg0 + kGateTokens / 256);
+  for (int seg = seg0; seg < seg1; ++seg) {
     const int t = seg * 256 + tid;
     const bool ok = t < len;
     const float bc = ok ? A.wBc[(int64_t)h * A.tokens + bos + t] : 0.f;
@@ -906,32 +911,42 @@ __global__ __launch_bounds__(256) void chunk_bwd_gate_kernel(BwdArgs A) {
   for (int off = 32; off > 0; off >>= 1) dg_acc += __shfl_xor(dg_acc, off);
   if (lane == 0) sG[w] = dg_acc;
   __syncthreads();
-  if (tid == 0) {
-    A.wDgPart[(int64_t)n * a.H + h] = sG[0] + sG[1] + sG[2] + sG[3];
+  if (tid == 0) A.wDgPart[((int64_t)n * a.H + h) * n_pieces + piece] = sG[0] + sG[1] + sG[2] + sG[3];
+  if (piece == 0 && w == 1) {
+    // dIp share of this (sequence, head): the tiles' terms and, with an initial state, -sum dJ_0
     double s = 0.0;
-    for (int c = 0; c < nchunks; ++c) s += (double)A.wSig[(int64_t)(cbase + c) * a.H + h];
+    for (int c = lane; c < nchunks; c += 64) s += (double)A.wSig[(int64_t)(cbase + c) * a.H + h];
     if (a.init_mu) {
       const int nblk = carry_scan_blocks((int64_t)a.dv * a.dk);
-      for (int b2 = 0; b2 < nblk; ++b2) s -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
+      for (int b2 = lane; b2 < nblk; b2 += 64) s -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
     }
-    A.wDIpPart[(int64_t)n * a.H + h] = s;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (lane == 0) A.wDIpPart[(int64_t)n * a.H + h] = s;
   }
 }
 
-__global__ void chunk_bwd_head_reduce_kernel(BwdArgs A) {
+// dg[h], dIp[h]: one wave per head sums the shares (fixed order: lane-strided, then the lanes)
+__global__ __launch_bounds__(64) void chunk_bwd_head_reduce_kernel(BwdArgs A, int n_pieces) {
   const ChunkArgs& a = A.c;
-  const int h = blockIdx.x * blockDim.x + threadIdx.x;
-  if (h >= a.H) return;
+  const int h = blockIdx.x, lane = threadIdx.x;
   double sg = 0.0, si = 0.0;
-  for (int n = 0; n < a.n_seqs; ++n) {
-    sg += A.wDgPart[(int64_t)n * a.H + h];
-    si += A.wDIpPart[(int64_t)n * a.H + h];
+  for (int j = lane; j < a.n_seqs * n_pieces; j += 64) {
+    const int n = j / n_pieces, pc = j - n * n_pieces;
+    sg += A.wDgPart[((int64_t)n * a.H + h) * n_pieces + pc];
   }
-  A.dg[h] = (float)sg;
-  A.dIp[h] = (float)si;
+  for (int n = lane; n < a.n_seqs; n += 64) si += A.wDIpPart[(int64_t)n * a.H + h];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    sg += __shfl_xor(sg, off);
+    si += __shfl_xor(si, off);
+  }
+  if (lane == 0) {
+    A.dg[h] = (float)sg;
+    A.dIp[h] = (float)si;
+  }
 }
 
-// ------------------------------------------------------------------- host
 struct BwdLayout {
   size_t oDM, oDJ, oFtot, oSig, oBnd, oE, oBc, oInit, oDg, oDIp, total;
 };
@@ -952,7 +967,7 @@ static BwdLayout bwd_layout(const PalDims* d) {
   L.oE = o; o = align256(o + tokens * d->n_heads * 4);
   L.oBc = o; o = align256(o + tokens * d->n_heads * 4);
   L.oInit = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * (E / 256) * 4);
-  L.oDg = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * 8);
+  L.oDg = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * gate_pieces(d->seq_len) * 8);
   L.oDIp = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * 8);
   L.total = o;
   return L;
@@ -1084,9 +1099,11 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
     if (rc) return rc;
     PAL_HIP_LAUNCH_CHECK();
   }
-  PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads)), dim3(256), 0, s, A);
+  const int n_pieces = gate_pieces(dd.seq_len);
+  if (n_pieces > 65535) return PAL_E_DIM;
+  PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads), (unsigned)n_pieces), dim3(256), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
-  PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((dd.n_heads + 63) / 64), dim3(64), 0, s, A);
+  PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((unsigned)dd.n_heads), dim3(64), 0, s, A, n_pieces);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
