@@ -7,7 +7,7 @@
 //   dMloc_t = G_t / I_t,  dJloc_t = -G_t M_t / I_t^2 (- scale dovar_t (q_t*q_t)^T / I_t^2)
 // and the state gradients obey the reverse recurrence dM_s = dMloc_s + f_{s+1} dM_{s+1}
 // (:360-384).  All tiles of 64 tokens are processed in parallel; what crosses a
-// tile boundary is handled by two small extra passes:
+// tile boundary is handled by two small extra passes (scan, apply); the gate gradient is finished in the second:
 //
 //  local   per (tile, head): recompute M_t, I_t from the tile-start state (as the
 //          forward does), form dMloc/dJloc, dq; feed them straight from the MFMA
@@ -28,6 +28,8 @@
 //                         beta_r = <v_r, dv^carry_r> + <b_r, db^carry_r> from the apply pass and
 //                         (M_0, J_0) the state at the start of the tile.
 //          dgt = -g dlogf, dg = -sum gt dlogf, dIp = sum dJloc (- sum dJ_0 with an initial state).
+//          Every term belongs to the token's own tile: the apply kernel writes dgt and the tile's share of dg,
+//          a last small kernel sums the shares per head.
 #include <type_traits>
 
 #include "chunk_common.h"
@@ -46,11 +48,9 @@ struct BwdArgs {
   void *wDM, *wDJ;        // [total_chunks,H,dv,dk] local carries, then incoming carries, in the dtype of the rows
   float* wFtot;           // [total_chunks,H] log2 of the total decay of a tile
   float* wSig;            // [total_chunks,H] sum over the tile of dJloc
-  float* wBnd;            // [total_chunks,H] F_C <carry, state at the start of the tile>
   float* wE;              // [H, tokens]  local part of d log f
-  float* wBc;             // [H, tokens]  beta_r of the carry terms
   float* wInitPart;       // [n_seqs,H,dv*dk/256] partial sums of dJ_0
-  double *wDgPart, *wDIpPart;  // [n_seqs,H,pieces of the gate pass], [n_seqs,H]
+  float* wDgTile;         // [total_chunks,H] the tiles' shares of dg
   int32_t tokens;
   int32_t apply_alias;     // carry apply: db^carry shares LDS with the bf16 carries (large head dims)
 };
@@ -620,9 +620,21 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   int bos, len, cbase;
   seq_lookup(a, seq, bos, len, cbase);
   const bool last = cis == (len + kC - 1) / kC - 1;
+  // Gate gradient of the tile's tokens, by wave 0 once the carry terms are known:
+  //   d log f_t = (local part, from the tile kernel) + (carry terms of the earlier tokens of the tile) + (boundary term),
+  //   dgt_t = -g d log f_t, and the tile's share of dg = -sum_t gt_t d log f_t.
+  auto gate_grad = [&](float bc, float bnd) {
+    const bool ok = lane < clen;
+    const float pre = wave_inclusive_scan(bc, lane) - bc;
+    const int64_t tok = (int64_t)t0 + lane;
+    const float dlogf = ok ? A.wE[(int64_t)h * A.tokens + tok] + pre + bnd : 0.f;
+    const float gt = ok ? load_gate(a.gt, tok * H + h, a.gate_bf16) : 0.f;
+    if (ok) A.dgt[tok * H + h] = -a.g[h] * dlogf;
+    const float share = wave_sum(-gt * dlogf);
+    if (lane == 0) A.wDgTile[(int64_t)cidx * H + h] = share;
+  };
   if (last) {  // nothing flows in from beyond the end of the sequence (uniform for the block)
-    if (tid == 0) A.wBnd[(int64_t)cidx * H + h] = 0.f;
-    if (tid < clen) A.wBc[(int64_t)h * A.tokens + t0 + tid] = 0.f;
+    if (w == 0) gate_grad(0.f, 0.f);
     return;
   }
   const float gh = a.g[h] * kLog2e;
@@ -667,7 +679,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     if (lane == 0) sW4[w] = acc;
   }
   __syncthreads();
-  if (tid == 0) A.wBnd[(int64_t)cidx * H + h] = sW4[4] * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);
+  const float bnd = sW4[4] * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);   // every thread; the slots are rewritten only after later barriers
 
   const int srow = 16 * w + i;            // operand row (token) of this lane
   const bool row_ok = srow < clen;
@@ -868,74 +880,33 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       }
       __syncthreads();   // SEQ: the result buffer is free for the next pass; last pass: sBt is complete
     }
-    if (tid < clen) {
+    if (w == 0) {
       float bsum = 0.f;
-      for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[tid * groups + c8];   // fixed order
-      A.wBc[(int64_t)h * A.tokens + t0 + tid] = bsum;
+      if (lane < clen)
+        for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[lane * groups + c8];   // fixed order
+      gate_grad(bsum, bnd);
     }
   }
 }
 
-// ----------------------------------------------------------------- gate pass
-// one block per (sequence, head, piece of kGateTokens tokens); a wave per tile: local part + prefix of the carry
-// terms + boundary term.  The pieces only share the sums dg and dIp, which leave as per-block shares.
-constexpr int kGateTokens = 512;
-__host__ __device__ inline int gate_pieces(int max_len) { return (max_len + kGateTokens - 1) / kGateTokens; }
-
-__global__ __launch_bounds__(256) void chunk_bwd_gate_kernel(BwdArgs A) {
-  const ChunkArgs& a = A.c;
-  __shared__ double sG[4];
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int h = blockIdx.x % a.H, n = blockIdx.x / a.H;
-  const int piece = blockIdx.y, n_pieces = gridDim.y;
-  int bos, len, cbase;
-  seq_lookup(a, n, bos, len, cbase);
-  const float gh = a.g[h];
-  double dg_acc = 0.0;
-  const int nchunks = (len + kC - 1) / kC;
-  const int seg0 = piece * (kGateTokens / 256), seg1 = min((len + 255) / 256, seg0 + kGateTokens / 256);
-  for (int seg = seg0; seg < seg1; ++seg) {
-    const int t = seg * 256 + tid;
-    const bool ok = t < len;
-    const float bc = ok ? A.wBc[(int64_t)h * A.tokens + bos + t] : 0.f;
-    const float pre = wave_inclusive_scan(bc, lane) - bc;   // carry terms of the earlier tokens of the tile
-    if (ok) {
-      const int tile = seg * 4 + w;
-      const float dlogf = A.wE[(int64_t)h * A.tokens + bos + t] + pre + A.wBnd[(int64_t)(cbase + tile) * a.H + h];
-      const float gt = load_gate(a.gt, (int64_t)(bos + t) * a.H + h, a.gate_bf16);
-      A.dgt[(int64_t)(bos + t) * a.H + h] = -gh * dlogf;
-      dg_acc -= (double)gt * (double)dlogf;
-    }
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) dg_acc += __shfl_xor(dg_acc, off);
-  if (lane == 0) sG[w] = dg_acc;
-  __syncthreads();
-  if (tid == 0) A.wDgPart[((int64_t)n * a.H + h) * n_pieces + piece] = sG[0] + sG[1] + sG[2] + sG[3];
-  if (piece == 0 && w == 1) {
-    // dIp share of this (sequence, head): the tiles' terms and, with an initial state, -sum dJ_0
-    double s = 0.0;
-    for (int c = lane; c < nchunks; c += 64) s += (double)A.wSig[(int64_t)(cbase + c) * a.H + h];
-    if (a.init_mu) {
-      const int nblk = carry_scan_blocks((int64_t)a.dv * a.dk);
-      for (int b2 = lane; b2 < nblk; b2 += 64) s -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
-    if (lane == 0) A.wDIpPart[(int64_t)n * a.H + h] = s;
-  }
-}
-
-// dg[h], dIp[h]: one wave per head sums the shares (fixed order: lane-strided, then the lanes)
-__global__ __launch_bounds__(64) void chunk_bwd_head_reduce_kernel(BwdArgs A, int n_pieces) {
+// ----------------------------------------------------------------- head sums
+// dg[h] = sum over the tiles of their shares; dIp[h] = sum over the tiles of the local terms and, with an initial
+// state, - sum dJ_0 (J_0 = I_0 - Ip).  One wave per head, lane-strided then over the lanes (fixed order), in double.
+__global__ __launch_bounds__(64) void chunk_bwd_head_reduce_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   const int h = blockIdx.x, lane = threadIdx.x;
   double sg = 0.0, si = 0.0;
-  for (int j = lane; j < a.n_seqs * n_pieces; j += 64) {
-    const int n = j / n_pieces, pc = j - n * n_pieces;
-    sg += A.wDgPart[((int64_t)n * a.H + h) * n_pieces + pc];
+  for (int c = lane; c < a.total_chunks; c += 64) {
+    sg += (double)A.wDgTile[(int64_t)c * a.H + h];
+    si += (double)A.wSig[(int64_t)c * a.H + h];
   }
-  for (int n = lane; n < a.n_seqs; n += 64) si += A.wDIpPart[(int64_t)n * a.H + h];
+  if (a.init_mu) {
+    const int nblk = carry_scan_blocks((int64_t)a.dv * a.dk);
+    for (int j = lane; j < a.n_seqs * nblk; j += 64) {
+      const int n = j / nblk, b2 = j - n * nblk;
+      si -= (double)A.wInitPart[((int64_t)n * a.H + h) * nblk + b2];
+    }
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     sg += __shfl_xor(sg, off);
@@ -948,7 +919,7 @@ __global__ __launch_bounds__(64) void chunk_bwd_head_reduce_kernel(BwdArgs A, in
 }
 
 struct BwdLayout {
-  size_t oDM, oDJ, oFtot, oSig, oBnd, oE, oBc, oInit, oDg, oDIp, total;
+  size_t oDM, oDJ, oFtot, oSig, oE, oInit, oDgTile, total;
 };
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -963,12 +934,9 @@ static BwdLayout bwd_layout(const PalDims* d) {
   L.oDJ = o; o = align256(o + tiles * E * 4);
   L.oFtot = o; o = align256(o + tiles * 4);
   L.oSig = o; o = align256(o + tiles * 4);
-  L.oBnd = o; o = align256(o + tiles * 4);
   L.oE = o; o = align256(o + tokens * d->n_heads * 4);
-  L.oBc = o; o = align256(o + tokens * d->n_heads * 4);
   L.oInit = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * (E / 256) * 4);
-  L.oDg = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * gate_pieces(d->seq_len) * 8);
-  L.oDIp = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * 8);
+  L.oDgTile = o; o = align256(o + tiles * 4);
   L.total = o;
   return L;
 }
@@ -1063,9 +1031,9 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   A.d_init_mu = gr->d_init_mu; A.d_init_I = gr->d_init_I;
   char* ws = (char*)workspace;
   A.wDM = ws + L.oDM; A.wDJ = ws + L.oDJ;
-  A.wFtot = (float*)(ws + L.oFtot); A.wSig = (float*)(ws + L.oSig); A.wBnd = (float*)(ws + L.oBnd);
-  A.wE = (float*)(ws + L.oE); A.wBc = (float*)(ws + L.oBc); A.wInitPart = (float*)(ws + L.oInit);
-  A.wDgPart = (double*)(ws + L.oDg); A.wDIpPart = (double*)(ws + L.oDIp);
+  A.wFtot = (float*)(ws + L.oFtot); A.wSig = (float*)(ws + L.oSig);
+  A.wE = (float*)(ws + L.oE); A.wInitPart = (float*)(ws + L.oInit);
+  A.wDgTile = (float*)(ws + L.oDgTile);
   A.tokens = dd.batch * dd.seq_len;
   hipStream_t s = (hipStream_t)stream;
   const bool bf = dd.dtype == PAL_DTYPE_BF16;
@@ -1099,11 +1067,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
     if (rc) return rc;
     PAL_HIP_LAUNCH_CHECK();
   }
-  const int n_pieces = gate_pieces(dd.seq_len);
-  if (n_pieces > 65535) return PAL_E_DIM;
-  PAL_TIMED_LAUNCH(kKernBwdGate, s, chunk_bwd_gate_kernel, dim3((unsigned)(dd.n_seqs * dd.n_heads), (unsigned)n_pieces), dim3(256), 0, s, A);
-  PAL_HIP_LAUNCH_CHECK();
-  PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((unsigned)dd.n_heads), dim3(64), 0, s, A, n_pieces);
+  PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((unsigned)dd.n_heads), dim3(64), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }

@@ -12,7 +12,7 @@ enum KernelId {
   kKernBwdLocal,
   kKernBwdCarryScan,
   kKernBwdCarryApply,
-  kKernBwdGate,
+  kKernBwdGate,   // unused since the gate gradients moved into the carry apply kernel (kept: ids are positional)
   kKernBwdHeadReduce,
   kKernRecurrentBwdFwdPass,
   kKernRecurrentBwd,
