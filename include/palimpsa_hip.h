@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PAL_ABI_VERSION 1
+#define PAL_ABI_VERSION 2
 
 /* element types of tensors handed over the boundary */
 #define PAL_DTYPE_F32 0
@@ -42,6 +42,13 @@ extern "C" {
 #define PAL_FLAG_HAS_INIT 2u    /* init_mu / init_I given                    */
 #define PAL_FLAG_STORE_FINAL 4u /* final_mu / final_I requested              */
 #define PAL_FLAG_HAS_VAR 8u     /* o_var (fwd) / do_var (bwd) present        */
+/* How the chunked entry points (pal_chunk_fwd, pal_gla_chunk_fwd, pal_gla_chunk_bwd) build the states at the start
+ * of every tile; no counterpart in the reference, results agree to rounding.  Neither bit: chosen by shape.
+ * Meant for tests and measurements. */
+#define PAL_FLAG_STATES_TWO_KERNELS 256u /* per-tile contributions by all tiles in parallel, then a scan over
+                                            the tiles (any shape and dtype)                                  */
+#define PAL_FLAG_STATES_ONE_PASS 512u    /* one pass per (sequence, head) that keeps the running state in
+                                            registers, wherever it applies (bf16 rows)                       */
 
 /* error codes (negative) */
 #define PAL_OK 0
@@ -149,8 +156,12 @@ int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
  * (chunk_palimpsa_forgetting_scalar.py:66-218, :441-517).  Fills chunk_mu /
  * chunk_I (the reference's intermediate_mu_state / intermediate_I_state,
  * :187-188) for the backward.  The prefix products of the output kernel use f16
- * operands with a per-tile block exponent: |k| <= 128 and
- * max(|v|,|b|) * max(1,|k|^2) < 2^28 are required of the rows of a 64-token tile. */
+ * operands normalised per 64-token tile by three block exponents (of k, v and b),
+ * so results do not depend on the magnitude of the rows; within a tile, entries
+ * more than 2^26 below the largest of their tensor lose precision.
+ * cu_seqlens (varlen) must ascend from 0 to the token count; the kernels clamp
+ * every sequence and tile to the token range, so a malformed array cannot make
+ * them address memory beyond the tensors (results are then unspecified). */
 int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
 /* Chunked forward without the precision state (scalar-gated linear attention):
@@ -160,7 +171,8 @@ int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
  * :293-300; flash-linear-attention is a dependency of the reference, not part
  * of its tree).  Reads q, k, v, gt, g, [init_mu], cu_seqlens + chunk tables;
  * writes o, [final_mu] and, on this path, two buffers of total_chunks*H*dv*dk
- * entries: chunk_mu is fp32 scratch (free after the call), chunk_I receives the
+ * entries: chunk_mu is fp32 scratch (free after the call; may be NULL when
+ * pal_state_pass_applies(dims, 0) is 1), chunk_I receives the
  * tile-start states S in bf16 (2 bytes per entry; what the backward needs).
  * b, Ip, o_var, init_I, final_I are ignored; PAL_FLAG_HAS_VAR is rejected with
  * PAL_E_STATE.  init_mu / final_mu hold S as [N,H,dv,dk] fp32. */
@@ -270,25 +282,25 @@ size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims *dims);
 int pal_epilogue_bwd(const PalGlueDims *dims, const PalEpilogueTensors *t, const PalEpilogueGrads *gr,
                      void *workspace, size_t workspace_bytes, void *stream);
 
-/* ------------------------------------------------------------ tuning knob */
+/* ------------------------------------------------------------ shape queries */
 
-/* How the chunked entry points (pal_chunk_fwd, pal_gla_chunk_fwd, pal_gla_chunk_bwd) build the
- * states at the start of every tile; no counterpart in the reference, results agree to rounding.
- *   0 (default): chosen by shape;
- *   1: per-tile contributions by all tiles in parallel, then a scan over the tiles
- *      (any shape and dtype);
- *   2: one pass per (sequence, head) that keeps the running state in registers, wherever it
- *      applies (bf16 rows).
- * Process-global; meant for tests and measurements. */
-void pal_set_state_pass_mode(int mode);
+/* 1 if the chunked entry points would build the tile-start states of this call (dims as handed to them,
+ * including the PAL_FLAG_STATES_* bits) in one pass, 0 if with the two-kernel form.  With the one-pass form
+ * pal_gla_chunk_fwd never touches its fp32 scratch (chunk_mu), which may then be NULL-sized by the caller. */
+int pal_state_pass_applies(const PalDims *dims, int has_precision_state);
+
+/* PAL_OK if pal_chunk_bwd serves this head-dim pair, PAL_E_HEADDIM otherwise (see pal_chunk_bwd); lets a caller
+ * refuse in its forward what its backward could not do. */
+int pal_chunk_bwd_supported(int32_t dk, int32_t dv);
 
 /* ------------------------------------------------------------ measurement */
 
 /* Per-kernel timing aid; no counterpart in the reference.  While enabled, every
  * kernel launch of the library is bracketed by two HIP events on the launch
  * stream; pal_profile_read waits for the outstanding ones and returns the
- * accumulated time and launch count of one kernel.  Process-global, for
- * benchmarks only (not thread-safe while enabled). */
+ * accumulated time and launch count of one kernel.  The switch and the
+ * counters belong to the calling thread (thread-local): launches made by
+ * other threads are neither timed nor counted.  For benchmarks only. */
 int pal_profile_enable(int on);               /* also resets the counters */
 int pal_profile_kernel_count(void);
 const char *pal_profile_kernel_name(int kernel_id);

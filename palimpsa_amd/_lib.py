@@ -12,9 +12,10 @@ from typing import Optional
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libpalimpsa_hip.so")
 
-PAL_ABI_VERSION = 1
+PAL_ABI_VERSION = 2
 PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
+PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS = 256, 512
 PAL_CHUNK = 64
 
 PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5
@@ -121,8 +122,10 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_size_t
         fn.argtypes = [P(PalGlueDims)]
-    lib.pal_set_state_pass_mode.restype = None
-    lib.pal_set_state_pass_mode.argtypes = [C.c_int]
+    lib.pal_state_pass_applies.restype = C.c_int
+    lib.pal_state_pass_applies.argtypes = [P(PalDims), C.c_int]
+    lib.pal_chunk_bwd_supported.restype = C.c_int
+    lib.pal_chunk_bwd_supported.argtypes = [C.c_int32, C.c_int32]
     lib.pal_profile_enable.restype = C.c_int
     lib.pal_profile_enable.argtypes = [C.c_int]
     lib.pal_profile_kernel_count.restype = C.c_int
@@ -133,11 +136,25 @@ def load() -> C.CDLL:
     lib.pal_profile_read.argtypes = [C.c_int, P(C.c_double), P(C.c_int64)]
     if lib.pal_abi_version() != PAL_ABI_VERSION:
         raise ImportError(f"{LIB_PATH}: ABI version {lib.pal_abi_version()} != expected {PAL_ABI_VERSION}; rebuild")
-    mode = os.environ.get("PALIMPSA_STATE_PASS_MODE")
-    if mode is not None:
-        lib.pal_set_state_pass_mode(int(mode))
     _lib = lib
     return lib
+
+
+# How the chunked entry points build the tile-start states (PAL_FLAG_STATES_* of the C ABI): 0 = chosen by shape,
+# 1 = two kernels, 2 = one pass wherever it applies.  A knob of this Python layer for tests and measurements (the
+# library itself keeps no such state); initial value from the environment variable PALIMPSA_STATE_PASS_MODE.
+_state_pass_mode = int(os.environ.get("PALIMPSA_STATE_PASS_MODE", "0"))
+
+
+def set_state_pass_mode(mode: int) -> None:
+    global _state_pass_mode
+    if mode not in (0, 1, 2):
+        raise ValueError(f"state pass mode must be 0, 1 or 2, got {mode!r}")
+    _state_pass_mode = mode
+
+
+def state_pass_flags() -> int:
+    return (0, PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS)[_state_pass_mode]
 
 
 def strerror(code: int) -> str:

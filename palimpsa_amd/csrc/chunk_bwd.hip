@@ -941,6 +941,47 @@ static BwdLayout bwd_layout(const PalDims* d) {
   return L;
 }
 
+// Launch shapes that depend on the head dims only; worked out before the first launch so that a head-dim pair the
+// backward cannot serve is refused while nothing has been enqueued.
+struct BwdPlan {
+  int nb_local;        // column blocks per pass of the tile kernel
+  size_t lds_local;
+  size_t lds_apply;
+  int apply_alias, apply_seq, apply_ksmax;
+};
+
+static size_t local_lds_bytes(int NB, bool var) {
+  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
+         (size_t)NB * 2 * 8 * 64 * 16;
+}
+
+static int bwd_plan(int dk, int dv, bool var, BwdPlan& P) {
+  const int nb_total = dk / 16;
+  if (nb_total < 1 || nb_total > 16) return PAL_E_HEADDIM;
+  // at most 4 column blocks (16 waves) per workgroup; wider heads are split into equal passes
+  const int n_pass = (nb_total + 3) / 4;
+  P.nb_local = (nb_total + n_pass - 1) / n_pass;
+  P.lds_local = local_lds_bytes(P.nb_local, var);
+  if (P.lds_local > kMaxLds) return PAL_E_HEADDIM;
+  const int dmax = dk > dv ? dk : dv;
+  const size_t rt_bytes = 2 * (size_t)2 * dk * (dv + 8), o_bytes = sizeof(float) * kC * (dmax + 4);
+  const size_t lds_fixed = sizeof(float) * (kC + 8 + kC * (dv >> 3)) + o_bytes;
+  size_t lds = lds_fixed + o_bytes + rt_bytes;
+  P.apply_alias = 0;
+  if (lds > kMaxLds) {
+    P.apply_alias = 1;
+    lds = lds_fixed + (rt_bytes > o_bytes ? rt_bytes : o_bytes);
+  }
+  // one result buffer used twice when that lets more workgroups share a compute unit
+  const size_t lds_seq = lds_fixed + rt_bytes;
+  P.apply_seq = lds_seq <= kMaxLds && kMaxLds / lds_seq > (lds > kMaxLds ? 0 : kMaxLds / lds);
+  if (P.apply_seq) { lds = lds_seq; P.apply_alias = 0; }
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  P.lds_apply = lds;
+  P.apply_ksmax = dmax <= 64 ? 2 : dmax <= 128 ? 4 : 8;
+  return PAL_OK;
+}
+
 template <typename TIn, int NB>
 static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   const bool var = A.c.flags & PAL_FLAG_HAS_VAR;
@@ -948,8 +989,7 @@ static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   // four wave roles per block of 16 key columns, NB such blocks at a time (see chunk_bwd_local_roles_kernel)
   const int NT = 4 * NB * 64;
-  const size_t lds = sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
-                     (size_t)NB * 2 * 8 * 64 * 16;
+  const size_t lds = local_lds_bytes(NB, var);
   if (lds > kMaxLds) return PAL_E_HEADDIM;
   const bool multi = A.c.dk != 16 * NB;
   auto go = [&](auto kern) -> int {
@@ -970,12 +1010,8 @@ static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
 }
 
 template <typename TIn>
-static int launch_local(const BwdArgs& A, hipStream_t s) {
-  // at most 4 column blocks (16 waves) per workgroup; wider heads are split into equal passes
-  const int nb_total = A.c.dk / 16;
-  if (nb_total < 1 || nb_total > 16) return PAL_E_HEADDIM;
-  const int n_pass = (nb_total + 3) / 4;
-  switch ((nb_total + n_pass - 1) / n_pass) {
+static int launch_local(const BwdArgs& A, const BwdPlan& P, hipStream_t s) {
+  switch (P.nb_local) {
     case 1: return launch_local_nb<TIn, 1>(A, s);
     case 2: return launch_local_nb<TIn, 2>(A, s);
     case 3: return launch_local_nb<TIn, 3>(A, s);
@@ -1002,7 +1038,15 @@ static int launch_carry_apply(const BwdArgs& A, int ksmax, bool seq, unsigned bl
 
 extern "C" size_t pal_chunk_bwd_workspace_bytes(const PalDims* d) {
   if (pal_validate_dims(d) != PAL_OK || d->total_chunks <= 0) return 0;
+  pal::BwdPlan P;
+  if (pal::bwd_plan(d->dk, d->dv, (d->flags & PAL_FLAG_HAS_VAR) != 0, P) != PAL_OK) return 0;
   return pal::bwd_layout(d).total;
+}
+
+extern "C" int pal_chunk_bwd_supported(int32_t dk, int32_t dv) {
+  if (dk < 16 || dk > 256 || (dk & 15) || dv < 16 || dv > 256 || (dv & 15)) return PAL_E_HEADDIM;
+  pal::BwdPlan P;
+  return pal::bwd_plan(dk, dv, true, P);
 }
 
 extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const PalBwdTensors* gr, void* workspace,
@@ -1020,6 +1064,12 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   if (rc) return rc;
   rc = check_bwd_common(&dd, gr);
   if (rc) return rc;
+  BwdPlan P;
+  rc = bwd_plan(dd.dk, dd.dv, (dd.flags & PAL_FLAG_HAS_VAR) != 0, P);
+  if (rc) return rc;
+  if ((int64_t)dd.total_chunks * dd.n_heads > 0x7fffffff ||
+      (int64_t)dd.n_seqs * dd.n_heads * carry_scan_blocks((int64_t)dd.dv * dd.dk) > 0x7fffffff)
+    return PAL_E_DIM;
   const BwdLayout L = bwd_layout(&dd);
   if (!workspace || workspace_bytes < L.total || !is_aligned16(workspace)) return PAL_E_WORKSPACE;
   BwdArgs A;
@@ -1037,7 +1087,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   A.tokens = dd.batch * dd.seq_len;
   hipStream_t s = (hipStream_t)stream;
   const bool bf = dd.dtype == PAL_DTYPE_BF16;
-  rc = bf ? launch_local<bf16_t>(A, s) : launch_local<float>(A, s);
+  rc = bf ? launch_local<bf16_t>(A, P, s) : launch_local<float>(A, P, s);
   if (rc) return rc;
   {
     const int64_t blocks = (int64_t)dd.n_seqs * dd.n_heads * carry_scan_blocks((int64_t)dd.dv * dd.dk);
@@ -1048,22 +1098,9 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   }
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
-    const int dmax = dd.dk > dd.dv ? dd.dk : dd.dv;
-    const size_t rt_bytes = 2 * (size_t)2 * dd.dk * (dd.dv + 8), o_bytes = sizeof(float) * kC * (dmax + 4);
-    const size_t lds_fixed = sizeof(float) * (kC + 8 + kC * (dd.dv >> 3)) + o_bytes;
-    size_t lds = lds_fixed + o_bytes + rt_bytes;
-    A.apply_alias = 0;
-    if (lds > kMaxLds) {
-      A.apply_alias = 1;
-      lds = lds_fixed + (rt_bytes > o_bytes ? rt_bytes : o_bytes);
-    }
-    // one result buffer used twice when that lets more workgroups share a compute unit
-    const size_t lds_seq = lds_fixed + rt_bytes;
-    const bool seq = lds_seq <= kMaxLds && kMaxLds / lds_seq > (lds > kMaxLds ? 0 : kMaxLds / lds);
-    if (seq) { lds = lds_seq; A.apply_alias = 0; }
-    if (lds > kMaxLds) return PAL_E_HEADDIM;
-    const int ksmax = dmax <= 64 ? 2 : dmax <= 128 ? 4 : 8;
-    rc = bf ? launch_carry_apply<bf16_t>(A, ksmax, seq, blocks, lds, s) : launch_carry_apply<float>(A, ksmax, seq, blocks, lds, s);
+    A.apply_alias = P.apply_alias;
+    rc = bf ? launch_carry_apply<bf16_t>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s)
+            : launch_carry_apply<float>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s);
     if (rc) return rc;
     PAL_HIP_LAUNCH_CHECK();
   }

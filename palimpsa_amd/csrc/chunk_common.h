@@ -38,7 +38,12 @@ struct ChunkArgs {
 __device__ __forceinline__ void chunk_lookup(const ChunkArgs& a, int c, int& seq, int& t0, int& clen, int& cis) {
   if (a.chunk_table) {
     const int32_t* row = a.chunk_table + 4 * (int64_t)c;
-    seq = row[0]; t0 = row[1]; clen = row[2]; cis = row[3];
+    seq = min(max(row[0], 0), a.n_seqs - 1);
+    cis = row[3];
+    // a tile stays inside the packed token axis whatever the table holds (its first token always exists:
+    // masked lanes still address it)
+    t0 = min(max(row[1], 0), a.T - 1);
+    clen = min(max(row[2], 0), min(kC, a.T - t0));
   } else {
     const int per = (a.T + kC - 1) / kC;
     seq = c / per;
@@ -51,9 +56,10 @@ __device__ __forceinline__ void chunk_lookup(const ChunkArgs& a, int c, int& seq
 // sequence n -> (first token, length, index of its first tile)
 __device__ __forceinline__ void seq_lookup(const ChunkArgs& a, int n, int& bos, int& len, int& cbase) {
   if (a.cu_seqlens) {
-    bos = a.cu_seqlens[n];
-    len = a.cu_seqlens[n + 1] - bos;
-    cbase = a.chunk_offsets[n];
+    packed_seq_bounds(a.cu_seqlens, n, a.T, bos, len);
+    // the tiles of a sequence stay inside the per-tile buffers
+    cbase = min(max(a.chunk_offsets[n], 0), a.total_chunks);
+    len = min(len, (a.total_chunks - cbase) * kC);
   } else {
     bos = n * a.T;
     len = a.T;
@@ -61,15 +67,25 @@ __device__ __forceinline__ void seq_lookup(const ChunkArgs& a, int n, int& bos, 
   }
 }
 
-// Block exponent E of a tile for the f16 operands of the prefix products.  The operands
-// X^M = k v 2^-E and X^J = k^2 b 2^-E are built with packed f16 multiplies from k, k^2 (f16) and the
-// staged rows v 2^-E, b 2^-E (f16); the decay operand carries the 2^E back (L 2^E <= 2^15), so the
-// fp32 accumulators hold the unscaled sums.  E = 0 unless max(|v|,|b|) max(1,|k|^2) over the tile
-// exceeds 2^12; supported range: |k| <= 128 and max(|v|,|b|) max(1,|k|^2) < 2^28.
+// Block exponents of a tile for the f16 operands of the prefix products.  The operands
+//   X^M = (k 2^-ek)(v 2^-ev)  and  X^J = (k 2^-ek)^2 (b 2^-eb)
+// are built with packed f16 multiplies from f16 copies of the scaled rows; ek, ev, eb bring the largest |k| of the
+// tile to [1, 2) and the largest |v|, |b| to [2^11, 2^12), so that the operands use the top of the f16 range whatever
+// the magnitude of the rows (entries more than 2^26 below the largest of their tensor in the tile lose bits, which
+// is an absolute error far below that of the bf16 rows).  The sums then hold M 2^-(ek+ev) and J 2^-(2ek+eb); the
+// tile-start state enters with the same factors and mu = M / I is put right once per output by 2^(ev-ek-eb), so the
+// scaling costs nothing per state entry.  A tensor that is all zero (or holds inf/nan) gets exponent 0.
 // Every thread of the workgroup calls this (it synchronises); sMax is LDS scratch of 3 floats per wave.
+struct TileExponents { int ek, ev, eb; };
+
+__device__ __forceinline__ int block_exponent_of(float m, int target) {
+  // m is a maximum of absolute values: zero, inf and nan keep exponent 0 (the arithmetic then yields what fp32 would)
+  return (m > 0.f && m < __builtin_inff()) ? ilogbf(m) - target : 0;
+}
+
 template <typename TIn>
-__device__ __forceinline__ int tile_block_exponent(const TIn* kt, const TIn* vt, const TIn* bt, int H, int dk, int dv,
-                                                   int clen, int tid, int nthreads, float* sMax) {
+__device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, const TIn* vt, const TIn* bt, int H, int dk,
+                                                              int dv, int clen, int tid, int nthreads, float* sMax) {
   float km = 0.f, vm = 0.f, bm = 0.f;
   const int gk = dk >> 3, gv = dv >> 3;
   for (int idx = tid; idx < kC * gk; idx += nthreads) {
@@ -103,8 +119,11 @@ __device__ __forceinline__ int tile_block_exponent(const TIn* kt, const TIn* vt,
   km = 0.f; vm = 0.f; bm = 0.f;
   for (int x = 0; x < nw; ++x) { km = fmaxf(km, sMax[3 * x]); vm = fmaxf(vm, sMax[3 * x + 1]); bm = fmaxf(bm, sMax[3 * x + 2]); }
   __syncthreads();
-  const float m = fmaxf(vm, bm) * fmaxf(1.f, km * km);
-  return (m > 4096.f) ? min(15, ilogbf(m) - 12) : 0;
+  TileExponents e;
+  e.ek = block_exponent_of(km, 0);
+  e.ev = block_exponent_of(vm, 11);
+  e.eb = block_exponent_of(bm, 11);
+  return e;
 }
 
 // inclusive prefix sum over the 64 lanes of a wave: four shifted adds inside each row of 16 lanes (DPP

@@ -379,9 +379,12 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
     }
   }
   stage_load(0);
-  // block exponent of the f16 operands (see tile_block_exponent); sO doubles as its scratch
-  const int bexp = tile_block_exponent((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
-  const float down = __builtin_amdgcn_exp2f(-(float)bexp);
+  // block exponents of the f16 operands (see tile_block_exponents); sO doubles as its scratch
+  const TileExponents bexp =
+      tile_block_exponents((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
+  const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
+  const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
+  const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
   auto stage_store = [&](int buf) {
 #pragma unroll
     for (int it = 0; it < NITEM; ++it) {
@@ -390,8 +393,8 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
       if (idx < kC * kDG / 4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          sV[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(vst[it][e] * down);
-          sB[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(bst[it][e] * down);
+          sV[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(vst[it][e] * down_v);
+          sB[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(bst[it][e] * down_b);
         }
       }
     }
@@ -400,14 +403,18 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   __syncthreads();
 
   // ---- per-wave constants of this tile
-  float F[4], Gi[4], ct[4];
+  // the sums hold M 2^-(ek+ev) and J 2^-(2ek+eb): the tile-start state and the prior enter with the same factors
+  // (two steps each, so that no factor leaves the fp32 range where the rows themselves do not)
+  float Fm[4], Fj[4], Gi[4], ct[4];
 #pragma unroll
   for (int tb = 0; tb < 4; ++tb) {
     ct[tb] = sC[16 * tb + i];
-    F[tb] = fast_exp2(ct[tb]);
-    Gi[tb] = (1.f - F[tb]) * Ip;
+    const float F = fast_exp2(ct[tb]);
+    Fm[tb] = (F * down_k) * down_v;
+    Fj[tb] = ((F * down_k) * down_k) * down_b;
+    Gi[tb] = ((((1.f - F) * Ip) * down_k) * down_k) * down_b;
   }
-  f16x8 Lr[6];            // decay operand times 2^E
+  f16x8 Lr[6];            // decay operand
   f16x8 kA[2], kk[2];     // k and k*k of the wave's key column for the 64 tokens, operand layout
   {
 #pragma unroll
@@ -418,18 +425,21 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int s = 8 * g + j + 32 * ks;
-        kA[ks][j] = (f16_t)kraw[ks][j];
-        kk[ks][j] = (f16_t)(kraw[ks][j] * kraw[ks][j]);
+        const float ksc = kraw[ks][j] * down_k;
+        kA[ks][j] = (f16_t)ksc;
+        kk[ks][j] = (f16_t)(ksc * ksc);
 #pragma unroll
         for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
           const int t = 16 * tb + i;
-          const float lv = (s <= t) ? fast_exp2(ct[tb] - cs[j] + (float)bexp) : 0.f;
+          const float lv = (s <= t) ? fast_exp2(ct[tb] - cs[j]) : 0.f;
           Lr[lidx(tb, ks)][j] = (f16_t)lv;
         }
       }
     }
   }
-  const float scale = a.scale;
+  // mu = M / I comes out times 2^(ek+eb-ev) and 1 / I times 2^(2ek+eb): put right once per output
+  const float scale = ((a.scale * __builtin_amdgcn_exp2f((float)bexp.ev)) * down_k) * down_b;
+  const float scale_var = ((a.scale * down_k) * down_k) * down_b;
   const float* cmu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
   const float* cI = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
 
@@ -475,8 +485,8 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
         float acc = 0.f, accv = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float Mf = fmaf(F[tb], M0[r], accM[r]);
-          const float If = fmaf(F[tb], I0[r], accI[r]);
+          const float Mf = fmaf(Fm[tb], M0[r], accM[r]);
+          const float If = fmaf(Fj[tb], I0[r], accI[r]);
           const float rI = fast_rcp(If);
           acc = fmaf(Mf * rI, qD[tb][r], acc);
           if (HAS_VAR) accv = fmaf(qD[tb][r] * qD[tb][r], rI, accv);
@@ -508,7 +518,7 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
         for (int e = 0; e < 4; ++e) op[e] = from_f32<TIn>(acc[e] * scale);
         if (HAS_VAR) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) store_rt(a.o_var, off + e, accv[e] * scale, a.var_bf16);
+          for (int e = 0; e < 4; ++e) store_rt(a.o_var, off + e, accv[e] * scale_var, a.var_bf16);
         }
       }
     }

@@ -319,8 +319,6 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
   }
 }
 
-static int g_state_pass_mode = 0;   // 0: by shape, 1: always the two-kernel form, 2: the one-pass form where it applies
-
 template <bool HAS_J, int NIK>
 static int launch_state_pass_t(const StatePassArgs& A, int kern_id, unsigned grid, size_t lds, hipStream_t s) {
   if (int rc = allow_lds((const void*)&chunk_states_kernel<HAS_J, NIK>, lds)) return rc;
@@ -343,11 +341,11 @@ static int launch_state_pass_j(const StatePassArgs& A, int kern_id, unsigned gri
 // Whether the one-pass form serves this call: bf16 rows, and enough (sequence, head, slice) workgroups that
 // the serial walk over the tiles does not leave most of the GPU idle.
 bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j) {
-  if (dtype != PAL_DTYPE_BF16 || g_state_pass_mode == 1) return false;
+  if (dtype != PAL_DTYPE_BF16 || (a.flags & PAL_FLAG_STATES_TWO_KERNELS)) return false;
   if (a.dk < 16 || a.dk > 256 || a.dk % 16 || a.dv % 16) return false;
   // rows are addressed with 32-bit byte offsets from the first row of a sequence
   if ((int64_t)a.T * a.H * (a.dk > a.dv ? a.dk : a.dv) * 2 >= 0x7fffffffLL) return false;
-  if (g_state_pass_mode == 2) return true;
+  if (a.flags & PAL_FLAG_STATES_ONE_PASS) return true;
   // The walk over the tiles is serial per workgroup (0.4-0.7 us per tile): with fewer workgroups than this the
   // two-kernel form, which spreads the tiles over the whole GPU, is faster.
   return (int64_t)a.n_seqs * a.H * (a.dv / 16) >= 192;
@@ -389,4 +387,10 @@ int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tile
 
 }  // namespace pal
 
-extern "C" void pal_set_state_pass_mode(int mode) { pal::g_state_pass_mode = (mode >= 0 && mode <= 2) ? mode : 0; }
+extern "C" int pal_state_pass_applies(const PalDims* d, int has_precision_state) {
+  if (pal_validate_dims(d) != PAL_OK) return 0;
+  pal::ChunkArgs a = {};
+  a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv; a.n_seqs = d->n_seqs;
+  a.flags = d->flags;
+  return pal::state_pass_applies(a, d->dtype, has_precision_state != 0) ? 1 : 0;
+}

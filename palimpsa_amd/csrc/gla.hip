@@ -598,9 +598,10 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
 extern "C" int pal_gla_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
   using namespace pal;
   if (int rc = check_gla(d, t)) return rc;
-  if (!t->chunk_mu) return PAL_E_NULL;
   ChunkArgs a;
   fill_gla_args(a, d, t);
+  // the fp32 scratch is only used by the two-kernel form of the tile-start states
+  if (!t->chunk_mu && !state_pass_applies(a, d->dtype, false)) return PAL_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   if (int rc = launch_tile_states(a, d->dtype, false, s)) return rc;
   GlaTileArgs A{};

@@ -47,6 +47,16 @@ __device__ __forceinline__ float load_rt(const void* p, int64_t i, int is_bf16) 
   return is_bf16 ? (float)((const bf16_t*)p)[i] : ((const float*)p)[i];
 }
 
+// First token and length of sequence n of a packed batch of `total` tokens.  Both ends are clamped to the token
+// range (a length below zero becomes zero), so that a cu_seqlens array that is not what the interface asks for
+// (ascending from 0 to the token count) cannot make a kernel address memory beyond the tensors.
+__device__ __forceinline__ void packed_seq_bounds(const int32_t* cu, int n, int total, int& bos, int& len) {
+  const int s = min(max(cu[n], 0), total);
+  const int e = min(max(cu[n + 1], s), total);
+  bos = s;
+  len = e - s;
+}
+
 // ---------------------------------------------------------- vector loads
 // VW consecutive elements starting at p (aligned to VW*sizeof(T)) -> fp32
 template <int VW>

@@ -1,7 +1,6 @@
-// Per-kernel timing aid: when enabled, every kernel launch of the library is
-// bracketed by two HIP events on the launch stream.  Meant for benchmarks; it
-// keeps process-global state and is not thread-safe while enabled.
-#include <mutex>
+// Per-kernel timing aid: when enabled, every kernel launch the calling thread makes through the
+// library is bracketed by two HIP events on the launch stream.  Meant for benchmarks.  All of its
+// state is thread-local, so the library keeps no mutable state that two threads share.
 #include <vector>
 
 #include "pal_common.h"
@@ -9,12 +8,11 @@
 
 namespace pal {
 
-static bool g_on = false;
-static std::mutex g_mu;
 struct Pair { int id; hipEvent_t a, b; };
-static std::vector<Pair> g_pending;
-static double g_ms[kKernCount];
-static long long g_n[kKernCount];
+static thread_local bool g_on = false;
+static thread_local std::vector<Pair> g_pending;
+static thread_local double g_ms[kKernCount];
+static thread_local long long g_n[kKernCount];
 
 ProfScope::ProfScope(int id_, hipStream_t s_) : id(id_), s(s_), e0(nullptr), on(g_on) {
   if (!on) return;
@@ -26,12 +24,10 @@ ProfScope::~ProfScope() {
   hipEvent_t e1;
   if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return; }
   (void)hipEventRecord(e1, s);
-  std::lock_guard<std::mutex> lk(g_mu);
   g_pending.push_back({id, e0, e1});
 }
 
 static void drain() {
-  std::lock_guard<std::mutex> lk(g_mu);
   for (auto& p : g_pending) {
     float ms = 0.f;
     if (hipEventSynchronize(p.b) == hipSuccess && hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {

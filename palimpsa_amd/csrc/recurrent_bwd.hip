@@ -39,6 +39,7 @@ struct RecBwdArgs {
   float *pdIp, *pInit;   // [ND][N, H]
   double *dgPart, *dIpPart;  // [N, H]
   int32_t T, H, dk, dv, n_seqs, S, tokens, ND;
+  int32_t seg_cap;       // segments the checkpoint buffers hold
   int32_t gate_bf16, var_bf16, out_bf16;
   uint32_t flags;
   float scale;
@@ -53,9 +54,12 @@ struct NMapB {
 
 __device__ __forceinline__ void rec_seq(const RecBwdArgs& a, int n, int64_t& bos, int& len, int& segbase) {
   if (a.cu_seqlens) {
-    bos = a.cu_seqlens[n];
-    len = a.cu_seqlens[n + 1] - (int)bos;
-    segbase = a.seg_off[n];
+    int b0;
+    packed_seq_bounds(a.cu_seqlens, n, a.T, b0, len);
+    bos = b0;
+    // the segments of a sequence stay inside the checkpoint buffers
+    segbase = min(a.seg_off[n], a.seg_cap);
+    len = min(len, (a.seg_cap - segbase) * a.S);
   } else {
     bos = (int64_t)n * a.T;
     len = a.T;
@@ -68,7 +72,8 @@ __global__ void recurrent_bwd_segoff_kernel(RecBwdArgs a) {
   int acc = 0;
   a.seg_off[0] = 0;
   for (int n = 0; n < a.n_seqs; ++n) {
-    const int len = a.cu_seqlens[n + 1] - a.cu_seqlens[n];
+    int b0, len;
+    packed_seq_bounds(a.cu_seqlens, n, a.T, b0, len);
     acc += (len + a.S - 1) / a.S;
     a.seg_off[n + 1] = acc;
   }
@@ -442,6 +447,7 @@ extern "C" int pal_recurrent_bwd(const PalDims* d, const PalFwdTensors* t, const
   a.dgPart = (double*)(ws + L.oDg); a.dIpPart = (double*)(ws + L.oDIp);
   a.T = dd.seq_len; a.H = dd.n_heads; a.dk = dd.dk; a.dv = dd.dv; a.n_seqs = dd.n_seqs;
   a.S = L.S; a.tokens = dd.batch * dd.seq_len; a.ND = L.ND;
+  a.seg_cap = (int32_t)(L.segments > 0x7fffffff ? 0x7fffffff : L.segments);
   a.gate_bf16 = dd.gate_dtype == PAL_DTYPE_BF16;
   a.var_bf16 = dd.var_dtype == PAL_DTYPE_BF16;
   a.out_bf16 = dd.dtype == PAL_DTYPE_BF16;

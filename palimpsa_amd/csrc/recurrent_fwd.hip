@@ -58,8 +58,9 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
   int64_t bos;
   int T;
   if (a.cu_seqlens) {
-    bos = a.cu_seqlens[n];
-    T = a.cu_seqlens[n + 1] - (int)bos;
+    int b0;
+    packed_seq_bounds(a.cu_seqlens, n, a.T, b0, T);
+    bos = b0;
   } else {
     bos = (int64_t)n * a.T;
     T = a.T;

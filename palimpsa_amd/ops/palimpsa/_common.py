@@ -4,6 +4,7 @@ filling the C structs.  PyTorch is used for device memory and streams only."""
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from dataclasses import dataclass
 from typing import Optional
 
@@ -125,6 +126,48 @@ def prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_
                     dk, dv, dk_p, dv_p, n_seqs, cd)
 
 
+# chunk bookkeeping of the packed batches seen last, per cu_seqlens tensor object: the layers of a model hand the
+# same tensor to every operator call of a step, so the device-to-host copy (a stream synchronisation) and the
+# table happen once per step instead of once per layer
+_chunk_meta_cache: dict = {}
+_CHUNK_META_CACHE_MAX = 8
+
+
+def chunk_meta(cu_seqlens: torch.Tensor, total_tokens: int, device: torch.device):
+    """cu_seqlens (any int dtype/device) -> (packed int32 metadata on ``device``, total_chunks).
+
+    The metadata is ``[N+1]`` cumulative chunk counts followed by ``[total_chunks,4]`` rows (sequence, first
+    token, length, index in sequence).  Raises ValueError unless cu_seqlens starts at 0, never decreases and
+    ends at ``total_tokens`` (the kernels take sequence bounds from it).  Results are kept per tensor object
+    (weakly referenced, invalidated by in-place writes through torch), not per address: a new tensor that
+    reuses the memory of a dead one is looked at again."""
+    key = id(cu_seqlens)
+    hit = _chunk_meta_cache.get(key)
+    if hit is not None:
+        ref, version, tokens, dev, packed, total = hit
+        if ref() is cu_seqlens and version == cu_seqlens._version and tokens == total_tokens and dev == device:
+            return packed, total
+    if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
+        raise ValueError(f"cu_seqlens must be a 1-D tensor of at least two entries, got shape {tuple(cu_seqlens.shape)}")
+    cu_host = cu_seqlens.detach().to("cpu", torch.int64).numpy()
+    if int(cu_host[0]) != 0 or bool((cu_host[1:] < cu_host[:-1]).any()) or int(cu_host[-1]) != int(total_tokens):
+        raise ValueError(
+            "cu_seqlens must start at 0, be non-decreasing and end at the token count "
+            f"({total_tokens}); got first={int(cu_host[0])}, last={int(cu_host[-1])}, "
+            f"decreasing={bool((cu_host[1:] < cu_host[:-1]).any())}")
+    table, offsets = L.build_chunk_table(cu_host)
+    packed = torch.cat([torch.from_numpy(offsets), torch.from_numpy(table.reshape(-1))]).to(torch.int32).to(device)
+    total = int(table.shape[0])
+    if len(_chunk_meta_cache) >= _CHUNK_META_CACHE_MAX:
+        _chunk_meta_cache.pop(next(iter(_chunk_meta_cache)))
+    try:
+        ref = weakref.ref(cu_seqlens, lambda _r, k=key: _chunk_meta_cache.pop(k, None))
+    except TypeError:
+        return packed, total
+    _chunk_meta_cache[key] = (ref, cu_seqlens._version, int(total_tokens), device, packed, total)
+    return packed, total
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
@@ -134,7 +177,7 @@ def make_dims(p: Prepared, scale: float, flags: int, total_chunks: int = 0, var_
     return L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=p.dk_p, dv=p.dv_p,
                      total_chunks=total_chunks, dtype=_pal_dtype(p.compute_dtype),
                      gate_dtype=_pal_dtype(p.gt.dtype), var_dtype=_pal_dtype(var_dtype),
-                     flags=flags, scale=float(scale))
+                     flags=flags | L.state_pass_flags(), scale=float(scale))
 
 
 def make_fwd_tensors(p: Prepared, o, o_var, final_mu, final_I, chunk_table=None, chunk_offsets=None,

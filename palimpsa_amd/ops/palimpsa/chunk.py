@@ -29,14 +29,6 @@ from ... import _lib as L
 from . import _common as cm
 
 
-def _chunk_meta(cu_seqlens: torch.Tensor):
-    """cu_seqlens (any int dtype/device) -> (packed int32 metadata tensor on CPU, total_chunks)."""
-    cu_host = cu_seqlens.detach().to("cpu", torch.int64).numpy()
-    table, offsets = L.build_chunk_table(cu_host)
-    packed = torch.cat([torch.from_numpy(offsets), torch.from_numpy(table.reshape(-1))]).to(torch.int32)
-    return packed, int(table.shape[0])
-
-
 def _count_chunks(T: int, B: int) -> int:
     return (T + L.PAL_CHUNK - 1) // L.PAL_CHUNK * B
 
@@ -71,7 +63,7 @@ def _windowed_forward(p, scale, output_uncertainty, o, o_var, final_mu, final_I,
         for j in range(n_seg):
             s, e = j * seg, min(T, (j + 1) * seg)
             out_mu, out_I = (final_mu, final_I) if (n_seg - 1 - j) % 2 == 0 else scratch
-            flags = L.PAL_FLAG_STORE_FINAL
+            flags = L.PAL_FLAG_STORE_FINAL | L.state_pass_flags()
             if cur_mu is not None:
                 flags |= L.PAL_FLAG_HAS_INIT
             if output_uncertainty:
@@ -104,7 +96,7 @@ class ChunkPalimpsa(torch.autograd.Function):
         table = offsets = None
         if p.cu_seqlens is not None:
             if chunk_offsets is None:
-                chunk_offsets, _ = _chunk_meta(cu_seqlens)
+                chunk_offsets, _ = cm.chunk_meta(cu_seqlens, T, dev)
             meta = chunk_offsets.to(device=dev, dtype=torch.int32).contiguous()
             offsets = meta[: p.n_seqs + 1]
             table = meta[p.n_seqs + 1:]
@@ -243,8 +235,7 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
     if cu_seqlens is not None:
         if q.shape[0] != 1:
             raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
-        chunk_offsets, total_chunks = _chunk_meta(cu_seqlens)
-        chunk_offsets = chunk_offsets.to(q.device)
+        chunk_offsets, total_chunks = cm.chunk_meta(cu_seqlens, q.shape[1], q.device)
     else:
         total_chunks = _count_chunks(q.shape[1], q.shape[0])
     H = q.shape[-2]
@@ -253,6 +244,9 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
     # a long single sequence that no backward will follow is run in windows instead (see _windowed_forward)
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state))
+    if needs_grad:
+        # refuse here what the backward could not serve, instead of at .backward() time
+        L.check(L.load().pal_chunk_bwd_supported(dk_p, dv_p), "chunk_palimpsa (backward head dims)")
     if not needs_grad and cu_seqlens is None and q.shape[0] == 1 and total_chunks > _window_tiles(H, dv_p, dk_p):
         int_mu = int_I = None
     else:

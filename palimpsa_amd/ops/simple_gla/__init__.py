@@ -29,7 +29,7 @@ import torch
 from ... import _lib as L
 from ..palimpsa import _common as cm
 from ..palimpsa import chunk_palimpsa, fused_recurrent_palimpsa
-from ..palimpsa.chunk import _chunk_meta, _count_chunks
+from ..palimpsa.chunk import _count_chunks
 
 __all__ = ["chunk_simple_gla", "fused_recurrent_simple_gla", "ChunkSimpleGLA", "SimpleGlaDecodeStep"]
 
@@ -87,8 +87,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
         table = offsets = None
         flags = 0
         if p.cu_seqlens is not None:
-            meta, total_chunks = _chunk_meta(cu_seqlens)
-            meta = meta.to(dev)
+            meta, total_chunks = cm.chunk_meta(cu_seqlens, T, dev)
             offsets, table = meta[: p.n_seqs + 1], meta[p.n_seqs + 1:]
             flags |= L.PAL_FLAG_VARLEN
         else:
@@ -97,12 +96,15 @@ class ChunkSimpleGLA(torch.autograd.Function):
             flags |= L.PAL_FLAG_HAS_INIT
         o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
         # per-tile contributions (fp32, only needed inside the call) and tile-start states (bf16, kept for the backward)
-        scratch = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
         tile_S = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.bfloat16, device=dev)
         final = None
         if output_final_state:
             final = torch.empty(p.n_seqs, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
         dims = cm.make_dims(p, scale, flags | (L.PAL_FLAG_STORE_FINAL if output_final_state else 0), total_chunks)
+        # the fp32 scratch (4 bytes per state entry and tile) only exists for the two-kernel form of the tile states
+        scratch = None
+        if not L.load().pal_state_pass_applies(dims, 0):
+            scratch = torch.empty(total_chunks, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(p.q), k=pt(p.k), v=pt(p.v), gt=pt(p.gt), g=pt(p.g), o=pt(o), init_mu=pt(p.init_mu),
                                final_mu=pt(final), cu_seqlens=pt(p.cu_seqlens), chunk_table=pt(table),
@@ -114,7 +116,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
             ctx.set_materialize_grads(False)
             ctx.save_for_backward(p.q, p.k, p.v, p.gt, p.g, p.init_mu, p.cu_seqlens, table, offsets, tile_S)
             ctx.meta = dict(dk=p.dk, dv=p.dv, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype, scale=float(scale),
-                            flags=flags, total_chunks=total_chunks, in_dtypes=(q.dtype, k.dtype, v.dtype, g.dtype),
+                            flags=flags | L.state_pass_flags(), total_chunks=total_chunks, in_dtypes=(q.dtype, k.dtype, v.dtype, g.dtype),
                             init_dtype=None if initial_state is None else initial_state.dtype)
         o = cm.unpad_last(o, p.dv).to(q.dtype)
         if final is not None:
@@ -167,9 +169,11 @@ def _check_chunk_args(q, g, cu_seqlens):
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
     if g.shape != q.shape[:3]:
         raise ValueError(f"g must have shape {tuple(q.shape[:3])}, got {tuple(g.shape)}")
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
+        cm.chunk_meta(cu_seqlens, q.shape[1], q.device)   # validates; the table is kept for the call below
     cm._require_gpu(q, g)
-    if cu_seqlens is not None and q.shape[0] != 1:
-        raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
 
 
 @cm.no_compile

@@ -146,3 +146,36 @@ def test_no_cpu_fallback_anywhere():
     for cls in (DecodeStep, SimpleGlaDecodeStep):
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             cls(1, 2, 16, 16, "cpu")
+
+
+@pytest.mark.parametrize("cu", [[1, 8], [0, 5, 3, 8], [0, 4, 9], [0, 4, 7], [0]])
+def test_cu_seqlens_is_validated_before_anything_runs(cu):
+    """cu_seqlens must start at 0, never decrease and end at the token count: the kernels take sequence bounds
+    from it, so a malformed array is refused on the host (ValueError) whatever device the tensors are on."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    H, d, T = 2, 16, 8
+    q = torch.zeros(1, T, H, d)
+    gt = torch.zeros(1, T, H)
+    with pytest.raises(ValueError, match="cu_seqlens"):
+        chunk_palimpsa(q, q, q, q, gt, torch.ones(H), torch.ones(H), cu_seqlens=torch.tensor(cu))
+    with pytest.raises(ValueError, match="cu_seqlens"):
+        chunk_simple_gla(q, q, q, gt, cu_seqlens=torch.tensor(cu))
+
+
+def test_chunk_table_is_kept_per_cu_seqlens_tensor():
+    """The chunk bookkeeping of a packed batch is computed once per cu_seqlens tensor object (every layer of a step
+    passes the same one) and recomputed after an in-place change or for another tensor with the same contents."""
+    from palimpsa_amd.ops.palimpsa import _common as cm
+    cu = torch.tensor([0, 70, 130])
+    m1, n1 = cm.chunk_meta(cu, 130, torch.device("cpu"))
+    m2, n2 = cm.chunk_meta(cu, 130, torch.device("cpu"))
+    assert m1 is m2 and n1 == n2 == 3
+    cu[1] = 64                                  # in-place write: the version counter moves
+    m3, n3 = cm.chunk_meta(cu, 130, torch.device("cpu"))
+    assert m3 is not m1 and n3 == 3 and m3[: 3].tolist() == [0, 1, 3]
+    other = torch.tensor([0, 64, 130])
+    m4, _ = cm.chunk_meta(other, 130, torch.device("cpu"))
+    assert m4 is not m3 and torch.equal(m4, m3)
+    with pytest.raises(ValueError):
+        cm.chunk_meta(cu, 131, torch.device("cpu"))

@@ -172,6 +172,35 @@ def test_squared_error_loss_all_gradients_max_norm(gpu_device):
     _compare(grads, ref, NAMES)
 
 
+def _squared_error_case(inp, dev, cu=None, seed=50):
+    """Gradients of 0.5*sum((o - target)^2) through the kernel and through the float64 oracle (same dO for both)."""
+    gen = torch.Generator().manual_seed(seed)
+    target = 0.3 * torch.randn(inp["v"].shape, generator=gen)
+    o_ref, _, _, _ = hp.oracle_forward(inp, cu=cu, dtype=torch.float64)
+    do = (o_ref - target).float()
+    return _run_bwd(inp, dev, do, cu=cu), hp.oracle_grads(inp, do, cu=cu)
+
+
+def test_c1_shape_sub_batch_dg_dIp_max_norm(gpu_device):
+    """Sequence length, head dims and dtype of configuration 1 on a sub-batch that the float64 oracle can differentiate
+    as a whole (2 rows x 2 heads x 2048 tokens): dg and dIp are sums over every token of a head, so they need the
+    oracle on everything the kernel summed.  Plain max-norm bar for every gradient."""
+    inp = hp.rounded(po.make_inputs(2, 2048, 2, 64, 64, seed=0), torch.bfloat16)
+    inp["g"] = torch.tensor([1.0, 4.0])
+    grads, ref = _squared_error_case(inp, gpu_device)
+    _compare(grads, ref, NAMES)
+
+
+def test_c2_shape_sub_batch_dg_dIp_max_norm(gpu_device):
+    """Head dims and document-length law of configuration 2 (H heads of 96x96, lognormal documents, packed) on 3072
+    tokens x 2 heads; dg and dIp summed over the documents, plain max-norm bar for every gradient."""
+    cu = po.make_varlen_lengths(total_tokens=3072, seed=0)
+    inp = hp.rounded(po.make_inputs(1, cu[-1], 2, 96, 96, seed=2), torch.bfloat16)
+    inp["g"] = torch.tensor([1.0, 8.0])
+    grads, ref = _squared_error_case(inp, gpu_device, cu=cu)
+    _compare(grads, ref, NAMES)
+
+
 @pytest.mark.parametrize("cu", [[0, 0, 5, 5, 70], [0, 64, 64, 128], [0, 130, 130]])
 def test_bf16_backward_varlen_with_empty_documents(gpu_device, cu):
     """Packed batches may hold documents of length zero (they own no tile); their final state is the
@@ -212,7 +241,8 @@ def test_forward_and_backward_are_bitwise_reproducible(gpu_device):
 @pytest.mark.parametrize("dk,dv,ok", [(128, 192, True), (192, 128, True), (256, 64, True), (192, 192, False), (256, 256, False)])
 def test_head_dim_envelope_of_the_backward(gpu_device, dk, dv, ok):
     """The carry tile of the backward has to fit in LDS: the largest supported pairs work end to end, larger ones
-    are refused with a ValueError before any kernel runs (the forward has already succeeded)."""
+    are refused with a ValueError by the forward call when a gradient will be asked for (nothing is enqueued), while
+    a forward without gradients still runs."""
     from palimpsa_amd.ops.palimpsa import chunk_palimpsa
     B, T, H = 1, 100, 1
     inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=6), torch.bfloat16)
@@ -220,12 +250,16 @@ def test_head_dim_envelope_of_the_backward(gpu_device, dk, dv, ok):
     do = torch.randn(B, T, H, dv, generator=gen)
     dev = gpu_device
     leaves = {n: inp[n].to(dev).clone().requires_grad_(True) for n in ("q", "k", "v", "b", "gt", "g", "Ip")}
-    o = chunk_palimpsa(*[leaves[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")], chunk_size=64)
-    loss = (o.float() * do.to(dev)).sum()
     if not ok:
         with pytest.raises(ValueError, match="carry tile"):
-            loss.backward()
+            chunk_palimpsa(*[leaves[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")], chunk_size=64)
+        with torch.no_grad():
+            o = chunk_palimpsa(*[leaves[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")], chunk_size=64)
+        ref_o, _, _, _ = hp.oracle_forward(inp, dtype=torch.float64)
+        assert hp.max_abs(o.float(), ref_o) <= hp.BF16_OUT_ABS_TOL
         return
+    o = chunk_palimpsa(*[leaves[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")], chunk_size=64)
+    loss = (o.float() * do.to(dev)).sum()
     loss.backward()
     ref = hp.oracle_grads(inp, do)
     assert hp.max_abs(o.float(), ref["o"]) <= hp.BF16_OUT_ABS_TOL

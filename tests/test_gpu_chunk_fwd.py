@@ -116,10 +116,12 @@ def test_error_paths_match_reference(gpu_device):
         _call(ck, inp, cu_seqlens=torch.tensor([0, 8], device=gpu_device))
 
 
-@pytest.mark.parametrize("v_scale,k_scale", [(3.0e5, 1.0), (40.0, 30.0), (1.0e-4, 1.0)])
+@pytest.mark.parametrize("v_scale,k_scale", [(3.0e5, 1.0), (40.0, 30.0), (1.0e-4, 1.0), (1.0e-6, 1.0), (1.0e-8, 1.0),
+                                             (1.0, 300.0), (1.0e20, 1.0e-3), (1.0e-20, 1.0e3)])
 def test_block_exponent_of_the_f16_operands(gpu_device, v_scale, k_scale):
-    """Rows far from O(1): the output kernel's f16 operands carry a per-tile block exponent
-    (E > 0 for the first two cases, tiny values for the third); relative error as for O(1) rows."""
+    """Rows far from O(1), in both directions: the output kernel's f16 operands are normalised per tile by block
+    exponents of k, v and b, so the relative error is that of O(1) rows and nothing overflows or flushes
+    (|k| = 300 squares to 9e4, beyond the f16 range without the exponent of k)."""
     ck, _ = _ops()
     B, T, H, d = 1, 200, 2, 64
     inp = po.make_inputs(B, T, H, d, d, seed=77)

@@ -15,9 +15,8 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture
 def state_pass_mode():
     from palimpsa_amd import _lib
-    lib = _lib.load()
-    yield lib.pal_set_state_pass_mode
-    lib.pal_set_state_pass_mode(0)
+    yield _lib.set_state_pass_mode
+    _lib.set_state_pass_mode(0)
 
 
 def _pal_inputs(B, T, H, dk, dv, seed, dev):
