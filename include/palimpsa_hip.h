@@ -63,6 +63,10 @@ extern "C" {
 #define PAL_E_STATE -9       /* init/final state flags and pointers disagree  */
 #define PAL_E_CAPACITY -10   /* output table too small                        */
 #define PAL_E_ALIGN -11      /* pointer not aligned to 16 bytes               */
+#define PAL_E_SCRATCH -12    /* the call needs more than the library's static scratch */
+
+/* Bytes of device memory the library itself holds per GPU for pal_chunk_fwd_static. */
+#define PAL_STATIC_SCRATCH_BYTES (64u << 20)
 
 /* Tokens per chunk tile of the chunked kernels (the chunk size of the benchmark configurations). */
 #define PAL_CHUNK 64
@@ -163,6 +167,22 @@ int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
  * every sequence and tile to the token range, so a malformed array cannot make
  * them address memory beyond the tensors (results are then unspecified). */
 int pal_chunk_fwd(const PalDims *dims, const PalFwdTensors *t, void *stream);
+
+/* pal_chunk_fwd for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose wrapper allocates the
+ * intermediate states with torch, chunk_palimpsa_forgetting_scalar.py:652-653).  Same tensors and results as
+ * pal_chunk_fwd, except that the tile-start states are kept in a buffer of PAL_STATIC_SCRATCH_BYTES that the
+ * library holds on every GPU it runs on (a static device array; nothing is allocated or freed by the call):
+ *   - t->chunk_mu and t->chunk_I must be NULL (PAL_E_STATE otherwise); the states are not handed back, so no
+ *     backward can follow this call;
+ *   - total_chunks * n_heads * dv * dk * 8 bytes must fit: at most PAL_STATIC_SCRATCH_BYTES / 8 = 8 Mi state
+ *     entries per call (e.g. H = 16, 64x64: 128 tiles = 8192 tokens; H = 16, 128x128: 32 tiles = 2048 tokens);
+ *     PAL_E_SCRATCH otherwise.  Longer sequences are run in pieces through init_* / final_*;
+ *   - all calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different streams or
+ *     threads) race on it.  Calls on one stream, or otherwise ordered, are fine; nothing has to be cleared between
+ *     calls (every slot read by a call is written by that call first);
+ *   - the first call on each GPU looks the buffer's address up (hipGetSymbolAddress); make it outside graph capture. */
+int pal_chunk_fwd_static(const PalDims *dims, const PalFwdTensors *t, void *stream);
 
 /* Chunked forward without the precision state (scalar-gated linear attention):
  *   S_t = exp(-gt_t g) S_{t-1} + v_t k_t^T,  o_t = scale S_t q_t.

@@ -20,6 +20,8 @@ PAL_CHUNK = 64
 
 PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5
 PAL_E_CU_SEQLENS, PAL_E_WORKSPACE, PAL_E_CHUNK, PAL_E_STATE, PAL_E_CAPACITY, PAL_E_ALIGN = -6, -7, -8, -9, -10, -11
+PAL_E_SCRATCH = -12
+PAL_STATIC_SCRATCH_BYTES = 64 << 20
 
 # dk values the token-serial kernels are compiled for
 RECURRENT_DK = (16, 32, 48, 64, 96, 128, 192, 256)
@@ -95,7 +97,8 @@ def load() -> C.CDLL:
     lib.pal_validate_dims.argtypes = [P(PalDims)]
     lib.pal_build_chunk_table.restype = C.c_int
     lib.pal_build_chunk_table.argtypes = [P(C.c_int64), C.c_int32, P(C.c_int32), C.c_int32, P(C.c_int32)]
-    for name in ("pal_recurrent_fwd", "pal_chunk_fwd", "pal_gla_chunk_fwd", "pal_gla_recurrent_fwd"):
+    for name in ("pal_recurrent_fwd", "pal_chunk_fwd", "pal_chunk_fwd_static", "pal_gla_chunk_fwd",
+                 "pal_gla_recurrent_fwd"):
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [P(PalDims), P(PalFwdTensors), C.c_void_p]
@@ -166,7 +169,7 @@ def check(code: int, where: str) -> None:
     if code == 0:
         return
     text = strerror(code)
-    if code in (PAL_E_VARLEN_BATCH, PAL_E_CU_SEQLENS, PAL_E_HEADDIM, PAL_E_DIM, PAL_E_DTYPE, PAL_E_STATE):
+    if code in (PAL_E_VARLEN_BATCH, PAL_E_CU_SEQLENS, PAL_E_HEADDIM, PAL_E_DIM, PAL_E_DTYPE, PAL_E_STATE, PAL_E_SCRATCH):
         raise ValueError(f"{where}: {text} (code {code})")
     raise PalimpsaHipError(code, where, text)
 

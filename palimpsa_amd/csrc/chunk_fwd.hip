@@ -14,6 +14,8 @@
 //      M_t, I_t, 1/I_t, mu_t q_t in registers (the scan + division + output of
 //      the reference kernel, :190-207).  Output orientation is [n, t] so the
 //      sum over n stays inside a lane.
+#include <atomic>
+
 #include "chunk_common.h"
 #include "pal_host.h"
 #include "pal_profile.h"
@@ -649,6 +651,63 @@ int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s)
 }
 
 }  // namespace pal
+
+// ------------------------------------------------------------ forward on the library's own scratch
+// The tile-start states of pal_chunk_fwd_static live here instead of in caller memory.  Every GPU the library runs on
+// holds its own copy of this array (at its own address) until the process ends.
+static __device__ __align__(256) float scratch[PAL_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+namespace pal {
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle of the symbol,
+// not memory a kernel can touch: the address is asked for once per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+static std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return PAL_E_DIM;
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!addr) return (int)hipErrorInvalidSymbol;
+    p = (float*)addr;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
+  }
+  *out = p;
+  return PAL_OK;
+}
+
+}  // namespace pal
+
+extern "C" int pal_chunk_fwd_static(const PalDims* d, const PalFwdTensors* t, void* stream) {
+  using namespace pal;
+  if (!d || !t) return PAL_E_NULL;
+  if (t->chunk_mu || t->chunk_I) return PAL_E_STATE;   // the states live in the library's scratch on this path
+  PalFwdTensors tt = *t;
+  // any aligned non-null value passes the pointer checks; the real addresses follow once the size is known to fit
+  tt.chunk_mu = tt.chunk_I = (float*)(uintptr_t)256;
+  int rc = check_chunk_common(d, &tt);
+  if (rc) return rc;
+  const uint64_t entries = (uint64_t)d->total_chunks * (uint64_t)d->n_heads * (uint64_t)d->dv * (uint64_t)d->dk;
+  if (entries > PAL_STATIC_SCRATCH_BYTES / (2 * sizeof(float))) return PAL_E_SCRATCH;
+  float* base = nullptr;
+  rc = static_scratch(&base);
+  if (rc) return rc;
+  tt.chunk_mu = base;
+  tt.chunk_I = base + PAL_STATIC_SCRATCH_BYTES / (2 * sizeof(float));
+  ChunkArgs a;
+  fill_chunk_args(a, d, &tt);
+  hipStream_t s = (hipStream_t)stream;
+  // every slot the output kernel reads is written by the state kernels of this call first: nothing has to start at zero
+  if (int rc2 = launch_tile_states(a, d->dtype, true, s)) return rc2;
+  if (d->dtype == PAL_DTYPE_BF16) return launch_out<bf16_t>(a, s);
+  return launch_out<float>(a, s);
+}
 
 extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
   using namespace pal;

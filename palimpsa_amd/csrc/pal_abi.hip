@@ -24,6 +24,9 @@ const char* pal_strerror(int code) {
     case PAL_E_STATE: return "state flags and state pointers disagree";
     case PAL_E_CAPACITY: return "output table too small";
     case PAL_E_ALIGN: return "pointer not aligned to 16 bytes";
+    case PAL_E_SCRATCH:
+      return "the call needs more tile-start states than the library's static scratch holds "
+             "(total_chunks * n_heads * dv * dk * 8 bytes > PAL_STATIC_SCRATCH_BYTES); split the sequence";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
