@@ -1,7 +1,8 @@
 #!/usr/bin/env python
 """Benchmark of the Palimpsa attention operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla] [--no-layer-slice]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-decode] [--no-simple-gla]
+                    [--no-layer-slice] [--no-configs] [--no-recurrent]
 
 Headline workload (the metric's own configuration): chunked forward+backward at
 B=8, T=2048, H=12, dk=dv=64, bf16 rows and gates (--gates fp32: fp32 gates), fp32 states, 64-token tiles,
@@ -16,6 +17,13 @@ One JSON line is printed; it also carries
                 headline shape, its tile kernel against the HBM peak
   extra.layer_slice  fused prologue -> chunk_palimpsa -> fused epilogue, forward+backward, on the headline shape
                 (the layer between its projections and o_proj), the prologue backward against the HBM peak
+  extra.c0      config 0 (fp32 recurrent forward, B=2 T=256 H=4 d=32), with the CPU port beside it
+  extra.c2      config 2 (packed 32768 tokens, lognormal documents, H=16 d=96, chunked forward+backward)
+  extra.c4      config 4 (one sequence of 65536 tokens, H=16 d=128, chunked forward with initial and final state)
+  extra.recurrent  token-serial forward and backward (pal_recurrent_fwd / pal_recurrent_bwd) at B=8 T=2048 H=12
+                d=64 fp32, against the HBM peak as the metric asks (the kernels are bound by serial latency)
+Every chunked leg carries two bounds: the bf16 matrix peak priced with the fixed formula of the metric and the
+fp32 vector peak priced with the vector instructions the kernel issues (counter figures, see VALU_LANE_OPS).
 """
 from __future__ import annotations
 
@@ -31,7 +39,14 @@ if ROOT not in sys.path:
 
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E peak
+PEAK_FP32_VALU_TFLOPS = 157.3    # MI355X fp32 vector peak (an FMA counted as 2 flops on every lane)
 CHUNK = 64
+# Vector-ALU instructions (matrix instructions excluded) that the two dominant chunked kernels issue per state
+# entry (token x value row x key column), as lane operations: rocprofv3 SQ_INSTS_VALU minus SQ_INSTS_VALU_MFMA_*
+# per launch at the headline shape, times 64 lanes, divided by tokens*H*dk*dv
+# (profiles/bench_c1.sq_counters_pmc.txt).  Like the traffic figures below they cannot be read from inside this
+# process and are stale once those kernels change.
+VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 31.5, "chunk_out_kernel": 8.1}
 # HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
 # from inside this process, so the figures are carried here and are stale once those kernels change.
@@ -52,6 +67,80 @@ def make_inputs(torch, B, T, H, dk, dv, seed, dtype):
                 g=torch.ones(H), Ip=torch.ones(H))
 
 
+def make_varlen_lengths(total_tokens=32768, mu=6.5, sigma=1.0, lo=16, hi=4096, seed=0):
+    """cu_seqlens of config 2: document lengths round(exp(N(mu, sigma))) clipped to [lo, hi], drawn until the sum
+    reaches total_tokens; the last one is cut to fit (merged into the one before when shorter than lo)."""
+    import math
+
+    import numpy as np
+    rng = np.random.RandomState(seed)
+    lens, tot = [], 0
+    while tot < total_tokens:
+        ln = int(np.clip(round(math.exp(rng.normal(mu, sigma))), lo, hi))
+        ln = min(ln, total_tokens - tot)
+        if ln < lo and lens:
+            lens[-1] += ln
+        else:
+            lens.append(ln)
+        tot += ln
+    cu = [0]
+    for ln in lens:
+        cu.append(cu[-1] + ln)
+    return cu
+
+
+def timed_loop(torch, step, steps, warmup):
+    """warmup untimed steps, then exactly `steps` steps between two synchronisations (mean, the contract's figure);
+    then the same number again with an event pair around every step (median of the per-step device times: what
+    A/B comparisons should read) and with the library's per-kernel events on."""
+    from palimpsa_amd import _lib as L
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_mean = (time.perf_counter() - t0) * 1e3 / steps
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    per = sorted(a.elapsed_time(b) for a, b in ev)
+    ms_median = per[len(per) // 2]
+    L.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    kern = L.profile_read()
+    L.profile_enable(False)
+    kernels = {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()}
+    return ms_mean, ms_median, kernels
+
+
+def mfma_roofline(kernel, kernels, flops_per_launch, entries, note):
+    """Roofline entry of a chunked kernel: the bf16 matrix peak priced with the metric's fixed flop formula, and the
+    fp32 vector peak priced with the vector instructions the kernel issues per state entry."""
+    avg_ms = kernels.get(kernel, {"avg_ms": float("nan")})["avg_ms"]
+    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
+    out = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
+           "frac": achieved / PEAK_BF16_MFMA_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": flops_per_launch,
+           "avg_launch_ms": avg_ms, "note": note}
+    ops = VALU_LANE_OPS_PER_ENTRY.get(kernel)
+    if ops is not None:
+        valu = ops * entries * 2 / (avg_ms * 1e-3) / 1e12
+        out["valu"] = {"ops_per_entry": ops, "achieved": valu, "peak": PEAK_FP32_VALU_TFLOPS, "unit": "TFLOP/s",
+                       "frac": valu / PEAK_FP32_VALU_TFLOPS,
+                       "note": "vector (non-matrix) lane instructions per state entry x entries x 2 / time: the fp32 "
+                               "rate the vector ALUs would show if every instruction were an FMA; the peak assumes "
+                               "packed FMA issue, plain fp32 instructions issue at 0.73 of it on this GPU "
+                               "(profiles/issue_rates.txt), and matrix instructions stall the vector issue of "
+                               "their SIMD for their whole duration"}
+    return out
+
+
 def bench_chunk(torch, dev, steps, warmup, gates="bf16"):
     from palimpsa_amd import _lib as L
     from palimpsa_amd.ops.palimpsa import chunk_palimpsa
@@ -70,27 +159,7 @@ def bench_chunk(torch, dev, steps, warmup, gates="bf16"):
                            leaves["Ip"], chunk_size=CHUNK)
         o.backward(do)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    # untimed reference run without the event brackets, to show what they cost
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms_plain = (time.perf_counter() - t0) * 1e3 / steps
-
-    L.profile_enable(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kern = L.profile_read()
-    L.profile_enable(False)
-
-    ms_per_step = elapsed * 1e3 / steps
+    ms_per_step, ms_median, kernels = timed_loop(torch, step, steps, warmup)
     tokens = B * T
     E = d * d
     token_heads = B * T * H
@@ -98,26 +167,18 @@ def bench_chunk(torch, dev, steps, warmup, gates="bf16"):
     flops_step = (6 * CHUNK + 14) * E * token_heads
     # share of the dominant kernel: recompute L@X (M and J) + reverse L^T@dMloc (M and J)
     flops_local = 4 * (CHUNK + 1) * E * token_heads
-    ms_local, n_local = kern.get("chunk_bwd_local_kernel", (float("nan"), 1))
-    avg_local_ms = ms_local / max(n_local, 1)
-    achieved = flops_local / (avg_local_ms * 1e-3) / 1e12
-    roofline = {
-        "bound": "mfma", "kernel": "chunk_bwd_local_kernel",
-        "achieved": achieved, "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / PEAK_BF16_MFMA_TFLOPS,
-        "traffic": MEASURED_TRAFFIC_BYTES["chunk_bwd_local_kernel"],
-        "algorithmic_flops_per_launch": flops_local,
-        "avg_launch_ms": avg_local_ms,
-        "step_frac": flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
-        "note": "flops = 4(C+1)*dk*dv per token-head (recompute + reverse triangular contractions, C=64); "
-                "step_frac uses (6C+14)*dk*dv over the whole fwd+bwd step; the kernel is bound by fp32 VALU "
-                "issue in the tile epilogues, not by the matrix cores: rocprofv3 counters show the vector ALU "
-                "of every SIMD issuing 86 % of the kernel (forward output kernel: 90 %) with the matrix pipe "
-                "busy 22 % (profiles/bench_c1.sq_counters_pmc.txt)",
-    }
-    kernels = {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()}
-    return dict(value=tokens / (ms_per_step * 1e-3), ms_per_step=ms_per_step, ms_per_step_no_events=ms_plain,
-                roofline=roofline, kernels=kernels,
+    roofline = mfma_roofline(
+        "chunk_bwd_local_kernel", kernels, flops_local, token_heads * E,
+        "flops = 4(C+1)*dk*dv per token-head (recompute + reverse triangular contractions, C=64); step_frac uses "
+        "(6C+14)*dk*dv over the whole fwd+bwd step.  The kernel is bound by fp32 vector issue in the tile epilogues "
+        "(one division per state entry), not by the matrix cores: see roofline.valu and "
+        "profiles/bench_c1.sq_counters_pmc.txt")
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES["chunk_bwd_local_kernel"]
+    roofline["step_frac"] = flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
+    out_roof = mfma_roofline("chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * token_heads, token_heads * E,
+                             "flops = 2(C+1)*dk*dv per token-head (prefix products of M and J)")
+    return dict(value=tokens / (ms_per_step * 1e-3), ms_per_step=ms_per_step, ms_per_step_median=ms_median,
+                roofline=roofline, roofline_forward=out_roof, kernels=kernels,
                 config={"workload": f"c1: chunked fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows {gates} gates fp32 states C=64",
                         "B": B, "T": T, "H": H, "dk": d, "dv": d, "chunk": CHUNK})
 
@@ -307,6 +368,141 @@ def bench_layer_slice(torch, dev, steps, warmup):
                          "algorithmic_bytes_per_launch": bytes_pb, "avg_launch_ms": avg_pb}}
 
 
+def bench_c0(torch, dev, steps, warmup, with_cpu):
+    """Config 0: fp32 token-serial forward, B=2 T=256 H=4 dk=dv=32, final states returned."""
+    from palimpsa_amd.ops.palimpsa import fused_recurrent_palimpsa
+    B, T, H, d = 2, 256, 4, 32
+    inp = make_inputs(torch, B, T, H, d, d, 0, torch.float32)
+    dv_ = {n: x.to(dev) for n, x in inp.items()}
+
+    def step():
+        fused_recurrent_palimpsa(dv_["q"], dv_["k"], dv_["v"], dv_["b"], dv_["gt"], dv_["g"], dv_["Ip"],
+                                 output_final_state=True)
+
+    ms, med, kernels = timed_loop(torch, step, steps, warmup)
+    bytes_alg = B * T * H * (4 * (2 * d + 2 * d) + 4 + 4 * d) + 2 * B * H * d * d * 4
+    k_ms = kernels.get("recurrent_fwd_kernel", {"avg_ms": float("nan")})["avg_ms"]
+    out = {"workload": "c0: fused-recurrent forward fp32 B=2 T=256 H=4 dk=dv=32, final states",
+           "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_median": med, "kernels": kernels,
+           "roofline": {"bound": "hbm", "kernel": "recurrent_fwd_kernel", "achieved": bytes_alg / (k_ms * 1e-3) / 1e9,
+                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": bytes_alg / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                        "traffic": None, "algorithmic_bytes_per_launch": bytes_alg, "avg_launch_ms": k_ms,
+                        "note": "256 dependent token steps on 64 waves: the launch is bound by serial latency "
+                                "(about 0.2 us per token), not by any throughput roofline"}}
+    if with_cpu:
+        from oracle import palimpsa_oracle as po
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            po.palimpsa_recurrence(inp["q"], inp["k"], inp["v"], inp["b"], inp["gt"], inp["g"], inp["Ip"])
+        el = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": B * T / el, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the whole configuration, forward, fp32, {el * 1e3:.1f} ms"}
+    return out
+
+
+def bench_c2(torch, dev, steps, warmup):
+    """Config 2: one packed row of 32768 tokens, documents ~ lognormal(6.5, 1.0) clipped to [16, 4096], H=16,
+    dk=dv=96, bf16, chunked forward+backward, state reset at every document boundary."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    cu = make_varlen_lengths(seed=0)
+    T, H, d = cu[-1], 16, 96
+    inp = make_inputs(torch, 1, T, H, d, d, 0, torch.bfloat16)
+    leaves = {n: inp[n].to(dev).requires_grad_(True) for n in ("q", "k", "v", "b", "gt", "g", "Ip")}
+    do = torch.randn(1, T, H, d, generator=torch.Generator().manual_seed(1)).to(dev, torch.bfloat16)
+    cu_t = torch.tensor(cu, device=dev, dtype=torch.int32)
+
+    def step():
+        for x in leaves.values():
+            x.grad = None
+        o = chunk_palimpsa(leaves["q"], leaves["k"], leaves["v"], leaves["b"], leaves["gt"], leaves["g"], leaves["Ip"],
+                           chunk_size=CHUNK, cu_seqlens=cu_t)
+        o.backward(do)
+
+    ms, med, kernels = timed_loop(torch, step, steps, warmup)
+    E, th = d * d, T * H
+    roof = mfma_roofline("chunk_bwd_local_kernel", kernels, 4 * (CHUNK + 1) * E * th, th * E,
+                         "flops = 4(C+1)*dk*dv per token-head; step_frac uses (6C+14)*dk*dv; dk = 96 runs the tile kernel "
+                         "in two passes of three column blocks")
+    roof["step_frac"] = (6 * CHUNK + 14) * E * th / (ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
+    return {"workload": f"c2: packed varlen chunked fwd+bwd, {len(cu) - 1} documents, 32768 tokens, H=16 dk=dv=96 bf16",
+            "documents": len(cu) - 1, "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_median": med,
+            "kernels": kernels, "roofline": roof}
+
+
+def bench_c4(torch, dev, steps, warmup):
+    """Config 4: chunked forward of one sequence of 65536 tokens, H=16, dk=dv=128, bf16, with a non-zero fp32
+    initial state passed in and the final state returned."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    T, H, d = 65536, 16, 128
+    inp = make_inputs(torch, 1, T, H, d, d, 0, torch.bfloat16)
+    dv_ = {n: x.to(dev) for n, x in inp.items()}
+    gen = torch.Generator().manual_seed(3)
+    mu0 = (torch.randn(1, H, d, d, generator=gen) * 0.1).to(dev)
+    I0 = (1.0 + torch.nn.functional.softplus(torch.randn(1, H, d, d, generator=gen))).to(dev)
+
+    def step():
+        with torch.no_grad():
+            chunk_palimpsa(dv_["q"], dv_["k"], dv_["v"], dv_["b"], dv_["gt"], dv_["g"], dv_["Ip"], chunk_size=CHUNK,
+                           initial_mu_state=mu0, initial_I_state=I0, output_final_state=True)
+
+    ms, med, kernels = timed_loop(torch, step, steps, warmup)
+    E, th = d * d, T * H
+    # the forward runs in windows of tiles: the per-kernel averages are per window, the flops likewise
+    n_launch = max(1, kernels.get("chunk_out_kernel", {"launches": steps})["launches"] // steps)
+    roof = mfma_roofline("chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * th / n_launch, th * E / n_launch,
+                         f"flops = 2(C+1)*dk*dv per token-head (prefix products of M and J); the sequence is run in "
+                         f"{n_launch} windows of tiles handed through the state, one launch each; step_frac uses "
+                         "(2C+6)*dk*dv over the whole forward")
+    roof["step_frac"] = (2 * CHUNK + 6) * E * th / (ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
+    return {"workload": "c4: chunked forward B=1 T=65536 H=16 dk=dv=128 bf16, initial and final state",
+            "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_median": med, "kernels": kernels,
+            "roofline": roof}
+
+
+def bench_recurrent(torch, dev, steps, warmup):
+    """Token-serial forward and backward (the reference has no such backward) at the headline batch, fp32."""
+    from palimpsa_amd.ops.palimpsa import fused_recurrent_palimpsa
+    B, T, H, d = 8, 2048, 12, 64
+    inp = make_inputs(torch, B, T, H, d, d, 0, torch.float32)
+    leaves = {n: inp[n].to(dev).requires_grad_(True) for n in ("q", "k", "v", "b", "gt", "g", "Ip")}
+    do = torch.randn(B, T, H, d, generator=torch.Generator().manual_seed(1)).to(dev)
+    names = ("q", "k", "v", "b", "gt", "g", "Ip")
+
+    def fwd():
+        with torch.no_grad():
+            fused_recurrent_palimpsa(*[leaves[n] for n in names])
+
+    def fwd_bwd():
+        for x in leaves.values():
+            x.grad = None
+        fused_recurrent_palimpsa(*[leaves[n] for n in names]).backward(do)
+
+    ms_f, med_f, k_f = timed_loop(torch, fwd, steps, warmup)
+    ms_fb, med_fb, k_fb = timed_loop(torch, fwd_bwd, steps, warmup)
+    rows = B * T * H
+    bytes_f = rows * (4 * 4 * d + 4 + 4 * d)                      # q,k,v,b in, gt in, o out (fp32)
+    bytes_b = rows * (4 * 5 * d + 4 + 4 * 4 * d + 4)              # q,k,v,b,do + gt in; dq,dk,dv,db + dgt out (fp32)
+
+    def roof(kernel, kernels, nbytes, note):
+        k_ms = kernels.get(kernel, {"avg_ms": float("nan")})["avg_ms"]
+        gbs = nbytes / (k_ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": kernel, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": gbs / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes_per_launch": nbytes, "avg_launch_ms": k_ms,
+                "note": note}
+
+    return {"workload": "token-serial forward, and forward+backward, B=8 T=2048 H=12 dk=dv=64 fp32 rows",
+            "forward": {"tokens_per_s": B * T / (ms_f * 1e-3), "ms_per_step": ms_f, "ms_per_step_median": med_f, "kernels": k_f,
+                        "roofline": roof("recurrent_fwd_kernel", k_f, bytes_f,
+                                         "rows in, outputs out; 2048 dependent steps per wave with the state in registers: "
+                                         "bound by fp32 vector work and serial latency, not by HBM")},
+            "forward_backward": {"tokens_per_s": B * T / (ms_fb * 1e-3), "ms_per_step": ms_fb, "ms_per_step_median": med_fb,
+                                 "kernels": k_fb,
+                                 "roofline": roof("recurrent_bwd_kernel", k_fb, bytes_b,
+                                                  "rows and dO in, gradients out; the kernel also re-reads its state "
+                                                  "checkpoints and writes per-tile partial sums (workspace traffic not "
+                                                  "counted as algorithmic)")}}
+
+
 def cpu_baseline(torch):
     """Naive fp32 recurrence (CPU oracle, a port of the reference's palimpsa_ref) with autograd, on a bounded
     sample of the headline workload: batch rows 0-3 of 8, all heads, all 2048 tokens (about 15 s on 16 cores,
@@ -333,7 +529,7 @@ def cpu_baseline(torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--decode-steps", type=int, default=1024)
     ap.add_argument("--gates", choices=("bf16", "fp32"), default="bf16",
@@ -343,6 +539,8 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-simple-gla", action="store_true")
     ap.add_argument("--no-layer-slice", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the legs for configurations 0, 2 and 4")
+    ap.add_argument("--no-recurrent", action="store_true", help="skip the token-serial forward/backward leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -366,13 +564,21 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     res = bench_chunk(torch, dev, args.steps, args.warmup, args.gates)
-    extra = {"kernels": res["kernels"], "ms_per_step_no_events": res["ms_per_step_no_events"]}
+    extra = {"kernels": res["kernels"], "ms_per_step_median": res["ms_per_step_median"],
+             "roofline_forward": res["roofline_forward"]}
     if not args.no_decode:
         extra["decode"] = bench_decode(torch, dev, args.decode_steps)
     if not args.no_simple_gla:
         extra["simple_gla"] = bench_simple_gla(torch, dev, args.steps, args.warmup)
     if not args.no_layer_slice:
         extra["layer_slice"] = bench_layer_slice(torch, dev, args.steps, args.warmup)
+    if not args.no_configs:
+        short = max(5, min(args.steps, 20))     # 8-10 ms per step
+        extra["c0"] = bench_c0(torch, dev, args.steps, args.warmup, not args.no_cpu_baseline)
+        extra["c2"] = bench_c2(torch, dev, short, min(args.warmup, 3))
+        extra["c4"] = bench_c4(torch, dev, short, min(args.warmup, 3))
+    if not args.no_recurrent:
+        extra["recurrent"] = bench_recurrent(torch, dev, max(3, min(args.steps, 10)), 2)
     line = {
         "metric": "chunk fwd+bwd tokens/s (H=12,d=64,T=2048) %MFMA peak; decode tokens/s %HBM BW",
         "value": res["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -318,9 +318,11 @@ int pal_chunk_bwd_supported(int32_t dk, int32_t dv);
 /* Per-kernel timing aid; no counterpart in the reference.  While enabled, every
  * kernel launch of the library is bracketed by two HIP events on the launch
  * stream; pal_profile_read waits for the outstanding ones and returns the
- * accumulated time and launch count of one kernel.  The switch and the
- * counters belong to the calling thread (thread-local): launches made by
- * other threads are neither timed nor counted.  For benchmarks only. */
+ * accumulated time and launch count of one kernel.  This is the only state
+ * of the library that calls share (launches of every thread are counted: the
+ * backward entry points run on autograd's thread); the switch is atomic and
+ * the counters are guarded by a mutex, so it is safe under concurrent callers.
+ * Off by default; for benchmarks only. */
 int pal_profile_enable(int on);               /* also resets the counters */
 int pal_profile_kernel_count(void);
 const char *pal_profile_kernel_name(int kernel_id);

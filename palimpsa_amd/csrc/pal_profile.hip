@@ -1,6 +1,10 @@
-// Per-kernel timing aid: when enabled, every kernel launch the calling thread makes through the
-// library is bracketed by two HIP events on the launch stream.  Meant for benchmarks.  All of its
-// state is thread-local, so the library keeps no mutable state that two threads share.
+// Per-kernel timing aid: when enabled, every kernel launch made through the library (from any thread:
+// autograd runs the backward entry points on a thread of its own) is bracketed by two HIP events on the
+// launch stream.  Meant for benchmarks.  This is the only state of the library that calls share; the
+// switch is an atomic flag and the event list and counters are guarded by a mutex, so concurrent callers
+// are safe whether it is on or off, and when it is off (the default) a launch only reads the flag.
+#include <atomic>
+#include <mutex>
 #include <vector>
 
 #include "pal_common.h"
@@ -9,12 +13,13 @@
 namespace pal {
 
 struct Pair { int id; hipEvent_t a, b; };
-static thread_local bool g_on = false;
-static thread_local std::vector<Pair> g_pending;
-static thread_local double g_ms[kKernCount];
-static thread_local long long g_n[kKernCount];
+static std::atomic<bool> g_on{false};
+static std::mutex g_mu;                 // guards everything below
+static std::vector<Pair> g_pending;
+static double g_ms[kKernCount];
+static long long g_n[kKernCount];
 
-ProfScope::ProfScope(int id_, hipStream_t s_) : id(id_), s(s_), e0(nullptr), on(g_on) {
+ProfScope::ProfScope(int id_, hipStream_t s_) : id(id_), s(s_), e0(nullptr), on(g_on.load(std::memory_order_relaxed)) {
   if (!on) return;
   if (hipEventCreate(&e0) != hipSuccess) { on = false; return; }
   (void)hipEventRecord(e0, s);
@@ -24,9 +29,11 @@ ProfScope::~ProfScope() {
   hipEvent_t e1;
   if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return; }
   (void)hipEventRecord(e1, s);
+  std::lock_guard<std::mutex> lk(g_mu);
   g_pending.push_back({id, e0, e1});
 }
 
+// caller holds g_mu
 static void drain() {
   for (auto& p : g_pending) {
     float ms = 0.f;
@@ -53,9 +60,10 @@ static const char* kNames[kKernCount] = {
 extern "C" {
 
 int pal_profile_enable(int on) {
+  std::lock_guard<std::mutex> lk(pal::g_mu);
   pal::drain();
   for (int i = 0; i < pal::kKernCount; ++i) { pal::g_ms[i] = 0.0; pal::g_n[i] = 0; }
-  pal::g_on = on != 0;
+  pal::g_on.store(on != 0, std::memory_order_relaxed);
   return PAL_OK;
 }
 
@@ -67,6 +75,7 @@ const char* pal_profile_kernel_name(int id) {
 
 int pal_profile_read(int id, double* total_ms, int64_t* launches) {
   if (id < 0 || id >= pal::kKernCount || !total_ms || !launches) return PAL_E_DIM;
+  std::lock_guard<std::mutex> lk(pal::g_mu);
   pal::drain();
   *total_ms = pal::g_ms[id];
   *launches = pal::g_n[id];
