@@ -45,6 +45,11 @@ extern "C" {
 /* How the chunked entry points (pal_chunk_fwd, pal_gla_chunk_fwd, pal_gla_chunk_bwd) build the states at the start
  * of every tile; no counterpart in the reference, results agree to rounding.  Neither bit: chosen by shape.
  * Meant for tests and measurements. */
+/* fp32 rows (dtype == PAL_DTYPE_F32) through the chunked entry points: by default every matrix product takes its
+ * operands as sums of two bf16 numbers (three matrix instructions per product, fp32 accumulation), which keeps
+ * outputs, states and gradients within 1e-4 (relative, max-norm) of the fp32 recurrence.  With this flag the fp32
+ * rows are rounded to single bf16 / f16 operands like bf16 rows (errors of 1e-3 .. 1e-2, about twice as fast). */
+#define PAL_FLAG_FP32_FAST 1024u
 #define PAL_FLAG_STATES_TWO_KERNELS 256u /* per-tile contributions by all tiles in parallel, then a scan over
                                             the tiles (any shape and dtype)                                  */
 #define PAL_FLAG_STATES_ONE_PASS 512u    /* one pass per (sequence, head) that keeps the running state in
@@ -223,7 +228,9 @@ int pal_gla_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
  * side .sum(0) reductions of :609-613.  Needs chunk_mu / chunk_I as written by
  * pal_chunk_fwd on the same inputs.  Head dims: one kernel keeps a dk x dv
  * carry tile in LDS, so 4 dk (dv + 8) + 256 (max(dk, dv) + 4) + 32 dv + 288 must
- * not exceed 163840 (up to 128x192, 192x128, 256x64); PAL_E_HEADDIM otherwise. */
+ * not exceed 163840 (up to 128x192, 192x128, 256x64); PAL_E_HEADDIM otherwise.
+ * fp32 rows without PAL_FLAG_FP32_FAST keep a second bf16 plane of that tile (8 dk (dv + 8) in the sum above)
+ * and take head dims up to 128 (e.g. 96x96, 64x128, 128x64). */
 size_t pal_chunk_bwd_workspace_bytes(const PalDims *dims);
 int pal_chunk_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdTensors *gr,
                   void *workspace, size_t workspace_bytes, void *stream);
@@ -309,9 +316,10 @@ int pal_epilogue_bwd(const PalGlueDims *dims, const PalEpilogueTensors *t, const
  * pal_gla_chunk_fwd never touches its fp32 scratch (chunk_mu), which may then be NULL-sized by the caller. */
 int pal_state_pass_applies(const PalDims *dims, int has_precision_state);
 
-/* PAL_OK if pal_chunk_bwd serves this head-dim pair, PAL_E_HEADDIM otherwise (see pal_chunk_bwd); lets a caller
- * refuse in its forward what its backward could not do. */
-int pal_chunk_bwd_supported(int32_t dk, int32_t dv);
+/* PAL_OK if pal_chunk_bwd serves this head-dim pair for rows of `dtype` under `flags` (PAL_FLAG_FP32_FAST is
+ * the bit that matters), PAL_E_HEADDIM otherwise (see pal_chunk_bwd); lets a caller refuse in its forward what
+ * its backward could not do. */
+int pal_chunk_bwd_supported(int32_t dk, int32_t dv, int32_t dtype, uint32_t flags);
 
 /* ------------------------------------------------------------ measurement */
 

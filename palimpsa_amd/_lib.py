@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libpalimpsa_hip.so")
 PAL_ABI_VERSION = 2
 PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
-PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS = 256, 512
+PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS, PAL_FLAG_FP32_FAST = 256, 512, 1024
 PAL_CHUNK = 64
 
 PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5
@@ -128,7 +128,7 @@ def load() -> C.CDLL:
     lib.pal_state_pass_applies.restype = C.c_int
     lib.pal_state_pass_applies.argtypes = [P(PalDims), C.c_int]
     lib.pal_chunk_bwd_supported.restype = C.c_int
-    lib.pal_chunk_bwd_supported.argtypes = [C.c_int32, C.c_int32]
+    lib.pal_chunk_bwd_supported.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_uint32]
     lib.pal_profile_enable.restype = C.c_int
     lib.pal_profile_enable.argtypes = [C.c_int]
     lib.pal_profile_kernel_count.restype = C.c_int
@@ -156,8 +156,21 @@ def set_state_pass_mode(mode: int) -> None:
     _state_pass_mode = mode
 
 
+# fp32 rows through the chunked entry points: False (default) = operands split into two bf16 halves, results within
+# 1e-4 of the fp32 recurrence; True = single bf16/f16 operands as for bf16 rows (PAL_FLAG_FP32_FAST; about twice as
+# fast, errors of 1e-3 .. 1e-2).  Initial value from the environment variable PALIMPSA_FP32_FAST.
+_fp32_fast = os.environ.get("PALIMPSA_FP32_FAST", "0") not in ("", "0")
+
+
+def set_fp32_fast(on: bool) -> None:
+    global _fp32_fast
+    _fp32_fast = bool(on)
+
+
 def state_pass_flags() -> int:
-    return (0, PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS)[_state_pass_mode]
+    """The PalDims.flags bits this Python layer adds to every call of a chunked entry point."""
+    return (0, PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS)[_state_pass_mode] | \
+        (PAL_FLAG_FP32_FAST if _fp32_fast else 0)
 
 
 def strerror(code: int) -> str:

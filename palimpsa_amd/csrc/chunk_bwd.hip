@@ -76,8 +76,11 @@ __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2
 // Every role has its own loop (its own register allocation) with the same sequence of barriers.
 // NB <= 4 column blocks are in flight at a time (16 waves); a wider head dim takes several passes over
 // the tile, the later ones adding their dv/db/gate contributions to those of the earlier ones.
-template <typename TIn, int NB, bool HAS_VAR, bool MULTI>
-__global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(4)))
+// PREC (fp32 rows): every operand is carried as two bf16 halves and every product takes three matrix instructions
+// (split_bf16 / mfma16_split); the LDS slots hold 16 operands instead of 8 and a wave may use 256 registers
+// (two waves per SIMD), so at most 2 column blocks are in flight.
+template <typename TIn, int NB, bool HAS_VAR, bool MULTI, bool PREC>
+__global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(PREC ? 2 : 4)))
 void chunk_bwd_local_roles_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
@@ -90,7 +93,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
   float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [2*NB] sums of dJloc (padded to 16 floats)
   float* sMJ = sRed + NB * kC + 16;      // [NB][2 slots][2][16] tile-start M_0, J_0 of the row in flight
-  bf16x8* sX = (bf16x8*)(sMJ + NB * 64);   // [NB][2 slots][8 operands][64 lanes]
+  constexpr int OPN = PREC ? 16 : 8;       // operands per slot (PREC: the lo halves follow the 8 hi halves)
+  bf16x8* sX = (bf16x8*)(sMJ + NB * 64);   // [NB][2 slots][OPN operands][64 lanes]
   const int tid = threadIdx.x;
   int lane = tid & 63, i = lane & 15, g = lane >> 4;   // re-derived per pass from an opaque copy, see below
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: role branches are scalar
@@ -194,6 +198,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   auto producer = [&](auto hfc) {
     constexpr int HF = decltype(hfc)::value;   // token blocks 2HF, 2HF+1 (index tl)
     bf16x8 Lop[HF ? 4 : 2];   // forward operand L[t,s], s <= t: HF=0 [tl], HF=1 [2tl+ks]
+    bf16x8 Lol[PREC ? (HF ? 4 : 2) : 1];   // PREC: its lo halves
     float kk[HF ? 16 : 8];    // k in operand layout (n = i, s = 8g+j+32ks)
     float qq[8];              // q in result layout (t = 16tb+4g+r, n = i)
     float dq[8];
@@ -218,7 +223,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
           for (int tl = 0; tl < 2; ++tl) {
             const int t = 16 * (2 * HF + tl) + i;
-            Lop[HF ? 2 * tl + ks : tl][j] = (bf16_t)((s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f);
+            const float lv = (s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f;
+            const bf16_t lh = (bf16_t)lv;
+            Lop[HF ? 2 * tl + ks : tl][j] = lh;
+            if constexpr (PREC) Lol[HF ? 2 * tl + ks : tl][j] = (bf16_t)(lv - (float)lh);
           }
         }
       }
@@ -257,12 +265,25 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + i] = J0;
         }
         bf16x8 XM[HF + 1], XJ[HF + 1];
+        bf16x8 XMl[PREC ? HF + 1 : 1], XJl[PREC ? HF + 1 : 1];
 #pragma unroll
         for (int ks = 0; ks <= HF; ++ks) {
           const f32x4 v0 = *(const f32x4*)&sV[8 * g + 32 * ks];
           const f32x4 v1 = *(const f32x4*)&sV[8 * g + 32 * ks + 4];
           const f32x4 b0 = *(const f32x4*)&sB[8 * g + 32 * ks];
           const f32x4 b1 = *(const f32x4*)&sB[8 * g + 32 * ks + 4];
+          if constexpr (PREC) {
+            float xm[8], xj[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float vv = j < 4 ? v0[j & 3] : v1[j & 3], bb = j < 4 ? b0[j & 3] : b1[j & 3];
+              const float kx = kk[ks * 8 + j];
+              xm[j] = kx * vv;
+              xj[j] = (kx * bb) * kx;
+            }
+            split_bf16(xm, XM[ks], XMl[ks]);
+            split_bf16(xj, XJ[ks], XJl[ks]);
+          } else {
 #pragma unroll
           for (int j = 0; j < 8; j += 2) {
             const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
@@ -273,18 +294,29 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
             XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
           }
+          }
         }
         bf16x8 PM, PJ;
+        float pmf[PREC ? 8 : 1], pjf[PREC ? 8 : 1];   // PREC: the local gradients in fp32 until they are split
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl) {
           const int tb = 2 * HF + tl;
           f32x4 accM = {0.f, 0.f, 0.f, 0.f};
           f32x4 accI = {Ip, Ip, Ip, Ip};
+          if constexpr (PREC) {
+            accM = mfma16_split(Lop[HF ? 2 * tl : tl], Lol[HF ? 2 * tl : tl], XM[0], XMl[0], accM);
+            accI = mfma16_split(Lop[HF ? 2 * tl : tl], Lol[HF ? 2 * tl : tl], XJ[0], XJl[0], accI);
+            if (HF) {
+              accM = mfma16_split(Lop[2 * tl + HF], Lol[2 * tl + HF], XM[HF], XMl[HF], accM);
+              accI = mfma16_split(Lop[2 * tl + HF], Lol[2 * tl + HF], XJ[HF], XJl[HF], accI);
+            }
+          } else {
           accM = mfma16(Lop[HF ? 2 * tl : tl], XM[0], accM);
           accI = mfma16(Lop[HF ? 2 * tl : tl], XJ[0], accI);
           if (HF) {
             accM = mfma16(Lop[2 * tl + HF], XM[HF], accM);
             accI = mfma16(Lop[2 * tl + HF], XJ[HF], accI);
+          }
           }
           const f32x4 Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
           const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
@@ -309,13 +341,25 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             }
             sigacc += dJl[r];
           }
+          const int o4 = tl * 4;
+          if constexpr (PREC) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { pmf[o4 + r] = dMl[r]; pjf[o4 + r] = dJl[r]; }
+          } else {
           const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
           const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
-          const int o4 = tl * 4;
           PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
           PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
+          }
         }
-        bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * 8) * 64 + lane;
+        bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
+        if constexpr (PREC) {
+          bf16x8 PMl, PJl;
+          split_bf16(pmf, PM, PMl);
+          split_bf16(pjf, PJ, PJl);
+          slot[(8 + 0 + HF) * 64] = PMl; slot[(8 + 2 + HF) * 64] = PJl;
+          slot[(8 + 4 + HF) * 64] = XMl[HF]; slot[(8 + 6 + HF) * 64] = XJl[HF];
+        }
         slot[(0 + HF) * 64] = PM; slot[(2 + HF) * 64] = PJ;
         slot[(4 + HF) * 64] = XM[HF]; slot[(6 + HF) * 64] = XJ[HF];
       }
@@ -338,6 +382,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   auto consumer = [&](auto hfc) {
     constexpr int HF = decltype(hfc)::value;   // column-token blocks 2HF, 2HF+1 (index sl)
     bf16x8 Lop[6];    // reverse operand, HF=0 [2sl+p], HF=1 [sl] (p=1); strictly-lower operand, HF=0 [4+sl], HF=1 [2+2sl+ks]
+    bf16x8 Lol[PREC ? 6 : 1];   // PREC: its lo halves
     float kr[8];      // k in result layout (s = 16sb+i, n = 4g+r)
     float dkM[8], dkJ[8];
     float gate[2], Fs[2];
@@ -358,7 +403,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
           for (int sl = 0; sl < 2; ++sl) {
             const int t = 16 * (2 * HF + sl) + i;
-            Lop[HF ? 2 + 2 * sl + ks : 4 + sl][j] = (bf16_t)((s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f);
+            const float lv = (s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
+            const bf16_t lh = (bf16_t)lv;
+            Lop[HF ? 2 + 2 * sl + ks : 4 + sl][j] = lh;
+            if constexpr (PREC) Lol[HF ? 2 + 2 * sl + ks : 4 + sl][j] = (bf16_t)(lv - (float)lh);
           }
         }
       }
@@ -374,7 +422,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int t = 16 * (2 * p + (j >> 2)) + 4 * g + (j & 3);
-            Lop[HF ? sl : 2 * sl + p][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f);
+            const float lv = (t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f;
+            const bf16_t lh = (bf16_t)lv;
+            Lop[HF ? sl : 2 * sl + p][j] = lh;
+            if constexpr (PREC) Lol[HF ? sl : 2 * sl + p][j] = (bf16_t)(lv - (float)lh);
           }
         }
       }
@@ -401,12 +452,18 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         const int d = it - 1, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
-        const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * 8) * 64 + lane;
+        const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
         // HF=0 (column tokens 0..31): reverse needs both P halves, strictly-lower only X_0;
         // HF=1 (column tokens 32..63): reverse needs P_1 only, strictly-lower both X halves
         const bf16x8 PM1 = slot[1 * 64], PJ1 = slot[3 * 64], XM0 = slot[4 * 64], XJ0 = slot[6 * 64];
         const bf16x8 Ma = slot[(HF ? 5 : 0) * 64];   // HF=0: P^M_0, HF=1: X^M_1
         const bf16x8 Ja = slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
+        bf16x8 PM1l, PJ1l, XM0l, XJ0l, Mal, Jal;     // PREC: the lo halves of the six
+        if constexpr (PREC) {
+          PM1l = slot[(8 + 1) * 64]; PJ1l = slot[(8 + 3) * 64]; XM0l = slot[(8 + 4) * 64]; XJ0l = slot[(8 + 6) * 64];
+          Mal = slot[(8 + (HF ? 5 : 0)) * 64];
+          Jal = slot[(8 + (HF ? 7 : 2)) * 64];
+        }
         const f32x4 M0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 4 * g];
         const f32x4 J0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + 4 * g];
         float dvp[2], dbp[2];
@@ -415,7 +472,23 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           const int sb = 2 * HF + sl;
           f32x4 aM = {0.f, 0.f, 0.f, 0.f}, aJ = {0.f, 0.f, 0.f, 0.f};
           f32x4 sM = {0.f, 0.f, 0.f, 0.f}, sJ = {0.f, 0.f, 0.f, 0.f};
-          if (!HF) {
+          if constexpr (PREC) {
+            if (!HF) {
+              aM = mfma16_split(Ma, Mal, Lop[2 * sl], Lol[2 * sl], aM);
+              aJ = mfma16_split(Ja, Jal, Lop[2 * sl], Lol[2 * sl], aJ);
+              aM = mfma16_split(PM1, PM1l, Lop[2 * sl + 1], Lol[2 * sl + 1], aM);
+              aJ = mfma16_split(PJ1, PJ1l, Lop[2 * sl + 1], Lol[2 * sl + 1], aJ);
+              sM = mfma16_split(XM0, XM0l, Lop[4 + sl], Lol[4 + sl], sM);
+              sJ = mfma16_split(XJ0, XJ0l, Lop[4 + sl], Lol[4 + sl], sJ);
+            } else {
+              aM = mfma16_split(PM1, PM1l, Lop[sl], Lol[sl], aM);
+              aJ = mfma16_split(PJ1, PJ1l, Lop[sl], Lol[sl], aJ);
+              sM = mfma16_split(XM0, XM0l, Lop[2 + 2 * sl], Lol[2 + 2 * sl], sM);
+              sJ = mfma16_split(XJ0, XJ0l, Lop[2 + 2 * sl], Lol[2 + 2 * sl], sJ);
+              sM = mfma16_split(Ma, Mal, Lop[2 + 2 * sl + 1], Lol[2 + 2 * sl + 1], sM);
+              sJ = mfma16_split(Ja, Jal, Lop[2 + 2 * sl + 1], Lol[2 + 2 * sl + 1], sJ);
+            }
+          } else if (!HF) {
             aM = mfma16(Ma, Lop[2 * sl], aM);
             aJ = mfma16(Ja, Lop[2 * sl], aJ);
             aM = mfma16(PM1, Lop[2 * sl + 1], aM);
@@ -595,7 +668,9 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
 // SEQ the dv and db products take turns in one result buffer: less LDS, so that more workgroups share
 // a compute unit (the kernel is a chain of dependent load, product and store phases, and it is the
 // number of resident workgroups that hides them).
-template <typename TIn, int KSMAX, bool SEQ>
+// PREC (fp32 rows): operands as two bf16 halves, three matrix instructions per product; the transposed copy of the
+// carries then holds a second plane with the lo halves (never shared with a result buffer).
+template <typename TIn, int KSMAX, bool SEQ, bool PREC>
 __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
@@ -612,6 +687,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const bool alias = !SEQ && A.apply_alias != 0;
   bf16_t* sRT = (bf16_t*)(alias ? sO2 : sO2 + kC * (dmax + 4));
   const int RS = dv + 8;
+  bf16_t* sRTl = sRT + 2 * dk * RS;        // PREC: [2][dk][dv + 8] lo halves
   const int OS = dmax + 4;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
@@ -671,8 +747,13 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
       for (int x = 0; x < 4; ++x) {
         acc = fmaf(rm[x], mu[x] * I[x], acc);
         acc = fmaf(rj[x], I[x] - Ipb, acc);
-        sRT[(4 * c4 + x) * RS + d] = (bf16_t)rm[x];
-        sRT[(dk + 4 * c4 + x) * RS + d] = (bf16_t)rj[x];
+        const bf16_t mh = (bf16_t)rm[x], jh = (bf16_t)rj[x];
+        sRT[(4 * c4 + x) * RS + d] = mh;
+        sRT[(dk + 4 * c4 + x) * RS + d] = jh;
+        if constexpr (PREC) {
+          sRTl[(4 * c4 + x) * RS + d] = (bf16_t)(rm[x] - (float)mh);
+          sRTl[(dk + 4 * c4 + x) * RS + d] = (bf16_t)(rj[x] - (float)jh);
+        }
       }
     }
     acc = wave_sum(acc);
@@ -691,6 +772,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   {
     const int KS = (dv + 31) / 32;
     bf16x8 A3[KSMAX], A4[KSMAX];
+    bf16x8 A3l[PREC ? KSMAX : 1], A4l[PREC ? KSMAX : 1];
     const TIn* vp = (const TIn*)a.v + tokA * dv;
     const TIn* bp = (const TIn*)a.b + tokA * dv;
 #pragma unroll
@@ -705,10 +787,17 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) { vv[j] = 0.f; bb[j] = 0.f; }
         }
+        if constexpr (PREC) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { vv[j] *= as; bb[j] *= as; }
+          split_bf16(vv, A3[ks], A3l[ks]);
+          split_bf16(bb, A4[ks], A4l[ks]);
+        } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           A3[ks][j] = (bf16_t)(as * vv[j]);
           A4[ks][j] = (bf16_t)(as * bb[j]);
+        }
         }
       }
     }
@@ -739,8 +828,18 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) { B3[j] = (bf16_t)0.f; B4[j] = (bf16_t)0.f; }
           }
+          if constexpr (PREC) {
+            bf16x8 B3l = B3, B4l = B4;   // zero beyond dv
+            if (d0 < dv) {
+              B3l = *(const bf16x8*)&sRTl[(16 * nbk + i) * RS + d0];
+              B4l = *(const bf16x8*)&sRTl[(dk + 16 * nbk + i) * RS + d0];
+            }
+            accM = mfma16_split(A3[ks], A3l[ks], B3, B3l, accM);
+            accJ = mfma16_split(A4[ks], A4l[ks], B4, B4l, accJ);
+          } else {
           accM = mfma16(A3[ks], B3, accM);
           accJ = mfma16(A4[ks], B4, accJ);
+          }
         }
       }
       // rows s = 16w + 4g + r, column n = 16nbk + i
@@ -774,6 +873,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   {
     const int KS = (dk + 31) / 32;
     bf16x8 A1[KSMAX], A2[KSMAX];
+    bf16x8 A1l[PREC ? KSMAX : 1], A2l[PREC ? KSMAX : 1];
     const TIn* kp = (const TIn*)a.k + tokA * dk;
 #pragma unroll
     for (int ks = 0; ks < KSMAX; ++ks) {
@@ -787,10 +887,18 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) kv[j] = 0.f;
         }
+        if constexpr (PREC) {
+          float k1[8], k2[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { k1[j] = as * kv[j]; k2[j] = k1[j] * kv[j]; }
+          split_bf16(k1, A1[ks], A1l[ks]);
+          split_bf16(k2, A2[ks], A2l[ks]);
+        } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           A1[ks][j] = (bf16_t)(as * kv[j]);
           A2[ks][j] = (bf16_t)(as * kv[j] * kv[j]);
+        }
         }
       }
     }
@@ -812,6 +920,19 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
             bf16x8 B1, B2;
 #pragma unroll
             for (int j = 0; j < 8; ++j) { B1[j] = (bf16_t)0.f; B2[j] = (bf16_t)0.f; }
+            bf16x8 B1l = B1, B2l = B2;
+            if constexpr (PREC) {
+              if (n0 < dk) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                  if (doV) { B1[j] = sRT[(n0 + j) * RS + 16 * db_ + i]; B1l[j] = sRTl[(n0 + j) * RS + 16 * db_ + i]; }
+                  if (doB) { B2[j] = sRT[(dk + n0 + j) * RS + 16 * db_ + i]; B2l[j] = sRTl[(dk + n0 + j) * RS + 16 * db_ + i]; }
+                }
+              }
+              if (doV) accV = mfma16_split(A1[ks], A1l[ks], B1, B1l, accV);
+              if (doB) accB = mfma16_split(A2[ks], A2l[ks], B2, B2l, accB);
+              continue;
+            }
             if (n0 < dk && !alias) {
               // 8 consecutive key columns of value row d = 16db_ + i: a column walk through the transposed
               // bf16 copy in LDS (the fp32 carries in global memory would miss L2 on this second read)
@@ -950,12 +1071,13 @@ struct BwdPlan {
   int apply_alias, apply_seq, apply_ksmax;
 };
 
-static size_t local_lds_bytes(int NB, bool var) {
+static size_t local_lds_bytes(int NB, bool var, bool prec) {
   return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
-         (size_t)NB * 2 * 8 * 64 * 16;
+         (size_t)NB * 2 * (prec ? 16 : 8) * 64 * 16;
 }
 
-static int bwd_plan(int dk, int dv, bool var, BwdPlan& P) {
+// prec: the fp32-accurate variants (fp32 rows without PAL_FLAG_FP32_FAST)
+static int bwd_plan(int dk, int dv, bool var, bool prec, BwdPlan& P) {
   const int nb_total = dk / 16;
   if (nb_total < 1 || nb_total > 16) return PAL_E_HEADDIM;
   // At most 4 column blocks (16 waves, 128 registers each: one workgroup per compute unit) in flight; wider heads
@@ -963,14 +1085,16 @@ static int bwd_plan(int dk, int dv, bool var, BwdPlan& P) {
   // 8 waves then share a compute unit and fill each other's barrier waits, which measured 14-17 % faster than
   // passes of 3 (12 waves, one workgroup per unit) at dk = 80 and 96 and the same as 4 + 3 at dk = 112.
   P.nb_local = nb_total <= 4 ? nb_total : (nb_total % 4 == 0 ? 4 : 2);
-  P.lds_local = local_lds_bytes(P.nb_local, var);
+  if (prec && P.nb_local > 2) P.nb_local = 2;   // 16-operand slots: at most two column blocks fit the LDS
+  P.lds_local = local_lds_bytes(P.nb_local, var, prec);
   if (P.lds_local > kMaxLds) return PAL_E_HEADDIM;
   const int dmax = dk > dv ? dk : dv;
-  const size_t rt_bytes = 2 * (size_t)2 * dk * (dv + 8), o_bytes = sizeof(float) * kC * (dmax + 4);
+  const size_t rt_bytes = (prec ? 2 : 1) * 2 * (size_t)2 * dk * (dv + 8), o_bytes = sizeof(float) * kC * (dmax + 4);
+  if (prec && dmax > 128) return PAL_E_HEADDIM;
   const size_t lds_fixed = sizeof(float) * (kC + 8 + kC * (dv >> 3)) + o_bytes;
   size_t lds = lds_fixed + o_bytes + rt_bytes;
   P.apply_alias = 0;
-  if (lds > kMaxLds) {
+  if (lds > kMaxLds && !prec) {
     P.apply_alias = 1;
     lds = lds_fixed + (rt_bytes > o_bytes ? rt_bytes : o_bytes);
   }
@@ -984,14 +1108,14 @@ static int bwd_plan(int dk, int dv, bool var, BwdPlan& P) {
   return PAL_OK;
 }
 
-template <typename TIn, int NB>
+template <typename TIn, int NB, bool PREC>
 static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   const bool var = A.c.flags & PAL_FLAG_HAS_VAR;
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   // four wave roles per block of 16 key columns, NB such blocks at a time (see chunk_bwd_local_roles_kernel)
   const int NT = 4 * NB * 64;
-  const size_t lds = local_lds_bytes(NB, var);
+  const size_t lds = local_lds_bytes(NB, var, PREC);
   if (lds > kMaxLds) return PAL_E_HEADDIM;
   const bool multi = A.c.dk != 16 * NB;
   auto go = [&](auto kern) -> int {
@@ -1001,39 +1125,40 @@ static int launch_local_nb(const BwdArgs& A, hipStream_t s) {
   };
   int rc;
   if constexpr (NB == 2 || NB == 4) {   // the only block counts that run several passes (see bwd_plan)
-    if (multi) rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, true>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, true>);
-    else rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false>);
+    if (multi) rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, true, PREC>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, true, PREC>);
+    else rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false, PREC>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false, PREC>);
   } else {
-    rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false>);
+    rc = var ? go(&chunk_bwd_local_roles_kernel<TIn, NB, true, false, PREC>) : go(&chunk_bwd_local_roles_kernel<TIn, NB, false, false, PREC>);
   }
   if (rc) return rc;
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
 
-template <typename TIn>
+template <typename TIn, bool PREC>
 static int launch_local(const BwdArgs& A, const BwdPlan& P, hipStream_t s) {
   switch (P.nb_local) {
-    case 1: return launch_local_nb<TIn, 1>(A, s);
-    case 2: return launch_local_nb<TIn, 2>(A, s);
-    case 3: return launch_local_nb<TIn, 3>(A, s);
-    case 4: return launch_local_nb<TIn, 4>(A, s);
+    case 1: return launch_local_nb<TIn, 1, PREC>(A, s);
+    case 2: return launch_local_nb<TIn, 2, PREC>(A, s);
+    case 3: if constexpr (!PREC) return launch_local_nb<TIn, 3, false>(A, s); else return PAL_E_HEADDIM;
+    case 4: if constexpr (!PREC) return launch_local_nb<TIn, 4, false>(A, s); else return PAL_E_HEADDIM;
     default: return PAL_E_HEADDIM;
   }
 }
 
-template <typename TIn, int KSMAX, bool SEQ>
+template <typename TIn, int KSMAX, bool SEQ, bool PREC>
 static int launch_carry_apply_t(const BwdArgs& A, unsigned blocks, size_t lds, hipStream_t s) {
-  if (int rc = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ>, lds)) return rc;
-  PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ>), dim3(blocks), dim3(256), lds, s, A);
+  if (int rc = allow_lds((const void*)&chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ, PREC>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kKernBwdCarryApply, s, (chunk_bwd_carry_apply_kernel<TIn, KSMAX, SEQ, PREC>), dim3(blocks), dim3(256), lds, s, A);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
-template <typename TIn>
+template <typename TIn, bool PREC>
 static int launch_carry_apply(const BwdArgs& A, int ksmax, bool seq, unsigned blocks, size_t lds, hipStream_t s) {
-  if (ksmax == 2) return seq ? launch_carry_apply_t<TIn, 2, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 2, false>(A, blocks, lds, s);
-  if (ksmax == 4) return seq ? launch_carry_apply_t<TIn, 4, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 4, false>(A, blocks, lds, s);
-  return seq ? launch_carry_apply_t<TIn, 8, true>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 8, false>(A, blocks, lds, s);
+  if (ksmax == 2) return seq ? launch_carry_apply_t<TIn, 2, true, PREC>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 2, false, PREC>(A, blocks, lds, s);
+  if (ksmax == 4) return seq ? launch_carry_apply_t<TIn, 4, true, PREC>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 4, false, PREC>(A, blocks, lds, s);
+  if constexpr (PREC) return PAL_E_HEADDIM;   // the split operands of 256-wide heads do not fit the registers
+  else return seq ? launch_carry_apply_t<TIn, 8, true, false>(A, blocks, lds, s) : launch_carry_apply_t<TIn, 8, false, false>(A, blocks, lds, s);
 }
 
 }  // namespace pal
@@ -1041,14 +1166,16 @@ static int launch_carry_apply(const BwdArgs& A, int ksmax, bool seq, unsigned bl
 extern "C" size_t pal_chunk_bwd_workspace_bytes(const PalDims* d) {
   if (pal_validate_dims(d) != PAL_OK || d->total_chunks <= 0) return 0;
   pal::BwdPlan P;
-  if (pal::bwd_plan(d->dk, d->dv, (d->flags & PAL_FLAG_HAS_VAR) != 0, P) != PAL_OK) return 0;
+  const bool prec = d->dtype == PAL_DTYPE_F32 && !(d->flags & PAL_FLAG_FP32_FAST);
+  if (pal::bwd_plan(d->dk, d->dv, (d->flags & PAL_FLAG_HAS_VAR) != 0, prec, P) != PAL_OK) return 0;
   return pal::bwd_layout(d).total;
 }
 
-extern "C" int pal_chunk_bwd_supported(int32_t dk, int32_t dv) {
+extern "C" int pal_chunk_bwd_supported(int32_t dk, int32_t dv, int32_t dtype, uint32_t flags) {
   if (dk < 16 || dk > 256 || (dk & 15) || dv < 16 || dv > 256 || (dv & 15)) return PAL_E_HEADDIM;
+  if (dtype != PAL_DTYPE_F32 && dtype != PAL_DTYPE_BF16) return PAL_E_DTYPE;
   pal::BwdPlan P;
-  return pal::bwd_plan(dk, dv, true, P);
+  return pal::bwd_plan(dk, dv, true, dtype == PAL_DTYPE_F32 && !(flags & PAL_FLAG_FP32_FAST), P);
 }
 
 extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const PalBwdTensors* gr, void* workspace,
@@ -1067,7 +1194,8 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   rc = check_bwd_common(&dd, gr);
   if (rc) return rc;
   BwdPlan P;
-  rc = bwd_plan(dd.dk, dd.dv, (dd.flags & PAL_FLAG_HAS_VAR) != 0, P);
+  const bool prec = dd.dtype == PAL_DTYPE_F32 && !(dd.flags & PAL_FLAG_FP32_FAST);
+  rc = bwd_plan(dd.dk, dd.dv, (dd.flags & PAL_FLAG_HAS_VAR) != 0, prec, P);
   if (rc) return rc;
   if ((int64_t)dd.total_chunks * dd.n_heads > 0x7fffffff ||
       (int64_t)dd.n_seqs * dd.n_heads * carry_scan_blocks((int64_t)dd.dv * dd.dk) > 0x7fffffff)
@@ -1089,7 +1217,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   A.tokens = dd.batch * dd.seq_len;
   hipStream_t s = (hipStream_t)stream;
   const bool bf = dd.dtype == PAL_DTYPE_BF16;
-  rc = bf ? launch_local<bf16_t>(A, P, s) : launch_local<float>(A, P, s);
+  rc = bf ? launch_local<bf16_t, false>(A, P, s) : prec ? launch_local<float, true>(A, P, s) : launch_local<float, false>(A, P, s);
   if (rc) return rc;
   {
     const int64_t blocks = (int64_t)dd.n_seqs * dd.n_heads * carry_scan_blocks((int64_t)dd.dv * dd.dk);
@@ -1101,8 +1229,9 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   {
     const unsigned blocks = (unsigned)((int64_t)dd.total_chunks * dd.n_heads);
     A.apply_alias = P.apply_alias;
-    rc = bf ? launch_carry_apply<bf16_t>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s)
-            : launch_carry_apply<float>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s);
+    rc = bf     ? launch_carry_apply<bf16_t, false>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s)
+         : prec ? launch_carry_apply<float, true>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s)
+                : launch_carry_apply<float, false>(A, P.apply_ksmax, P.apply_seq != 0, blocks, P.lds_apply, s);
     if (rc) return rc;
     PAL_HIP_LAUNCH_CHECK();
   }

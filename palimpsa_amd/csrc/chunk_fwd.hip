@@ -15,6 +15,7 @@
 //      the reference kernel, :190-207).  Output orientation is [n, t] so the
 //      sum over n stays inside a lane.
 #include <atomic>
+#include <type_traits>
 
 #include "chunk_common.h"
 #include "pal_host.h"
@@ -89,17 +90,21 @@ __device__ __forceinline__ void staged8(const bf16_t* p, float* out) {
 
 // HAS_J = false drops the precision branch (b is not read, chunk_I is not written): the scalar-gated linear
 // attention that the layer uses without its precision state.
-template <typename TIn, bool HAS_J, typename TS>
-__global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
+// PREC (fp32 rows staged in fp32): operands split into two bf16 halves, three matrix instructions per product.
+template <typename TIn, bool HAS_J, typename TS, bool PREC>
+__global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a, int dvn) {
+  // blockIdx.y selects a piece of dvn value rows (dvn = dv: one piece; smaller where the staging tiles of all rows
+  // would not fit the LDS)
   extern __shared__ float smem[];
   constexpr int kTS = StageStride<TS>::value;
   const int H = a.H, dk = a.dk, dv = a.dv;
+  const int d0 = blockIdx.y * dvn, dn = min(dvn, dv - d0);
   float* sA = smem;                 // [64] decay from token s to the end of the tile
   TS* sKT = (TS*)(sA + kC);         // [dk][kTS]
-  TS* sVT = sKT + dk * kTS;         // [dv][kTS]
-  TS* sBT = sVT + dv * kTS;         // [dv][kTS]
+  TS* sVT = sKT + dk * kTS;         // [dvn][kTS]
+  TS* sBT = sVT + dvn * kTS;        // [dvn][kTS]
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
-  const int NB = dk >> 4, ND = dv >> 4;
+  const int NB = dk >> 4, ND = dn >> 4;
   const int cidx = blockIdx.x / H, h = blockIdx.x % H;
   int seq, t0, clen, cis;
   chunk_lookup(a, cidx, seq, t0, clen, cis);
@@ -110,45 +115,68 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a) {
     sA[lane] = fast_exp2((a.flags & kFlagDecayFromStart) ? cs : __shfl(cs, 63) - cs);
   }
   stage_transposed((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, (int64_t)H * dk, dk, clen, sKT, tid);
-  stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sVT, tid);
-  if (HAS_J) stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv, (int64_t)H * dv, dv, clen, sBT, tid);
+  stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv + d0, (int64_t)H * dv, dn, clen, sVT, tid);
+  if (HAS_J) stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv + d0, (int64_t)H * dv, dn, clen, sBT, tid);
   __syncthreads();
   float as[2][8];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) staged8(&sA[8 * g + 32 * ks], as[ks]);
   for (int nb = w; nb < NB; nb += 4) {
-    bf16x8 BK[2], BKK[2];
+    bf16x8 BK[2], BKK[2], BKl[2], BKKl[2];   // the *l halves only exist with PREC
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       float kv[8];
       staged8(&sKT[(16 * nb + i) * kTS + 8 * g + 32 * ks], kv);
+      if constexpr (PREC) {
+        float kq[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        BK[ks][j] = (bf16_t)kv[j];
-        BKK[ks][j] = (bf16_t)(kv[j] * kv[j]);
+        for (int j = 0; j < 8; ++j) kq[j] = kv[j] * kv[j];
+        split_bf16(kv, BK[ks], BKl[ks]);
+        split_bf16(kq, BKK[ks], BKKl[ks]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          BK[ks][j] = (bf16_t)kv[j];
+          BKK[ks][j] = (bf16_t)(kv[j] * kv[j]);
+        }
       }
     }
     for (int dt = 0; dt < ND; ++dt) {
-      bf16x8 AM[2], AJ[2];
+      bf16x8 AM[2], AJ[2], AMl[2], AJl[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         float vv[8], bb[8];
         staged8(&sVT[(16 * dt + i) * kTS + 8 * g + 32 * ks], vv);
         if (HAS_J) staged8(&sBT[(16 * dt + i) * kTS + 8 * g + 32 * ks], bb);
+        if constexpr (PREC) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          AM[ks][j] = (bf16_t)(as[ks][j] * vv[j]);
-          if (HAS_J) AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
+          for (int j = 0; j < 8; ++j) { vv[j] *= as[ks][j]; if (HAS_J) bb[j] *= as[ks][j]; }
+          split_bf16(vv, AM[ks], AMl[ks]);
+          if (HAS_J) split_bf16(bb, AJ[ks], AJl[ks]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            AM[ks][j] = (bf16_t)(as[ks][j] * vv[j]);
+            if (HAS_J) AJ[ks][j] = (bf16_t)(as[ks][j] * bb[j]);
+          }
         }
       }
       // the products are taken transposed (K as the row operand) so that a lane ends up with four consecutive
       // key columns of one value row: rows n = 16nb + 4g + r, column d = 16dt + i, one 16-byte store per lane
       f32x4 M = {0.f, 0.f, 0.f, 0.f}, J = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (PREC) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          M = mfma16_split(BK[ks], BKl[ks], AM[ks], AMl[ks], M);
+          if (HAS_J) J = mfma16_split(BKK[ks], BKKl[ks], AJ[ks], AJl[ks], J);
+        }
+      } else {
       M = mfma16(BK[0], AM[0], M);
       if (HAS_J) J = mfma16(BKK[0], AJ[0], J);
       M = mfma16(BK[1], AM[1], M);
       if (HAS_J) J = mfma16(BKK[1], AJ[1], J);
-      const int64_t co = (((int64_t)cidx * H + h) * dv + 16 * dt + i) * dk + 16 * nb + 4 * g;
+      }
+      const int64_t co = (((int64_t)cidx * H + h) * dv + d0 + 16 * dt + i) * dk + 16 * nb + 4 * g;
       *(f32x4*)&a.chunk_mu[co] = M;
       if (HAS_J) *(f32x4*)&a.chunk_I[co] = J;
     }
@@ -304,11 +332,14 @@ __device__ __forceinline__ constexpr int lidx(int tb, int ks) { return tb < 2 ? 
 // time for 5, 6, 7 and 8 column blocks).  With two waves per column block the waves spread evenly.
 // TS > 1 gives a workgroup TS (tile, head) pairs, each with its own NB * RS waves and its own piece of LDS (they only
 // share the barriers), so that a workgroup of two waves becomes one of four and covers all four SIMDs.
-template <typename TIn, int NB, bool HAS_VAR, int RS, int TS>
+// PREC (fp32 rows): the rows are staged in fp32, the operands X and L are formed in fp32 and split into two bf16
+// halves each, three matrix instructions per product (no block exponents: bf16 has the range of fp32).
+template <typename TIn, int NB, bool HAS_VAR, int RS, int TS, bool PREC>
 __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
+  using TSt = std::conditional_t<PREC, float, f16_t>;   // element type of the staged v, b rows
   constexpr int NT = NB * RS * 64;        // threads per (tile, head)
-  constexpr int kTileFloats = kC + (HAS_VAR ? 2 : 1) * NB * kDG * kC + (4 * kDG * kVH) / 2;
+  constexpr int kTileFloats = kC + (HAS_VAR ? 2 : 1) * NB * kDG * kC + (4 * kDG * kVH * (int)sizeof(TSt)) / 4;
   const int sub = TS == 1 ? 0 : (int)threadIdx.x / NT;
   const int tid = (int)threadIdx.x - sub * NT;
   const int64_t n_items = (int64_t)a.total_chunks * a.H;
@@ -316,8 +347,8 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   const bool valid = item_raw < n_items;          // a spare group of the last workgroup repeats the last item, unstored
   const int64_t item = valid ? item_raw : n_items - 1;
   float* sC = smem + sub * kTileFloats;   // [64] running log2-decay inside the tile
-  f16_t* sV = (f16_t*)(sC + kC);          // [2][16][kVH] v^T 2^-E of the current and the next value-row group, f16
-  f16_t* sB = sV + 2 * kDG * kVH;         // [2][16][kVH] b^T 2^-E
+  TSt* sV = (TSt*)(sC + kC);              // [2][16][kVH] v^T 2^-E of the current and the next value-row group
+  TSt* sB = sV + 2 * kDG * kVH;           // [2][16][kVH] b^T 2^-E
   float* sO = (float*)(sB + 2 * kDG * kVH);   // [NB][16][64] per-wave partial outputs
   float* sOv = sO + NB * kDG * kC;        // same for o_var
   const int lane = tid & 63, i = lane & 15, g = lane >> 4;
@@ -382,8 +413,9 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   }
   stage_load(0);
   // block exponents of the f16 operands (see tile_block_exponents); sO doubles as its scratch
-  const TileExponents bexp =
-      tile_block_exponents((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
+  TileExponents bexp = {0, 0, 0};
+  if constexpr (!PREC)
+    bexp = tile_block_exponents((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
   const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
   const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
   const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
@@ -395,8 +427,8 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
       if (idx < kC * kDG / 4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          sV[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(vst[it][e] * down_v);
-          sB[(buf * kDG + 4 * dq + e) * kVH + s] = (f16_t)(bst[it][e] * down_b);
+          sV[(buf * kDG + 4 * dq + e) * kVH + s] = (TSt)(vst[it][e] * down_v);
+          sB[(buf * kDG + 4 * dq + e) * kVH + s] = (TSt)(bst[it][e] * down_b);
         }
       }
     }
@@ -418,6 +450,9 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   }
   f16x8 Lr[6];            // decay operand
   f16x8 kA[2], kk[2];     // k and k*k of the wave's key column for the 64 tokens, operand layout
+  // the same with PREC: the decay operand as two bf16 halves, k and k*k in fp32 (the products are split per row)
+  bf16x8 Lh[PREC ? 6 : 1], Ll[PREC ? 6 : 1];
+  float kf[PREC ? 2 : 1][8], kkf[PREC ? 2 : 1][8];
   {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -428,13 +463,24 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
       for (int j = 0; j < 8; ++j) {
         const int s = 8 * g + j + 32 * ks;
         const float ksc = kraw[ks][j] * down_k;
-        kA[ks][j] = (f16_t)ksc;
-        kk[ks][j] = (f16_t)(ksc * ksc);
+        if constexpr (PREC) {
+          kf[ks][j] = ksc;
+          kkf[ks][j] = ksc * ksc;
+        } else {
+          kA[ks][j] = (f16_t)ksc;
+          kk[ks][j] = (f16_t)(ksc * ksc);
+        }
 #pragma unroll
         for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
           const int t = 16 * tb + i;
           const float lv = (s <= t) ? fast_exp2(ct[tb] - cs[j]) : 0.f;
-          Lr[lidx(tb, ks)][j] = (f16_t)lv;
+          if constexpr (PREC) {
+            const bf16_t hi = (bf16_t)lv;
+            Lh[lidx(tb, ks)][j] = hi;
+            Ll[lidx(tb, ks)][j] = (bf16_t)(lv - (float)hi);
+          } else {
+            Lr[lidx(tb, ks)][j] = (f16_t)lv;
+          }
         }
       }
     }
@@ -467,22 +513,42 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
 #pragma unroll
       for (int r = 0; r < 4; ++r) M0[r] = mu0[r] * I0[r];
       f16x8 XM[2], XJ[2];
+      bf16x8 XMh[PREC ? 2 : 1], XMl[PREC ? 2 : 1], XJh[PREC ? 2 : 1], XJl[PREC ? 2 : 1];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        // 8 consecutive tokens of the row: one 16-byte LDS read each; packed f16 products are the operands
-        XM[ks] = kA[ks] * *(const f16x8*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
-        XJ[ks] = kk[ks] * *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+        if constexpr (PREC) {
+          float xv[8], xb[8];
+          staged8((const float*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks], xv);
+          staged8((const float*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks], xb);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { xv[j] *= kf[ks][j]; xb[j] *= kkf[ks][j]; }
+          split_bf16(xv, XMh[ks], XMl[ks]);
+          split_bf16(xb, XJh[ks], XJl[ks]);
+        } else {
+          // 8 consecutive tokens of the row: one 16-byte LDS read each; packed f16 products are the operands
+          XM[ks] = kA[ks] * *(const f16x8*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+          XJ[ks] = kk[ks] * *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+        }
       }
       float p[4], pv[4];
 #pragma unroll
       for (int tb = 0; tb < 4; ++tb) {
         f32x4 accM = {0.f, 0.f, 0.f, 0.f};
         f32x4 accI = {Gi[tb], Gi[tb], Gi[tb], Gi[tb]};
+        if constexpr (PREC) {
+          accM = mfma16_split(XMh[0], XMl[0], Lh[lidx(tb, 0)], Ll[lidx(tb, 0)], accM);
+          accI = mfma16_split(XJh[0], XJl[0], Lh[lidx(tb, 0)], Ll[lidx(tb, 0)], accI);
+          if (tb >= 2) {
+            accM = mfma16_split(XMh[1], XMl[1], Lh[lidx(tb, 1)], Ll[lidx(tb, 1)], accM);
+            accI = mfma16_split(XJh[1], XJl[1], Lh[lidx(tb, 1)], Ll[lidx(tb, 1)], accI);
+          }
+        } else {
         accM = mfma16h(XM[0], Lr[lidx(tb, 0)], accM);
         accI = mfma16h(XJ[0], Lr[lidx(tb, 0)], accI);
         if (tb >= 2) {
           accM = mfma16h(XM[1], Lr[lidx(tb, 1)], accM);
           accI = mfma16h(XJ[1], Lr[lidx(tb, 1)], accI);
+        }
         }
         float acc = 0.f, accv = 0.f;
 #pragma unroll
@@ -528,29 +594,38 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   }
 }
 
-template <typename TIn, int NB>
-static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
+template <typename TIn, int NB, bool PREC>
+static int launch_out_nb_p(const ChunkArgs& a, hipStream_t s) {
   const bool var = a.flags & PAL_FLAG_HAS_VAR;
-  const size_t lds = sizeof(float) * (kC + (var ? 2 : 1) * NB * kDG * kC) + 4 * sizeof(f16_t) * kDG * kVH;
+  const size_t lds = sizeof(float) * (kC + (var ? 2 : 1) * NB * kDG * kC) + 4 * (PREC ? sizeof(float) : sizeof(f16_t)) * kDG * kVH;
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;
   // waves per column block, see chunk_out_kernel (7 blocks x 2 would need 128 VGPRs per wave and spills; with 1-3
   // blocks several workgroups share a compute unit and the repeated per-wave set-up costs more than the balance gains)
-  constexpr int RS = (NB == 5 || NB == 6) ? 2 : 1;
+  constexpr int RS = (!PREC && (NB == 5 || NB == 6)) ? 2 : 1;
   // (tile, head) pairs per workgroup, see chunk_out_kernel (measured: +9 % at two column blocks, nothing at one or three)
-  constexpr int TS = NB == 2 ? 2 : 1;
+  constexpr int TS = (!PREC && NB == 2) ? 2 : 1;
   const size_t lds_all = lds * TS;
   const unsigned grid = (unsigned)((blocks + TS - 1) / TS);
   if (var) {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true, RS, TS>, lds_all)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true, RS, TS>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, true, RS, TS, PREC>, lds_all)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, true, RS, TS, PREC>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
   } else {
-    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false, RS, TS>, lds_all)) return rc;
-    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false, RS, TS>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
+    if (int rc = allow_lds((const void*)&chunk_out_kernel<TIn, NB, false, RS, TS, PREC>, lds_all)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_kernel<TIn, NB, false, RS, TS, PREC>), dim3(grid), dim3(NB * RS * TS * 64), lds_all, s, a);
   }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
+}
+
+// fp32 rows take the fp32-accurate variant unless PAL_FLAG_FP32_FAST asks for single bf16/f16 operands
+template <typename TIn, int NB>
+static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
+  if constexpr (sizeof(TIn) == 4) {
+    if (!(a.flags & PAL_FLAG_FP32_FAST)) return launch_out_nb_p<TIn, NB, true>(a, s);
+  }
+  return launch_out_nb_p<TIn, NB, false>(a, s);
 }
 
 template <typename TIn>
@@ -605,25 +680,37 @@ int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tile
                       hipStream_t s);
 
 // Local contribution of every tile to the state, into chunk_mu (and chunk_I when has_j).
-template <typename TIn, bool HAS_J, typename TS>
+template <typename TIn, bool HAS_J, typename TS, bool PREC>
 static int launch_tile_delta_t(const ChunkArgs& a, hipStream_t s) {
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
-  const size_t lds = sizeof(float) * kC + sizeof(TS) * (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<TS>::value;
+  // value rows per workgroup: all of them, or the largest multiple of 16 whose staging tiles fit the LDS
+  int pieces = 1, dvn = a.dv;
+  size_t lds = 0;
+  for (;; ++pieces) {
+    dvn = ((a.dv / 16 + pieces - 1) / pieces) * 16;
+    lds = sizeof(float) * kC + sizeof(TS) * (size_t)(a.dk + (HAS_J ? 2 : 1) * dvn) * StageStride<TS>::value;
+    if (lds <= kMaxLds || dvn == 16) break;
+  }
   if (lds > kMaxLds) return PAL_E_HEADDIM;
-  if (int rc = allow_lds((const void*)&chunk_delta_kernel<TIn, HAS_J, TS>, lds)) return rc;
-  PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<TIn, HAS_J, TS>), dim3((unsigned)blocks), dim3(256), lds, s, a);
+  pieces = (a.dv + dvn - 1) / dvn;
+  if (int rc = allow_lds((const void*)&chunk_delta_kernel<TIn, HAS_J, TS, PREC>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kKernChunkState, s, (chunk_delta_kernel<TIn, HAS_J, TS, PREC>), dim3((unsigned)blocks, (unsigned)pieces),
+                   dim3(256), lds, s, a, dvn);
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
 
+// fp32 rows take the fp32-accurate variant (fp32 staging, operands split into two bf16 halves) unless
+// PAL_FLAG_FP32_FAST asks for single bf16 operands.
 template <typename TIn, bool HAS_J>
 static int launch_tile_delta_j(const ChunkArgs& a, hipStream_t s) {
   if constexpr (sizeof(TIn) == 4) {
+    if (!(a.flags & PAL_FLAG_FP32_FAST)) return launch_tile_delta_t<TIn, HAS_J, float, true>(a, s);
     const size_t lds_f32 = sizeof(float) * (kC + (size_t)(a.dk + (HAS_J ? 2 : 1) * a.dv) * StageStride<float>::value);
-    if (lds_f32 <= kMaxLds) return launch_tile_delta_t<TIn, HAS_J, float>(a, s);
+    if (lds_f32 <= kMaxLds) return launch_tile_delta_t<TIn, HAS_J, float, false>(a, s);
   }
-  return launch_tile_delta_t<TIn, HAS_J, bf16_t>(a, s);
+  return launch_tile_delta_t<TIn, HAS_J, bf16_t, false>(a, s);
 }
 
 int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s) {

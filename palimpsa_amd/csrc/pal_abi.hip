@@ -15,7 +15,9 @@ const char* pal_strerror(int code) {
     case PAL_E_HEADDIM:
       return "dk and dv must be multiples of 16 in [16, 256] (dk one of 16,32,48,64,96,128,192,256 for the recurrent "
              "Palimpsa path; the chunked Palimpsa backward also keeps a dk x dv carry tile in LDS: "
-             "4 dk (dv + 8) + 256 (max(dk, dv) + 4) + 32 dv + 288 <= 163840 bytes, e.g. up to 128x192, 192x128, 256x64)";
+             "4 dk (dv + 8) + 256 (max(dk, dv) + 4) + 32 dv + 288 <= 163840 bytes, e.g. up to 128x192, 192x128, 256x64; "
+             "fp32 rows without PAL_FLAG_FP32_FAST: 8 dk (dv + 8) in that sum and head dims up to 128, "
+             "e.g. 96x96, 64x128, 128x64)";
     case PAL_E_DTYPE: return "unsupported element type";
     case PAL_E_VARLEN_BATCH: return "cu_seqlens needs batch size 1";
     case PAL_E_CU_SEQLENS: return "cu_seqlens must start at 0, be non-decreasing and end at the token count";

@@ -195,6 +195,22 @@ __device__ __forceinline__ f32x4 mfma16h(f16x8 a, f16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+// Operands of the fp32-accurate variants of the chunked kernels: a value is carried as the sum of two bf16 numbers
+// (16 mantissa bits together) and a product of two such operands as three matrix instructions (the lo x lo term,
+// 2^-18 of the result, is dropped); accumulation is fp32 as always.
+__device__ __forceinline__ void split_bf16(const float* x, bf16x8& hi, bf16x8& lo) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    hi[j] = (bf16_t)x[j];
+    lo[j] = (bf16_t)(x[j] - (float)hi[j]);
+  }
+}
+__device__ __forceinline__ f32x4 mfma16_split(bf16x8 ah, bf16x8 al, bf16x8 bh, bf16x8 bl, f32x4 c) {
+  c = mfma16(al, bh, c);
+  c = mfma16(ah, bl, c);
+  return mfma16(ah, bh, c);
+}
+
 __device__ __forceinline__ bf16x2 pack2(float lo, float hi) {
   f32x2 x = {lo, hi};
   return __builtin_convertvector(x, bf16x2);

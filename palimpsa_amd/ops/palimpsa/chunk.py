@@ -145,7 +145,7 @@ class ChunkPalimpsa(torch.autograd.Function):
         ctx.save_for_backward(p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens,
                               table, offsets, int_mu, int_I)
         ctx.meta = dict(dk=p.dk, dv=p.dv, dk_p=p.dk_p, dv_p=p.dv_p, n_seqs=p.n_seqs, compute_dtype=p.compute_dtype,
-                        scale=float(scale), flags=flags & ~L.PAL_FLAG_STORE_FINAL, total_chunks=total_chunks,
+                        scale=float(scale), flags=(flags | L.state_pass_flags()) & ~L.PAL_FLAG_STORE_FINAL, total_chunks=total_chunks,
                         in_dtypes=(q.dtype, k.dtype, v.dtype, b.dtype, gt.dtype, g.dtype, Ip.dtype),
                         g_shape=tuple(g.shape), Ip_shape=tuple(Ip.shape), has_init=p.init_mu is not None,
                         output_uncertainty=bool(output_uncertainty))
@@ -246,7 +246,9 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
         isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state))
     if needs_grad:
         # refuse here what the backward could not serve, instead of at .backward() time
-        L.check(L.load().pal_chunk_bwd_supported(dk_p, dv_p), "chunk_palimpsa (backward head dims)")
+        rows_bf16 = all(x.dtype == torch.bfloat16 for x in (q, k, v, b))
+        L.check(L.load().pal_chunk_bwd_supported(dk_p, dv_p, L.PAL_DTYPE_BF16 if rows_bf16 else L.PAL_DTYPE_F32,
+                                                 L.state_pass_flags()), "chunk_palimpsa (backward head dims)")
     if not needs_grad and cu_seqlens is None and q.shape[0] == 1 and total_chunks > _window_tiles(H, dv_p, dk_p):
         int_mu = int_I = None
     else:

@@ -13,10 +13,10 @@ BF16_OUT_ABS_TOL = 2e-2
 # ("normalised" = by the largest reference entry; the reference script's own
 #  normalisation max|d|/mean|ref| (check_palimpsa.py:28-32) is printed next to it)
 BF16_GRAD_NORM_TOL = 5e-2
-# fp32 rows through the chunked kernels: outputs and states max|x - ref| / max(1, max|ref|), gradients
-# max|dx - dref| / max|dref|
-CHUNK_FP32_OUT_TOL = 2e-2
-CHUNK_FP32_GRAD_TOL = 5e-2
+# fp32 rows through the chunked kernels (operands split into two bf16 halves): the fp32 bar, outputs and states
+# max|x - ref| / max(1, max|ref|), gradients max|dx - dref| / max|dref|
+CHUNK_FP32_OUT_TOL = 1e-4
+CHUNK_FP32_GRAD_TOL = 1e-4
 
 
 def max_rel(x: torch.Tensor, ref: torch.Tensor) -> float:

@@ -172,6 +172,52 @@ def test_squared_error_loss_all_gradients_max_norm(gpu_device):
     _compare(grads, ref, NAMES)
 
 
+@pytest.mark.parametrize("dk,dv", [(16, 32), (64, 64), (48, 96), (96, 96), (128, 64), (64, 128), (80, 48), (31, 65)])
+def test_fp32_backward_meets_the_fp32_bar(gpu_device, dk, dv):
+    """fp32 rows: every gradient (initial state and uncertainty included) within 1e-4 (max-norm) of autograd through
+    the float64 oracle; packed documents in the same call for the first shapes."""
+    B, T, H = 2, 200, 2
+    cu = [0, 70, 71, 300, 400] if dk <= 64 else None
+    if cu is not None:
+        B, T = 1, cu[-1]
+    N = B if cu is None else len(cu) - 1
+    inp = po.make_inputs(B, T, H, dk, dv, seed=3 * dk + dv, normalize_qk=(dk != 31))
+    inp["g"] = torch.tensor([0.6, 7.0])
+    inp["Ip"] = torch.tensor([0.5, 1.6])
+    gen = torch.Generator().manual_seed(6)
+    mu0 = torch.randn(N, H, dv, dk, generator=gen) * 0.1
+    I0 = inp["Ip"].view(1, H, 1, 1) + torch.nn.functional.softplus(torch.randn(N, H, dv, dk, generator=gen))
+    target = 0.3 * torch.randn(B, T, H, dv, generator=gen)
+    o_ref, _, _, _ = hp.oracle_forward(inp, mu0=mu0, I0=I0, cu=cu, scale=0.5, dtype=torch.float64)
+    do = (o_ref - target).float()        # squared-error loss: dO correlated with the state, dg and dIp well conditioned
+    dovar = torch.randn(B, T, H, dv, generator=gen) * 0.3
+    ref = hp.oracle_grads(inp, do, dovar, scale=0.5, mu0=mu0, I0=I0, cu=cu)
+    grads = _run_bwd(inp, gpu_device, do, dovar, mu0=mu0, I0=I0, cu=cu, scale=0.5)
+    assert grads["q"].dtype == torch.float32
+    _compare(grads, ref, NAMES + ["mu0", "I0"], tol=hp.CHUNK_FP32_GRAD_TOL)
+
+
+def test_fp32_backward_head_dim_envelope(gpu_device):
+    """The split operands of the fp32 path need twice the LDS: head dims above 128 (and pairs like 128 x 128) are
+    refused by the forward call when a gradient is wanted; the single-operand mode still serves them."""
+    from palimpsa_amd import _lib
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    inp = po.make_inputs(1, 100, 1, 128, 128, seed=6)
+    names = ("q", "k", "v", "b", "gt", "g", "Ip")
+    leaves = {n: inp[n].to(gpu_device).clone().requires_grad_(True) for n in names}
+    with pytest.raises(ValueError, match="head dims"):
+        chunk_palimpsa(*[leaves[n] for n in names])
+    try:
+        _lib.set_fp32_fast(True)
+        o = chunk_palimpsa(*[leaves[n] for n in names])
+        o.sum().backward()
+    finally:
+        _lib.set_fp32_fast(False)
+    ref = hp.oracle_grads(inp, torch.ones_like(inp["v"]))
+    for n in names:
+        assert hp.max_rel(leaves[n].grad, ref[n]) <= hp.BF16_GRAD_NORM_TOL, n
+
+
 def _squared_error_case(inp, dev, cu=None, seed=50):
     """Gradients of 0.5*sum((o - target)^2) through the kernel and through the float64 oracle (same dO for both)."""
     gen = torch.Generator().manual_seed(seed)
