@@ -8,7 +8,7 @@
  *
  * Conventions
  *   - every buffer is owned by the caller, device-resident, densely packed:
- *       q,k [B,T,H,dk]  v,b,o,o_var [B,T,H,dv]  gt [B,T,H]  g,Ip [H]
+ *       q,k [B,T,H,dk] (or [B,T,Hq,dk], see PalDims.n_qk_heads)  v,b,o,o_var [B,T,H,dv]  gt [B,T,H]  g,Ip [H]
  *       states [N,H,dv,dk] fp32 in (mu, I) form
  *     (layouts enforced by the reference through .contiguous():
  *      chunk_palimpsa_forgetting_scalar.py:14-20, and raw pointer arithmetic:
@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PAL_ABI_VERSION 2
+#define PAL_ABI_VERSION 3
 
 /* element types of tensors handed over the boundary */
 #define PAL_DTYPE_F32 0
@@ -89,6 +89,11 @@ typedef struct PalDims {
   int32_t var_dtype;    /* PAL_DTYPE_* of o_var / do_var                      */
   uint32_t flags;       /* PAL_FLAG_*                                         */
   float scale;          /* output scale (reference default dk^-0.5)           */
+  int32_t n_qk_heads;   /* heads of q, k, dq, dk: 0 or H = one per value head (the reference's layout); a divisor
+                           Hq of H = q,k [B,T,Hq,dk], value head h reads q/k head h / (H / Hq) (what the layers
+                           obtain by repeating heads, palimpsa/layers/meta_mamba2.py:281-282, palimpsa.py:266-267,
+                           without materialising the repeat); dq, dk [B,T,Hq,dk] are summed over each group.
+                           Palimpsa entry points only; the pal_gla_* entry points want 0 or H.                  */
 } PalDims;
 
 /* Forward-side tensors.  Unused optional pointers are NULL. */

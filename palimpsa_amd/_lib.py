@@ -12,7 +12,7 @@ from typing import Optional
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libpalimpsa_hip.so")
 
-PAL_ABI_VERSION = 2
+PAL_ABI_VERSION = 3
 PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
 PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS, PAL_FLAG_FP32_FAST = 256, 512, 1024
@@ -32,7 +32,7 @@ class PalDims(C.Structure):
         ("batch", C.c_int32), ("seq_len", C.c_int32), ("n_seqs", C.c_int32), ("n_heads", C.c_int32),
         ("dk", C.c_int32), ("dv", C.c_int32), ("total_chunks", C.c_int32),
         ("dtype", C.c_int32), ("gate_dtype", C.c_int32), ("var_dtype", C.c_int32),
-        ("flags", C.c_uint32), ("scale", C.c_float),
+        ("flags", C.c_uint32), ("scale", C.c_float), ("n_qk_heads", C.c_int32),
     ]
 
 

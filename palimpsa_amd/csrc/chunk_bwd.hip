@@ -155,7 +155,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * st_q + e) * kVS2 + st_s] = st[x][e];
   };
-  const int64_t rs = (int64_t)H * dk;   // token stride of q, k
+  const int64_t rs = qk_stride(a);      // token stride of q, k
+  const int64_t rso = (int64_t)H * dk;  // token stride of dq, dk (one row per value head)
   const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
   const int n_groups = dv / kDG2;
   int pass = 0, nb = nbl, n_act = NB;   // set per pass: global column block of this wave, active blocks
@@ -204,8 +205,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     float dq[8];
     float sigacc = 0.f;
     {
-      const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb;
-      const TIn* qp = (const TIn*)a.q + ((int64_t)t0 * H + h) * dk + 16 * nb;
+      const TIn* kp = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
+      const TIn* qp = (const TIn*)a.q + qk_row(a, t0, h) + 16 * nb;
       float ct[2];
 #pragma unroll
       for (int tl = 0; tl < 2; ++tl) ct[tl] = sC[16 * (2 * HF + tl) + i];
@@ -372,7 +373,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int t = 16 * (2 * HF + tl) + 4 * g + r;
-        if (t < clen) (dqp + (int64_t)t * rs)[i] = from_f32<TIn>(dq[tl * 4 + r]);
+        if (t < clen) (dqp + (int64_t)t * rso)[i] = from_f32<TIn>(dq[tl * 4 + r]);
       }
     const float x = wave_sum(sigacc);
     if (lane == 0) sRed[NB * kC + HF * NB + nbl] = x;
@@ -387,7 +388,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     float dkM[8], dkJ[8];
     float gate[2], Fs[2];
     {
-      const TIn* kp4 = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb;
+      const TIn* kp4 = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
       float ct[2];
 #pragma unroll
       for (int sl = 0; sl < 2; ++sl) ct[sl] = sC[16 * (2 * HF + sl) + i];
@@ -542,7 +543,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
       if (s < clen) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          (dkp + (int64_t)s * rs)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
+          (dkp + (int64_t)s * rso)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
       }
       const float x = rows4_sum(gate[sl]);
       if (g == 0) sRed[nbl * kC + 16 * (2 * HF + sl) + i] = x;
@@ -801,13 +802,13 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
         }
       }
     }
-    const TIn* kin = (const TIn*)a.k + tok0 * dk;
+    const TIn* kin = (const TIn*)a.k + qk_row(a, t0, h);
     // k of the result entries (row s = 16w + 4g + r, column n = 16nbk + i), fetched one step ahead
     auto load_k4 = [&](int nbk, float* kv) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int s = 16 * w + 4 * g + r;
-        kv[r] = (s < clen) ? to_f32(kin[(int64_t)s * H * dk + 16 * nbk + i]) : 0.f;
+        kv[r] = (s < clen) ? to_f32(kin[(int64_t)s * qk_stride(a) + 16 * nbk + i]) : 0.f;
       }
     };
     float kcur[4], knext[4] = {0.f, 0.f, 0.f, 0.f};
@@ -874,7 +875,7 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
     const int KS = (dk + 31) / 32;
     bf16x8 A1[KSMAX], A2[KSMAX];
     bf16x8 A1l[PREC ? KSMAX : 1], A2l[PREC ? KSMAX : 1];
-    const TIn* kp = (const TIn*)a.k + tokA * dk;
+    const TIn* kp = (const TIn*)a.k + qk_row(a, t0 + (row_ok ? srow : 0), h);
 #pragma unroll
     for (int ks = 0; ks < KSMAX; ++ks) {
       if (ks < KS) {
@@ -1040,8 +1041,33 @@ __global__ __launch_bounds__(64) void chunk_bwd_head_reduce_kernel(BwdArgs A) {
 }
 
 struct BwdLayout {
-  size_t oDM, oDJ, oFtot, oSig, oE, oInit, oDgTile, total;
+  size_t oDM, oDJ, oFtot, oSig, oE, oInit, oDgTile, oDqFull, oDkFull, total;
 };
+
+// dq, dk of a q/k head shared by `rep` value heads: the kernels leave one row per value head ([tokens, H, dk]) in the
+// workspace, this adds the rows of a group in a fixed order (fp32) into the caller's [tokens, Hq, dk].
+template <typename T>
+__global__ __launch_bounds__(256) void group_sum_kernel(const T* src_q, const T* src_k, T* dst_q, T* dst_k, int64_t n4,
+                                                        int Hq, int rep, int dk) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // four consecutive columns of one (token, q/k head) row
+  if (idx >= n4) return;
+  const int per = dk >> 2;
+  const int c4 = (int)(idx % per);
+  const int64_t row = idx / per;                                 // token * Hq + hq
+  const int64_t tok = row / Hq;
+  const int hq = (int)(row - tok * Hq);
+  float aq[4] = {0.f, 0.f, 0.f, 0.f}, ak[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < rep; ++r) {
+    const int64_t so = ((tok * Hq + hq) * rep + r) * (int64_t)dk + 4 * c4;   // value head hq * rep + r
+    float x[4], y[4];
+    load_vec<4>(src_q + so, x);
+    load_vec<4>(src_k + so, y);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { aq[e] += x[e]; ak[e] += y[e]; }
+  }
+  store_vec<4>(dst_q + row * dk + 4 * c4, aq);
+  store_vec<4>(dst_k + row * dk + 4 * c4, ak);
+}
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -1058,6 +1084,12 @@ static BwdLayout bwd_layout(const PalDims* d) {
   L.oE = o; o = align256(o + tokens * d->n_heads * 4);
   L.oInit = o; o = align256(o + (size_t)d->n_seqs * d->n_heads * (E / 256) * 4);
   L.oDgTile = o; o = align256(o + tiles * 4);
+  L.oDqFull = L.oDkFull = o;
+  if (d->n_qk_heads > 0 && d->n_qk_heads != d->n_heads) {
+    const size_t full = tokens * d->n_heads * d->dk * (d->dtype == PAL_DTYPE_BF16 ? 2 : 4);
+    L.oDqFull = o; o = align256(o + full);
+    L.oDkFull = o; o = align256(o + full);
+  }
   L.total = o;
   return L;
 }
@@ -1207,6 +1239,11 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   A.d_o = gr->d_o;
   A.d_o_var = (dd.flags & PAL_FLAG_HAS_VAR) ? gr->d_o_var : nullptr;
   A.dq = gr->dq; A.dk = gr->dk; A.dv = gr->dv; A.db = gr->db;
+  const bool grouped = A.c.Hq != A.c.H;
+  if (grouped) {   // one row per value head first, summed over each group at the end
+    A.dq = (char*)workspace + L.oDqFull;
+    A.dk = (char*)workspace + L.oDkFull;
+  }
   A.dgt = gr->dgt; A.dg = gr->dg; A.dIp = gr->dIp;
   A.d_init_mu = gr->d_init_mu; A.d_init_I = gr->d_init_I;
   char* ws = (char*)workspace;
@@ -1237,5 +1274,15 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   }
   PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((unsigned)dd.n_heads), dim3(64), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
+  if (grouped) {
+    const int64_t n4 = (int64_t)A.tokens * A.c.Hq * (dd.dk / 4);
+    const unsigned gblocks = (unsigned)((n4 + 255) / 256);
+    const int rep = A.c.H / A.c.Hq;
+    if (bf) hipLaunchKernelGGL(group_sum_kernel<bf16_t>, dim3(gblocks), dim3(256), 0, s, (const bf16_t*)A.dq, (const bf16_t*)A.dk,
+                               (bf16_t*)gr->dq, (bf16_t*)gr->dk, n4, A.c.Hq, rep, dd.dk);
+    else hipLaunchKernelGGL(group_sum_kernel<float>, dim3(gblocks), dim3(256), 0, s, (const float*)A.dq, (const float*)A.dk,
+                            (float*)gr->dq, (float*)gr->dk, n4, A.c.Hq, rep, dd.dk);
+    PAL_HIP_LAUNCH_CHECK();
+  }
   return PAL_OK;
 }

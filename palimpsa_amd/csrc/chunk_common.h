@@ -29,10 +29,17 @@ struct ChunkArgs {
   const int32_t *cu_seqlens, *chunk_table, *chunk_offsets;
   float *chunk_mu, *chunk_I;
   int32_t T, H, dk, dv, n_seqs, total_chunks;
+  int32_t Hq;   // heads of q and k: H, or a divisor of it when a group of H / Hq value heads shares one q/k head
   int32_t gate_bf16, var_bf16;
   uint32_t flags;
   float scale;
 };
+
+// q and k rows of value head h: element offset of token t's row, and the token stride, in a [tokens, Hq, dk] tensor
+__device__ __forceinline__ int64_t qk_row(const ChunkArgs& a, int64_t t, int h) {
+  return (t * a.Hq + h / (a.H / a.Hq)) * a.dk;
+}
+__device__ __forceinline__ int64_t qk_stride(const ChunkArgs& a) { return (int64_t)a.Hq * a.dk; }
 
 // tile c -> (sequence, first token in the packed/batched token axis, tokens in tile, index in sequence)
 __device__ __forceinline__ void chunk_lookup(const ChunkArgs& a, int c, int& seq, int& t0, int& clen, int& cis) {
@@ -84,16 +91,17 @@ __device__ __forceinline__ int block_exponent_of(float m, int target) {
 }
 
 template <typename TIn>
-__device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, const TIn* vt, const TIn* bt, int H, int dk,
-                                                              int dv, int clen, int tid, int nthreads, float* sMax) {
+__device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, const TIn* vt, const TIn* bt, int Hq, int H,
+                                                              int dk, int dv, int clen, int tid, int nthreads,
+                                                              float* sMax) {
   float km = 0.f, vm = 0.f, bm = 0.f;
   const int gk = dk >> 3, gv = dv >> 3;
   for (int idx = tid; idx < kC * gk; idx += nthreads) {
     const int s = idx / gk, c = idx - s * gk;
     if (s < clen) {
       float x[8];
-      load_vec<4>(kt + (int64_t)s * H * dk + 8 * c, x);
-      load_vec<4>(kt + (int64_t)s * H * dk + 8 * c + 4, x + 4);
+      load_vec<4>(kt + (int64_t)s * Hq * dk + 8 * c, x);
+      load_vec<4>(kt + (int64_t)s * Hq * dk + 8 * c + 4, x + 4);
 #pragma unroll
       for (int e = 0; e < 8; ++e) km = fmaxf(km, fabsf(x[e]));
     }

@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void chunk_delta_kernel(ChunkArgs a, int dvn) 
     const float cs = wave_inclusive_scan(-gt * gh, lane);
     sA[lane] = fast_exp2((a.flags & kFlagDecayFromStart) ? cs : __shfl(cs, 63) - cs);
   }
-  stage_transposed((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, (int64_t)H * dk, dk, clen, sKT, tid);
+  stage_transposed((const TIn*)a.k + qk_row(a, t0, h), qk_stride(a), dk, clen, sKT, tid);
   stage_transposed((const TIn*)a.v + ((int64_t)t0 * H + h) * dv + d0, (int64_t)H * dv, dn, clen, sVT, tid);
   if (HAS_J) stage_transposed((const TIn*)a.b + ((int64_t)t0 * H + h) * dv + d0, (int64_t)H * dv, dn, clen, sBT, tid);
   __syncthreads();
@@ -386,25 +386,25 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   // the wave's k column and q rows are requested first so that their latency overlaps the block-exponent pass
   float kraw[2][8];
   {
-    const TIn* kp = (const TIn*)a.k + ((int64_t)t0 * H + h) * dk + 16 * nb + i;
+    const TIn* kp = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb + i;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int s = 8 * g + j + 32 * ks;
         const bool ok = s < clen;
-        const float kv = to_f32(kp[(int64_t)(ok ? s : 0) * H * dk]);
+        const float kv = to_f32(kp[(int64_t)(ok ? s : 0) * qk_stride(a)]);
         kraw[ks][j] = ok ? kv : 0.f;
       }
   }
   float qD[4][4];
   {
-    const TIn* qp = (const TIn*)a.q + ((int64_t)t0 * H + h) * dk + 16 * nb + 4 * g;
+    const TIn* qp = (const TIn*)a.q + qk_row(a, t0, h) + 16 * nb + 4 * g;
 #pragma unroll
     for (int tb = 0; tb < 4; ++tb) {
       const int t = 16 * tb + i;
       if (t < clen) {
-        load_vec<4>(qp + (int64_t)t * H * dk, qD[tb]);
+        load_vec<4>(qp + (int64_t)t * qk_stride(a), qD[tb]);
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) qD[tb][r] = 0.f;
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   // block exponents of the f16 operands (see tile_block_exponents); sO doubles as its scratch
   TileExponents bexp = {0, 0, 0};
   if constexpr (!PREC)
-    bexp = tile_block_exponents((const TIn*)a.k + ((int64_t)t0 * H + h) * dk, vp, bp, H, dk, dv, clen, tid, NT, sO);
+    bexp = tile_block_exponents((const TIn*)a.k + qk_row(a, t0, h), vp, bp, a.Hq, H, dk, dv, clen, tid, NT, sO);
   const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
   const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
   const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
@@ -662,6 +662,7 @@ void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t) {
   a.chunk_offsets = (d->flags & PAL_FLAG_VARLEN) ? t->chunk_offsets : nullptr;
   a.chunk_mu = t->chunk_mu; a.chunk_I = t->chunk_I;
   a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv;
+  a.Hq = d->n_qk_heads > 0 ? d->n_qk_heads : d->n_heads;
   a.n_seqs = d->n_seqs; a.total_chunks = d->total_chunks;
   a.gate_bf16 = d->gate_dtype == PAL_DTYPE_BF16;
   a.var_bf16 = d->var_dtype == PAL_DTYPE_BF16;

@@ -96,8 +96,8 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
       kval[j] = idx < 32 * gk;
       ksp[j] = idx / gk;
       const int c8 = idx - ksp[j] * gk;
-      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * H * dk + 8 * c8) * 2) : 0x80000000u;
-      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * H * dk + 8 * c8) * 2) : 0x80000000u;
+      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * a.Hq * dk + 8 * c8) * 2) : 0x80000000u;
+      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * a.Hq * dk + 8 * c8) * 2) : 0x80000000u;
       kdst[j] = (uint32_t)(8 * c8 * (kStTS / 2) + ksp[j]);
     }
     const int vtid = st, btid = (st + 256 - 32 * gv) & 255;
@@ -115,10 +115,10 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
     // (the tail of its last tile, tiles past its end) are out of range and read as zero, so no fetch needs a
     // branch or a select.  Nothing touches a fetched value before it goes to LDS: any use here would make the
     // wave wait for everything it has in flight, which is what fetching ahead is meant to avoid.
-    const bf16_t* kbase = (const bf16_t*)a.k + ((int64_t)bos * H + h) * dk;
+    const bf16_t* kbase = (const bf16_t*)a.k + qk_row(a, bos, h);
     const bf16_t* vbase = (const bf16_t*)a.v + ((int64_t)bos * H + h) * dv + d0;
     const int esz = a.gate_bf16 ? 2 : 4;
-    const uint32_t kbytes = len > 0 ? (uint32_t)(((len - 1) * H * dk + dk) * 2) : 0u;
+    const uint32_t kbytes = len > 0 ? (uint32_t)(((len - 1) * a.Hq * dk + dk) * 2) : 0u;
     const uint32_t vbytes = len > 0 ? (uint32_t)(((len - 1) * H * dv + ds) * 2) : 0u;
     const uint32_t gbytes = len > 0 ? (uint32_t)(((len - 1) * H + 1) * esz) : 0u;
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, kbytes, 0x00020000);
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
       const int c = A.reverse ? nchunks - 1 - p : p;
       const bool live = p < nchunks;
       // a tile past the end: every offset out of range
-      const uint32_t tk = live ? (uint32_t)(c * kC * H * dk * 2) : 0x80000000u;
+      const uint32_t tk = live ? (uint32_t)(c * kC * a.Hq * dk * 2) : 0x80000000u;
       const uint32_t tv = live ? (uint32_t)(c * kC * H * dv * 2) : 0x80000000u;
 #pragma unroll
       for (int j = 0; j < NIK; ++j) {
@@ -391,6 +391,7 @@ extern "C" int pal_state_pass_applies(const PalDims* d, int has_precision_state)
   if (pal_validate_dims(d) != PAL_OK) return 0;
   pal::ChunkArgs a = {};
   a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv; a.n_seqs = d->n_seqs;
+  a.Hq = d->n_qk_heads > 0 ? d->n_qk_heads : d->n_heads;
   a.flags = d->flags;
   return pal::state_pass_applies(a, d->dtype, has_precision_state != 0) ? 1 : 0;
 }

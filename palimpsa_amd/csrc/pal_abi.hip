@@ -52,6 +52,7 @@ int pal_validate_dims(const PalDims* d) {
     if (d->n_seqs != d->batch) return PAL_E_DIM;
   }
   if (!(d->scale == d->scale)) return PAL_E_DIM;  // NaN
+  if (d->n_qk_heads < 0 || (d->n_qk_heads > 0 && d->n_heads % d->n_qk_heads != 0)) return PAL_E_DIM;
   return PAL_OK;
 }
 

@@ -40,6 +40,7 @@ struct RecBwdArgs {
   double *dgPart, *dIpPart;  // [N, H]
   int32_t T, H, dk, dv, n_seqs, S, tokens, ND;
   int32_t seg_cap;       // segments the checkpoint buffers hold
+  int32_t Hq;            // heads of q, k, dq, dk (H, or a divisor of it: a group of H / Hq value heads shares one)
   int32_t gate_bf16, var_bf16, out_bf16;
   uint32_t flags;
   float scale;
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
 #pragma unroll
     for (int e = 0; e < NPL; ++e) { M[e] = 0.f; J[e] = 0.f; }
   }
-  const TIn* kp = (const TIn*)a.k + (bos * H + h) * dk;
+  const TIn* kp = (const TIn*)a.k + (bos * a.Hq + h / (H / a.Hq)) * dk;
   const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv + drow;
   const TIn* bp = (const TIn*)a.b + (bos * H + h) * dv + drow;
   for (int t = 0; t < len; ++t) {
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
     }
     float kc[NPL];
 #pragma unroll
-    for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * H * dk + Map::vec_start(j, iv), kc + iv * VW);
+    for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
     const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
     const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
 #pragma unroll
@@ -148,8 +149,8 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
   const float gh = gval * kLog2e, Ip = a.Ip[h], scale = a.scale;
   const bool has_var = a.flags & PAL_FLAG_HAS_VAR;
   const int drow = tile * 4 + grp;
-  const TIn* qp = (const TIn*)a.q + (bos * H + h) * dk;
-  const TIn* kp = (const TIn*)a.k + (bos * H + h) * dk;
+  const TIn* qp = (const TIn*)a.q + (bos * a.Hq + h / (H / a.Hq)) * dk;
+  const TIn* kp = (const TIn*)a.k + (bos * a.Hq + h / (H / a.Hq)) * dk;
   const int64_t vrow = (bos * H + h) * dv + drow;
   const TIn* vp = (const TIn*)a.v + vrow;
   const TIn* bp = (const TIn*)a.b + vrow;
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
       if (jj + 1 < cnt) {
         float kc[NPL];
 #pragma unroll
-        for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * H * dk + Map::vec_start(j, iv), kc + iv * VW);
+        for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
         const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
         const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
 #pragma unroll
@@ -197,8 +198,8 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
       float kc[NPL], qc[NPL];
 #pragma unroll
       for (int iv = 0; iv < NV; ++iv) {
-        load_vec<VW>(kp + (int64_t)t * H * dk + Map::vec_start(j, iv), kc + iv * VW);
-        load_vec<VW>(qp + (int64_t)t * H * dk + Map::vec_start(j, iv), qc + iv * VW);
+        load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
+        load_vec<VW>(qp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), qc + iv * VW);
       }
       const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
       const float dov = scale * to_f32(dop[(int64_t)t * H * dv]);
@@ -285,15 +286,23 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
 }
 
 // --------------------------------------------------------------------- reduce
-// dq, dk: one thread per (token, head, n); d log f and dgt: one thread per (token, head)
+// dq, dk: one thread per (token, q/k head, n), summing the value-row tiles of every value head of the group in a
+// fixed order; d log f and dgt: one thread per (token, head)
 __global__ __launch_bounds__(256) void recurrent_bwd_reduce_kernel(RecBwdArgs a) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t nqk = (int64_t)a.tokens * a.H * a.dk;
-  if (idx < nqk) {
+  const int64_t nqk = (int64_t)a.tokens * a.H * a.dk;       // entries of one partial buffer (one row per value head)
+  const int64_t nout = (int64_t)a.tokens * a.Hq * a.dk;
+  if (idx < nout) {
+    const int rep = a.H / a.Hq;
+    const int n = (int)(idx % a.dk);
+    const int64_t row = idx / a.dk;                          // token * Hq + hq
     float sq = 0.f, sk = 0.f;
-    for (int w = 0; w < a.ND; ++w) {
-      sq += a.pdq[(int64_t)w * nqk + idx];
-      sk += a.pdk[(int64_t)w * nqk + idx];
+    for (int r = 0; r < rep; ++r) {
+      const int64_t src = (row * rep + r) * a.dk + n;        // value head hq * rep + r of the same token
+      for (int w = 0; w < a.ND; ++w) {
+        sq += a.pdq[(int64_t)w * nqk + src];
+        sk += a.pdk[(int64_t)w * nqk + src];
+      }
     }
     store_rt(a.g_dq, idx, sq, a.out_bf16);
     store_rt(a.g_dk, idx, sk, a.out_bf16);
@@ -446,6 +455,7 @@ extern "C" int pal_recurrent_bwd(const PalDims* d, const PalFwdTensors* t, const
   a.pdIp = (float*)(ws + L.oPdIp); a.pInit = (float*)(ws + L.oPInit);
   a.dgPart = (double*)(ws + L.oDg); a.dIpPart = (double*)(ws + L.oDIp);
   a.T = dd.seq_len; a.H = dd.n_heads; a.dk = dd.dk; a.dv = dd.dv; a.n_seqs = dd.n_seqs;
+  a.Hq = dd.n_qk_heads > 0 ? dd.n_qk_heads : dd.n_heads;
   a.S = L.S; a.tokens = dd.batch * dd.seq_len; a.ND = L.ND;
   a.seg_cap = (int32_t)(L.segments > 0x7fffffff ? 0x7fffffff : L.segments);
   a.gate_bf16 = dd.gate_dtype == PAL_DTYPE_BF16;

@@ -27,6 +27,7 @@ struct RecArgs {
   float *final_mu, *final_I;
   const int32_t* cu_seqlens;
   int32_t T, H, dk, dv, n_seqs;
+  int32_t Hq;   // heads of q and k (H, or a divisor of it: a group of H / Hq value heads shares one)
   int32_t gate_bf16, var_bf16;
   uint32_t flags;
   float scale;
@@ -98,8 +99,9 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
       for (int e = 0; e < NPL; ++e) { M[rr][e] = 0.f; J[rr][e] = 0.f; }
   }
 
-  const TIn* qp = (const TIn*)a.q + (bos * H + h) * dk;
-  const TIn* kp = (const TIn*)a.k + (bos * H + h) * dk;
+  const int Hq = a.Hq, hq = h / (H / Hq);
+  const TIn* qp = (const TIn*)a.q + (bos * Hq + hq) * dk;
+  const TIn* kp = (const TIn*)a.k + (bos * Hq + hq) * dk;
   const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv;
   const TIn* bp = (const TIn*)a.b + (bos * H + h) * dv;
   TIn* op = (TIn*)a.o + (bos * H + h) * dv;
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
 
   float kc[NPL], qc[NPL], vc[RD], bc[RD], gtc;
   auto load_token = [&](int t, float* kk_, float* qq_, float* vv_, float* bb_, float& gt_) {
-    const int64_t off_k = (int64_t)t * H * dk;
+    const int64_t off_k = (int64_t)t * Hq * dk;
     const int64_t off_v = (int64_t)t * H * dv;
 #pragma unroll
     for (int iv = 0; iv < NV; ++iv) {
@@ -226,6 +228,7 @@ extern "C" int pal_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, void*
   a.final_mu = t->final_mu; a.final_I = t->final_I;
   a.cu_seqlens = t->cu_seqlens;
   a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv; a.n_seqs = d->n_seqs;
+  a.Hq = d->n_qk_heads > 0 ? d->n_qk_heads : d->n_heads;
   a.gate_bf16 = d->gate_dtype == PAL_DTYPE_BF16;
   a.var_bf16 = d->var_dtype == PAL_DTYPE_BF16;
   a.flags = d->flags;

@@ -80,12 +80,17 @@ class Prepared:
 
 def prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens, recurrent: bool) -> Prepared:
     dev = _require_gpu(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state)
-    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or b.shape != v.shape or v.shape[:3] != q.shape[:3]:
-        raise ValueError("expected q,k [B,T,H,dk] and v,b [B,T,H,dv]")
-    if tuple(gt.shape) != tuple(q.shape[:3]):
-        raise ValueError(f"gt must be [B,T,H]={tuple(q.shape[:3])}, got {tuple(gt.shape)}")
-    B, T, H, dk = q.shape
-    dv = v.shape[-1]
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or b.shape != v.shape or v.shape[:2] != q.shape[:2]:
+        raise ValueError("expected q,k [B,T,Hq,dk] and v,b [B,T,H,dv] (Hq = H, or a divisor of H)")
+    B, T, H, dv = v.shape
+    Hq, dk = q.shape[2], q.shape[3]
+    # q and k may carry fewer heads than v: a group of H / Hq value heads then shares one q/k head, which is what
+    # the reference layers obtain by repeating heads before the call (layers/meta_mamba2.py:281-282,
+    # layers/palimpsa.py:266-267); the kernels index the shared rows instead
+    if Hq < 1 or H % Hq != 0:
+        raise ValueError(f"the {Hq} heads of q, k must divide the {H} heads of v, b")
+    if tuple(gt.shape) != (B, T, H):
+        raise ValueError(f"gt must be [B,T,H]={(B, T, H)}, got {tuple(gt.shape)}")
     if g.numel() != H or Ip.numel() != H:
         raise ValueError("g and Ip must have one entry per head")
     # one element type for q,k,v,b: bf16 stays bf16, everything else computes from fp32 rows
@@ -173,11 +178,11 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 def make_dims(p: Prepared, scale: float, flags: int, total_chunks: int = 0, var_dtype: torch.dtype = torch.float32) -> L.PalDims:
-    B, T, H, _ = p.q.shape
+    B, T, H, _ = p.v.shape
     return L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=p.dk_p, dv=p.dv_p,
                      total_chunks=total_chunks, dtype=_pal_dtype(p.compute_dtype),
                      gate_dtype=_pal_dtype(p.gt.dtype), var_dtype=_pal_dtype(var_dtype),
-                     flags=flags | L.state_pass_flags(), scale=float(scale))
+                     flags=flags | L.state_pass_flags(), scale=float(scale), n_qk_heads=p.q.shape[2])
 
 
 def make_fwd_tensors(p: Prepared, o, o_var, final_mu, final_I, chunk_table=None, chunk_offsets=None,

@@ -47,7 +47,7 @@ def _windowed_forward(p, scale, output_uncertainty, o, o_var, final_mu, final_I,
     state of the one before.  Same kernels and same tiles as the single call; the state crosses a
     segment boundary as (mu, I), which costs one fp32 rounding per boundary."""
     dev = p.q.device
-    _, T, H, _ = p.q.shape
+    _, T, H, _ = p.v.shape
     seg = window * L.PAL_CHUNK
     int_mu = torch.empty(window, H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
     int_I = torch.empty_like(int_mu)
@@ -71,7 +71,8 @@ def _windowed_forward(p, scale, output_uncertainty, o, o_var, final_mu, final_I,
             n_tiles = (e - s + L.PAL_CHUNK - 1) // L.PAL_CHUNK
             dims = L.PalDims(batch=1, seq_len=e - s, n_seqs=1, n_heads=H, dk=p.dk_p, dv=p.dv_p, total_chunks=n_tiles,
                              dtype=cm._pal_dtype(p.compute_dtype), gate_dtype=cm._pal_dtype(p.gt.dtype),
-                             var_dtype=cm._pal_dtype(p.compute_dtype), flags=flags, scale=float(scale))
+                             var_dtype=cm._pal_dtype(p.compute_dtype), flags=flags, scale=float(scale),
+                             n_qk_heads=p.q.shape[2])
             tens = L.PalFwdTensors(
                 q=pt(p.q[:, s:e]), k=pt(p.k[:, s:e]), v=pt(p.v[:, s:e]), b=pt(p.b[:, s:e]), gt=pt(p.gt[:, s:e]),
                 g=pt(p.g), Ip=pt(p.Ip), o=pt(o[:, s:e]), o_var=pt(o_var[:, s:e] if o_var is not None else None),
@@ -92,7 +93,7 @@ class ChunkPalimpsa(torch.autograd.Function):
         p = cm.prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens,
                               recurrent=False)
         dev = p.q.device
-        B, T, H, _ = p.q.shape
+        B, T, H, _ = p.v.shape
         table = offsets = None
         if p.cu_seqlens is not None:
             if chunk_offsets is None:
@@ -159,8 +160,8 @@ class ChunkPalimpsa(torch.autograd.Function):
         (q, k, v, b, gt, g, Ip, init_mu, init_I, cu, table, offsets, int_mu, int_I) = ctx.saved_tensors
         m = ctx.meta
         dev = q.device
-        B, T, H, dk_p = q.shape
-        dv_p = v.shape[-1]
+        B, T, H, dv_p = v.shape
+        dk_p = q.shape[-1]
         cd = m["compute_dtype"]
         has_var = m["output_uncertainty"] and do_var is not None
         if do is None:   # only o_var (or nothing) was used downstream
@@ -192,7 +193,7 @@ class ChunkPalimpsa(torch.autograd.Function):
             flags &= ~L.PAL_FLAG_HAS_VAR
         dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p,
                          total_chunks=m["total_chunks"], dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype),
-                         var_dtype=cm._pal_dtype(cd), flags=flags, scale=m["scale"])
+                         var_dtype=cm._pal_dtype(cd), flags=flags, scale=m["scale"], n_qk_heads=q.shape[2])
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
                                o_var=None, init_mu=pt(init_mu), init_I=pt(init_I), final_mu=None, final_I=None,
@@ -238,7 +239,7 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
         chunk_offsets, total_chunks = cm.chunk_meta(cu_seqlens, q.shape[1], q.device)
     else:
         total_chunks = _count_chunks(q.shape[1], q.shape[0])
-    H = q.shape[-2]
+    H = v.shape[-2]
     dk_p, dv_p = cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1])
     # chunk-start states, allocated outside the autograd Function as in the reference (chunk...py:652-653);
     # a long single sequence that no backward will follow is run in windows instead (see _windowed_forward)

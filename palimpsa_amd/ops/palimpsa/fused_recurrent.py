@@ -23,7 +23,7 @@ def _recurrent_forward(q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I
                        output_final_state, output_uncertainty, cu_seqlens):
     p = cm.prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_seqlens, recurrent=True)
     dev = p.q.device
-    B, T, H, _ = p.q.shape
+    B, T, H, _ = p.v.shape
     o = torch.empty(B, T, H, p.dv_p, dtype=p.compute_dtype, device=dev)
     # the reference leaves o_var in fp32 (fused...py:184-186 after the casts of :226-232)
     o_var = torch.empty(B, T, H, p.dv_p, dtype=torch.float32, device=dev) if output_uncertainty else None
@@ -73,8 +73,8 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
         q, k, v, b, gt, g, Ip, init_mu, init_I, cu = ctx.saved_tensors
         m = ctx.meta
         dev = q.device
-        B, T, H, dk_p = q.shape
-        dv_p = v.shape[-1]
+        B, T, H, dv_p = v.shape
+        dk_p = q.shape[-1]
         cd = m["compute_dtype"]
         has_var = m["output_uncertainty"] and do_var is not None
         if do is None:
@@ -103,7 +103,7 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
             flags |= L.PAL_FLAG_HAS_VAR
         dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
                          dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
-                         flags=flags, scale=m["scale"])
+                         flags=flags, scale=m["scale"], n_qk_heads=q.shape[2])
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
                                init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))

@@ -207,6 +207,57 @@ def test_meta_mamba2_call_shape_forward_backward(gpu_device, dk, dv):
     assert not bad, bad
 
 
+@pytest.mark.parametrize("path", ["chunk_bf16", "chunk_fp32", "recurrent_fp32"])
+def test_shared_qk_heads_are_indexed_not_repeated(gpu_device, path):
+    """q = C and k = B of MetaMamba2 belong to n_groups < H groups and the layer repeats them over the heads of a
+    group before the call (meta_mamba2.py:281-282; Palimpsa.forward does the same with num_heads < num_v_heads,
+    palimpsa.py:266-267).  Both entry points also take the un-repeated [B,T,Hq,dk] tensors and index the shared rows:
+    outputs, states and every gradient must equal the oracle on the repeated inputs, with dq, dk summed over the
+    heads of each group."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa, fused_recurrent_palimpsa
+    B, T, H, G, dk, dv = 2, 200, 6, 2, 48, 96
+    rep = H // G
+    full = _mamba_inputs(B, T, H, G, dk, dv, seed=31)
+    dtype = torch.bfloat16 if path == "chunk_bf16" else torch.float32
+    if dtype == torch.bfloat16:
+        full = hp.rounded(full, dtype)
+    gen = torch.Generator().manual_seed(32)
+    target = 0.05 * torch.randn(B, T, H, dv, generator=gen)
+    mu0 = torch.randn(B, H, dv, dk, generator=gen) * 0.05
+    I0 = 1.0 + torch.rand(B, H, dv, dk, generator=gen)
+    leaves64 = [full[n].double().clone().requires_grad_(True) for n in NAMES]
+    st64 = [mu0.double().clone().requires_grad_(True), I0.double().clone().requires_grad_(True)]
+    o_ref, _, fmu_ref, fI_ref = po.palimpsa_recurrence(*leaves64, *st64, scale=1.0, compute_dtype=torch.float64)
+    gr = torch.autograd.grad(0.5 * ((o_ref - target.double()) ** 2).sum(), leaves64 + st64)
+    ref = dict(zip(NAMES + ["mu0", "I0"], gr))
+    for n in ("q", "k"):     # the gradient of a shared row is the sum over the heads that read it
+        ref[n] = ref[n].reshape(B, T, G, rep, dk).sum(3)
+    dev = gpu_device
+    leaves = {n: full[n].to(dev).clone() for n in NAMES}
+    for n in ("q", "k"):
+        leaves[n] = leaves[n][:, :, ::rep].contiguous()              # one row per group
+        assert leaves[n].shape == (B, T, G, dk)
+    leaves = {n: x.requires_grad_(True) for n, x in leaves.items()}
+    leaves["mu0"] = mu0.to(dev).requires_grad_(True)
+    leaves["I0"] = I0.to(dev).requires_grad_(True)
+    fn = fused_recurrent_palimpsa if path == "recurrent_fp32" else chunk_palimpsa
+    o, fmu, fI = fn(*[leaves[n] for n in NAMES], scale=1.0, initial_mu_state=leaves["mu0"],
+                    initial_I_state=leaves["I0"], output_final_state=True)
+    (0.5 * ((o.float() - target.to(dev)) ** 2).sum()).backward()
+    bf = dtype == torch.bfloat16
+    assert hp.max_rel(o.float(), o_ref.detach()) <= (2e-2 if bf else hp.FP32_REL_TOL)
+    assert hp.max_rel(fmu, fmu_ref.detach()) <= (5e-3 if bf else hp.FP32_REL_TOL)
+    assert hp.max_rel(fI, fI_ref.detach()) <= (5e-3 if bf else hp.FP32_REL_TOL)
+    bad = {}
+    for n in NAMES + ["mu0", "I0"]:
+        assert leaves[n].grad.shape == leaves[n].shape
+        e = hp.max_rel(leaves[n].grad, ref[n])
+        print(f"d{n:4s}: max|d|/max|ref| = {e:.3e}")
+        if not e <= (hp.BF16_GRAD_NORM_TOL if bf else hp.CHUNK_FP32_GRAD_TOL):
+            bad[n] = e
+    assert not bad, bad
+
+
 # --------------------------------------------------------------------------- prefill -> decode hand-off
 def test_chunk_prefill_then_recurrent_decode_steps(gpu_device):
     """The layer's generate flow (layers/palimpsa.py:302-331): a chunked prefill returns (final_mu, final_I), which
