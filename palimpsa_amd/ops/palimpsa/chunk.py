@@ -27,6 +27,7 @@ import torch
 
 from ... import _lib as L
 from . import _common as cm
+from . import _custom_ops as _ops
 
 
 def _count_chunks(T: int, B: int) -> int:
@@ -222,7 +223,6 @@ class ChunkPalimpsa(torch.autograd.Function):
                 None, None, None, None, None, None, None, None)
 
 
-@cm.no_compile
 def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state=None, scale=None,
                    chunk_size=16, output_final_state=False, output_uncertainty=False, cu_seqlens=None):
     """Chunked Palimpsa attention; calling convention of chunk_palimpsa in the reference
@@ -232,6 +232,23 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
         scale = q.shape[-1] ** -0.5
     if not isinstance(chunk_size, int) or chunk_size <= 0:
         raise ValueError(f"chunk_size must be a positive int, got {chunk_size!r}")
+    if _ops.available() and torch.compiler.is_compiling():
+        # under a tracer the work is handed over as opaque library ops (see _custom_ops.py)
+        if cu_seqlens is not None and q.shape[0] != 1:
+            raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
+        o, o_var, final_mu_state, final_I_state, _, _ = _ops.chunk_fwd(
+            q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, float(scale), bool(output_uncertainty), cu_seqlens)
+        out = (o, o_var) if output_uncertainty else o
+        if output_final_state:
+            return out, final_mu_state, final_I_state
+        return out
+    return _eager_chunk(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size,
+                        output_final_state, output_uncertainty, cu_seqlens)
+
+
+@cm.no_compile
+def _eager_chunk(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, scale, chunk_size, output_final_state,
+                 output_uncertainty, cu_seqlens):
     chunk_offsets = None
     if cu_seqlens is not None:
         if q.shape[0] != 1:

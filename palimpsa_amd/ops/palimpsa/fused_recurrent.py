@@ -17,6 +17,7 @@ import torch
 
 from ... import _lib as L
 from . import _common as cm
+from . import _custom_ops as _ops
 
 
 def _recurrent_forward(q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I_state,
@@ -72,64 +73,80 @@ class FusedRecurrentPalimpsaFunction(torch.autograd.Function):
         # gradients arriving at the final states are ignored, as in the chunked path (chunk...py:522)
         q, k, v, b, gt, g, Ip, init_mu, init_I, cu = ctx.saved_tensors
         m = ctx.meta
-        dev = q.device
-        B, T, H, dv_p = v.shape
-        dk_p = q.shape[-1]
-        cd = m["compute_dtype"]
-        has_var = m["output_uncertainty"] and do_var is not None
-        if do is None:
-            do = torch.zeros(B, T, H, m["dv"], dtype=cd, device=dev)
+        p = cm.Prepared(q, k, v, b, gt, g, Ip, init_mu, init_I, cu, m["dk"], m["dv"], q.shape[-1], v.shape[-1],
+                        m["n_seqs"], m["compute_dtype"])
+        if not m["output_uncertainty"]:
+            do_var = None
+        gr = recurrent_backward(p, m["scale"], do, do_var, m["in_dtypes"], m["g_shape"], m["Ip_shape"])
+        return gr[:7] + (None, gr[7], gr[8], None, None, None)
 
-        def prep(x, dt):
-            x = x.to(dt)
-            if dv_p != m["dv"]:
-                x = torch.nn.functional.pad(x, (0, dv_p - m["dv"]))
-            return x.contiguous()
 
-        do_p = prep(do, cd)
-        dovar_p = prep(do_var, torch.float32) if has_var else None
-        dq, dk_, dv_, db = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(b)
-        dgt = torch.empty(B, T, H, dtype=torch.float32, device=dev)
-        dg = torch.empty(H, dtype=torch.float32, device=dev)
-        dIp = torch.empty(H, dtype=torch.float32, device=dev)
-        d_init_mu = torch.empty_like(init_mu) if m["has_init"] else None
-        d_init_I = torch.empty_like(init_I) if m["has_init"] else None
-        flags = 0
-        if cu is not None:
-            flags |= L.PAL_FLAG_VARLEN
-        if m["has_init"]:
-            flags |= L.PAL_FLAG_HAS_INIT
-        if has_var:
-            flags |= L.PAL_FLAG_HAS_VAR
-        dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
-                         dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
-                         flags=flags, scale=m["scale"], n_qk_heads=q.shape[2])
-        pt = cm._ptr
-        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
-                               init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))
-        grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk_), dv=pt(dv_), db=pt(db),
-                                dgt=pt(dgt), dg=pt(dg), dIp=pt(dIp), d_init_mu=pt(d_init_mu), d_init_I=pt(d_init_I))
-        lib = L.load()
-        ws_bytes = int(lib.pal_recurrent_bwd_workspace_bytes(dims))
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-        import ctypes as C
-        with torch.cuda.device(dev):
-            rc = lib.pal_recurrent_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes,
-                                       cm.current_stream_ptr(dev))
-        L.check(rc, "pal_recurrent_bwd")
-        dts = m["in_dtypes"]
-        dq = cm.unpad_last(dq, m["dk"]).to(dts[0])
-        dk_ = cm.unpad_last(dk_, m["dk"]).to(dts[1])
-        dv_ = cm.unpad_last(dv_, m["dv"]).to(dts[2])
-        db = cm.unpad_last(db, m["dv"]).to(dts[3])
-        if d_init_mu is not None and (dk_p != m["dk"] or dv_p != m["dv"]):
-            d_init_mu = d_init_mu[:, :, :m["dv"], :m["dk"]].contiguous()
-            d_init_I = d_init_I[:, :, :m["dv"], :m["dk"]].contiguous()
-        return (dq, dk_, dv_, db, dgt.to(dts[4]), dg.reshape(m["g_shape"]).to(dts[5]),
-                dIp.reshape(m["Ip_shape"]).to(dts[6]), None, d_init_mu, d_init_I, None, None, None)
+def recurrent_backward(p: "cm.Prepared", scale: float, do, do_var, in_dtypes, g_shape, Ip_shape):
+    """pal_recurrent_bwd on prepared (kernel-ready) inputs; returns (dq, dk, dv, db, dgt, dg, dIp, d_init_mu | None,
+    d_init_I | None) in the dtypes and shapes of the caller's tensors."""
+    import ctypes as C
+    q, k, v, b, gt, g, Ip, init_mu, init_I, cu = p.q, p.k, p.v, p.b, p.gt, p.g, p.Ip, p.init_mu, p.init_I, p.cu_seqlens
+    dev = q.device
+    B, T, H, dv_p = v.shape
+    dk_p = q.shape[-1]
+    cd = p.compute_dtype
+    has_init = init_mu is not None
+    has_var = do_var is not None
+    if do is None:
+        do = torch.zeros(B, T, H, p.dv, dtype=cd, device=dev)
+
+    def prep(x, dt):
+        x = x.to(dt)
+        if dv_p != p.dv:
+            x = torch.nn.functional.pad(x, (0, dv_p - p.dv))
+        return x.contiguous()
+
+    do_p = prep(do, cd)
+    dovar_p = prep(do_var, torch.float32) if has_var else None
+    dq, dk_, dv_, db = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(b)
+    dgt = torch.empty(B, T, H, dtype=torch.float32, device=dev)
+    dg = torch.empty(H, dtype=torch.float32, device=dev)
+    dIp = torch.empty(H, dtype=torch.float32, device=dev)
+    d_init_mu = torch.empty_like(init_mu) if has_init else None
+    d_init_I = torch.empty_like(init_I) if has_init else None
+    flags = 0
+    if cu is not None:
+        flags |= L.PAL_FLAG_VARLEN
+    if has_init:
+        flags |= L.PAL_FLAG_HAS_INIT
+    if has_var:
+        flags |= L.PAL_FLAG_HAS_VAR
+    dims = L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
+                     dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
+                     flags=flags, scale=float(scale), n_qk_heads=q.shape[2])
+    pt = cm._ptr
+    tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
+                           init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))
+    grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk_), dv=pt(dv_), db=pt(db),
+                            dgt=pt(dgt), dg=pt(dg), dIp=pt(dIp), d_init_mu=pt(d_init_mu), d_init_I=pt(d_init_I))
+    lib = L.load()
+    ws_bytes = int(lib.pal_recurrent_bwd_workspace_bytes(dims))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.pal_recurrent_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, cm.current_stream_ptr(dev))
+    L.check(rc, "pal_recurrent_bwd")
+    dts = in_dtypes
+    dq = cm.unpad_last(dq, p.dk).to(dts[0])
+    dk_ = cm.unpad_last(dk_, p.dk).to(dts[1])
+    dv_ = cm.unpad_last(dv_, p.dv).to(dts[2])
+    db = cm.unpad_last(db, p.dv).to(dts[3])
+    if d_init_mu is not None and (dk_p != p.dk or dv_p != p.dv):
+        d_init_mu = d_init_mu[:, :, :p.dv, :p.dk].contiguous()
+        d_init_I = d_init_I[:, :, :p.dv, :p.dk].contiguous()
+    return (dq, dk_, dv_, db, dgt.to(dts[4]), dg.reshape(g_shape).to(dts[5]), dIp.reshape(Ip_shape).to(dts[6]),
+            d_init_mu, d_init_I)
 
 
 @cm.no_compile
+def _eager_recurrent(*args):
+    return FusedRecurrentPalimpsaFunction.apply(*args)
+
+
 def fused_recurrent_palimpsa(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -159,9 +176,15 @@ def fused_recurrent_palimpsa(
             raise ValueError("Initial states mismatch sequence length.")
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    o, o_var, final_mu_state, final_I_state = FusedRecurrentPalimpsaFunction.apply(
-        q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I_state,
-        output_final_state, output_uncertainty, cu_seqlens)
+    if _ops.available() and torch.compiler.is_compiling():
+        # under a tracer the work is handed over as opaque library ops (see _custom_ops.py)
+        o, o_var, final_mu_state, final_I_state = _ops.recurrent_fwd(
+            q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, float(scale), bool(output_final_state),
+            bool(output_uncertainty), cu_seqlens)
+    else:
+        o, o_var, final_mu_state, final_I_state = _eager_recurrent(
+            q, k, v, b, gt, g, Ip, scale, initial_mu_state, initial_I_state, output_final_state, output_uncertainty,
+            cu_seqlens)
     out = (o, o_var) if output_uncertainty else o
     if output_final_state:
         return out, final_mu_state, final_I_state

@@ -211,26 +211,71 @@ def test_largest_head_dims_forward(gpu_device, dk, dv):
     assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
 
 
-def test_entry_point_under_torch_compile(gpu_device):
-    """A compiled function that calls the operator runs it as an opaque eager region (the reference was written with
-    torch.compile in mind): same results and gradients as eager."""
-    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
-    inp = hp.rounded(po.make_inputs(1, 100, 2, 32, 32, seed=8), torch.bfloat16)
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+@pytest.mark.parametrize("case", ["chunk_dense", "chunk_packed_state_var", "recurrent"])
+def test_entry_points_compile_without_a_graph_break(gpu_device, backend, case):
+    """torch.compile(fullgraph=True) over a function that calls the operators: the entry points hand the tracer
+    opaque library ops with shape-only implementations and registered gradients (the reference's wrapper was
+    written to be traceable, chunk...py:627-651), so there is no graph break; same values and gradients as eager
+    (the same kernels run).  'eager' exercises the tracer, 'aot_eager' also the fake tensors and the traced
+    backward; no code generation is involved in either."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa, fused_recurrent_palimpsa
     dev = gpu_device
+    names = ("q", "k", "v", "b", "gt", "g", "Ip")
+    extra = []
+    if case == "chunk_dense":
+        inp = hp.rounded(po.make_inputs(2, 100, 2, 32, 32, seed=8), torch.bfloat16)
 
-    def f(q, k, v, b, gt, g, Ip):
-        return (chunk_palimpsa(q * 1.0, k, v, b, gt, g, Ip, chunk_size=64).float() ** 2).sum()
+        def f(q, k, v, b, gt, g, Ip):
+            return (chunk_palimpsa(q * 1.0, k, v, b, gt, g, Ip, chunk_size=64).float() ** 2).sum()
+    elif case == "chunk_packed_state_var":
+        cu = torch.tensor([0, 70, 71, 200], device=dev)
+        inp = hp.rounded(po.make_inputs(1, 200, 2, 31, 65, seed=9), torch.bfloat16)     # padded head dims as well
+        gen = torch.Generator().manual_seed(1)
+        mu0 = (torch.randn(3, 2, 65, 31, generator=gen) * 0.1).to(dev).requires_grad_(True)
+        I0 = (1.0 + torch.rand(3, 2, 65, 31, generator=gen)).to(dev).requires_grad_(True)
+        extra = [mu0, I0]
+
+        def f(q, k, v, b, gt, g, Ip):
+            (o, ov), fmu, fI = chunk_palimpsa(q, k, v * 1.0, b, gt, g, Ip, initial_mu_state=mu0, initial_I_state=I0,
+                                              output_final_state=True, output_uncertainty=True, cu_seqlens=cu)
+            return (o.float() ** 2).sum() + ov.float().sum() + fmu.detach().sum() * 0.0
+    else:
+        inp = po.make_inputs(2, 40, 2, 32, 48, seed=10)
+
+        def f(q, k, v, b, gt, g, Ip):
+            o, fmu, fI = fused_recurrent_palimpsa(q, k * 1.0, v, b, gt, g, Ip, output_final_state=True)
+            return (o ** 2).sum() + fI.detach().sum() * 0.0
 
     def run(fn):
-        leaves = [inp[n].to(dev).clone().requires_grad_(n in ("q", "v")) for n in ("q", "k", "v", "b", "gt", "g", "Ip")]
+        leaves = [inp[n].to(dev).clone().requires_grad_(True) for n in names]
+        for x in extra:
+            x.grad = None
         out = fn(*leaves)
         out.backward()
-        return out.detach(), leaves[0].grad, leaves[2].grad
+        return [out.detach()] + [x.grad for x in leaves] + [x.grad.clone() for x in extra]
 
     eager = run(f)
-    compiled = run(torch.compile(f, backend="eager"))     # the tracer only: no code generation involved
+    torch._dynamo.reset()
+    compiled = run(torch.compile(f, backend=backend, fullgraph=True))
     for a, b_ in zip(eager, compiled):
         assert hp.max_rel(b_, a) <= 1e-6
+
+
+def test_library_ops_pass_opcheck(gpu_device):
+    """torch.library.opcheck on the four ops: schema, fake implementation against the real one, autograd registration."""
+    from palimpsa_amd.ops.palimpsa import _custom_ops as ops
+    dev = gpu_device
+    inp = hp.to_device(hp.rounded(po.make_inputs(1, 70, 2, 16, 32, seed=3), torch.bfloat16), dev)
+    q, k, v, b, gt, g, Ip = [inp[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")]
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    torch.library.opcheck(ops.chunk_fwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, True, None), test_utils=tests)
+    out = ops.chunk_fwd(q, k, v, b, gt, g, Ip, None, None, 0.25, False, None)
+    torch.library.opcheck(ops.chunk_bwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, None, out[4], out[5],
+                                          torch.ones_like(v), None), test_utils=tests)
+    torch.library.opcheck(ops.recurrent_fwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, True, True, None), test_utils=tests)
+    torch.library.opcheck(ops.recurrent_bwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, None, torch.ones_like(v), None),
+                          test_utils=tests)
 
 
 @pytest.mark.parametrize("dk,dv", [(96, 64), (80, 48), (32, 32)])
