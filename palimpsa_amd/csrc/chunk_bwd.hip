@@ -247,6 +247,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     const float* cI = a.chunk_I + tile_off + 16 * nb;
     float mu_n = cmu[i], I_n = cI[i];
 
+    // The producer of token blocks 2-3 has the longest iteration (both operand halves, twice the matrix instructions):
+    // the other three waves of its SIMD finish a row earlier and would leave it to issue alone at half rate, so it
+    // gets the issue slots first (measured: 1 % of the kernel; raising both producers or the consumers costs 3-10 %).
+    if (HF) __builtin_amdgcn_s_setprio(3);
     for (int it = 0; it <= dv; ++it) {
       if (it < dv) {
         const int d = it, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
@@ -367,6 +371,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
       iter_tail(it);
     }
 
+    if (HF) __builtin_amdgcn_s_setprio(0);
     TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb;
 #pragma unroll
     for (int tl = 0; tl < 2; ++tl)
