@@ -676,8 +676,9 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
 // number of resident workgroups that hides them).
 // PREC (fp32 rows): operands as two bf16 halves, three matrix instructions per product; the transposed copy of the
 // carries then holds a second plane with the lo halves (never shared with a result buffer).
+// (second launch bound: at most 256 registers per lane, so matrix results stay in ordinary vector registers)
 template <typename TIn, int KSMAX, bool SEQ, bool PREC>
-__global__ __launch_bounds__(256) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
+__global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
   const int H = a.H, dk = a.dk, dv = a.dv;

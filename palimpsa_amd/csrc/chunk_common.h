@@ -90,12 +90,15 @@ __device__ __forceinline__ int block_exponent_of(float m, int target) {
   return (m > 0.f && m < __builtin_inff()) ? ilogbf(m) - target : 0;
 }
 
+// vn > 0 restricts the maxima of v and b to the value rows [v0, v0 + vn) (a workgroup that only forms products of those)
 template <typename TIn>
 __device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, const TIn* vt, const TIn* bt, int Hq, int H,
                                                               int dk, int dv, int clen, int tid, int nthreads,
-                                                              float* sMax) {
+                                                              float* sMax, int v0 = 0, int vn = 0) {
   float km = 0.f, vm = 0.f, bm = 0.f;
-  const int gk = dk >> 3, gv = dv >> 3;
+  const int gk = dk >> 3, gv = (vn > 0 ? vn : dv) >> 3;
+  vt += v0;
+  bt += v0;
   for (int idx = tid; idx < kC * gk; idx += nthreads) {
     const int s = idx / gk, c = idx - s * gk;
     if (s < clen) {

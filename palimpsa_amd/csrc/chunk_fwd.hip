@@ -334,8 +334,10 @@ __device__ __forceinline__ constexpr int lidx(int tb, int ks) { return tb < 2 ? 
 // share the barriers), so that a workgroup of two waves becomes one of four and covers all four SIMDs.
 // PREC (fp32 rows): the rows are staged in fp32, the operands X and L are formed in fp32 and split into two bf16
 // halves each, three matrix instructions per product (no block exponents: bf16 has the range of fp32).
+// (the second launch bound caps the register budget at 256 per lane: the matrix results then stay in ordinary vector
+// registers instead of being copied out of accumulation registers, 32 copies per value row in this kernel)
 template <typename TIn, int NB, bool HAS_VAR, int RS, int TS, bool PREC>
-__global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs a) {
+__global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkArgs a) {
   extern __shared__ float smem[];
   using TSt = std::conditional_t<PREC, float, f16_t>;   // element type of the staged v, b rows
   constexpr int NT = NB * RS * 64;        // threads per (tile, head)
@@ -594,6 +596,244 @@ __global__ __launch_bounds__(NB * RS * TS * 64) void chunk_out_kernel(ChunkArgs 
   }
 }
 
+// The same outputs with the work of a (tile, head) laid out by value rows instead of by key columns: four waves, wave w
+// owns the value rows d = w mod 4 and walks over all column blocks of its rows, so a workgroup is four waves whatever
+// the head dim and every SIMD of a unit carries the same load.  A workgroup takes a slice of at most 64 value rows
+// (blockIdx.y), which keeps three workgroups on a compute unit.  v^T and b^T of the slice stay in LDS (f16,
+// block-scaled by the maxima of the slice); the k columns (scaled, with their squares) and the q rows of the next column
+// block are staged by the whole workgroup while the rows of the current one are processed (two buffers, one barrier per
+// column block), and the outputs are summed over the column blocks in an LDS tile that only the owning wave touches.
+// bf16 rows only.  Three waves per SIMD: 168 registers per lane, matrix results in ordinary vector registers.
+constexpr int kKH = 72;   // row stride (f16) of the staged k columns
+
+template <bool HAS_VAR>
+__global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int dvs) {
+  extern __shared__ float smem[];
+  using TIn = bf16_t;
+  const int tid = (int)threadIdx.x, lane = tid & 63, w = tid >> 6, i = lane & 15, g = lane >> 4;
+  const int H = a.H, dk = a.dk, dv = a.dv;
+  const int cidx = (int)(blockIdx.x / H), h = (int)(blockIdx.x % H);
+  const int r0 = (int)blockIdx.y * dvs, rn = min(dvs, dv - r0);   // value rows [r0, r0 + rn) of this workgroup
+  int seq, t0, clen, cis;
+  chunk_lookup(a, cidx, seq, t0, clen, cis);
+  float* sC = smem;                        // [64] running log2-decay inside the tile
+  f16_t* sV = (f16_t*)(sC + kC);           // [dvs][kVH] v^T 2^-ev
+  f16_t* sB = sV + dvs * kVH;              // [dvs][kVH] b^T 2^-eb
+  f16_t* sK = sB + dvs * kVH;              // [2][16][kKH] k^T 2^-ek of a column block
+  f16_t* sKK = sK + 2 * 16 * kKH;          // [2][16][kKH] its squares
+  bf16_t* sQ = (bf16_t*)(sKK + 2 * 16 * kKH);   // [2][64][16] q rows of a column block
+  float* sO = (float*)(sQ + 2 * kC * 16);  // [dvs][64] outputs summed over the column blocks
+  float* sOv = sO + dvs * kC;              // same for o_var
+  const float Ip = a.Ip[h];
+  const float gh = a.g[h] * kLog2e;
+  if (tid < 64) {
+    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    sC[lane] = wave_inclusive_scan(-gt * gh, lane);
+  }
+  const TIn* vp = (const TIn*)a.v + ((int64_t)t0 * H + h) * dv + r0;
+  const TIn* bp = (const TIn*)a.b + ((int64_t)t0 * H + h) * dv + r0;
+  const TIn* kbase = (const TIn*)a.k + qk_row(a, t0, h);
+  const TIn* qbase = (const TIn*)a.q + qk_row(a, t0, h);
+  // staging work item of this thread, for v, b (16 value rows per step) and for k, q (one column block per step):
+  // (token ss, 4 consecutive rows or columns sq)
+  const int ss = tid >> 2, sq = tid & 3;
+  const bool s_ok = ss < clen;
+  const unsigned kq_off = (unsigned)(s_ok ? ss : 0) * (unsigned)qk_stride(a) + 4u * sq;   // a tile spans < 2^31 elements
+  bf16x4 k_next, q_next;   // the thread's share of the next column block, as loaded
+  auto request = [&](int nb) {
+    k_next = *(const bf16x4*)(kbase + 16 * nb + kq_off);
+    q_next = *(const bf16x4*)(qbase + 16 * nb + kq_off);
+  };
+  request(0);
+  const TileExponents bexp = tile_block_exponents(kbase, vp - r0, bp - r0, a.Hq, H, dk, dv, clen, tid, 256, sO, r0, rn);
+  const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
+  const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
+  const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
+  auto deposit = [&](int buf) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float ksc = s_ok ? (float)k_next[e] * down_k : 0.f;
+      sK[(buf * 16 + 4 * sq + e) * kKH + ss] = (f16_t)ksc;
+      sKK[(buf * 16 + 4 * sq + e) * kKH + ss] = (f16_t)(ksc * ksc);
+    }
+    *(bf16x4*)&sQ[(buf * kC + ss) * 16 + 4 * sq] = q_next;
+  };
+  deposit(0);
+  {
+    const int n_groups = rn / kDG;
+#pragma unroll 2
+    for (int dg = 0; dg < n_groups; ++dg) {
+      float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f};
+      if (s_ok) {
+        load_vec<4>(vp + (int64_t)ss * H * dv + dg * kDG + 4 * sq, x);
+        load_vec<4>(bp + (int64_t)ss * H * dv + dg * kDG + 4 * sq, y);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sV[(dg * kDG + 4 * sq + e) * kVH + ss] = (f16_t)(x[e] * down_v);
+        sB[(dg * kDG + 4 * sq + e) * kVH + ss] = (f16_t)(y[e] * down_b);
+      }
+    }
+  }
+  __syncthreads();
+
+  // per-wave constants of the tile (see chunk_out_kernel)
+  float Fm[4], Fj[4], Gi[4], ct[4];
+#pragma unroll
+  for (int tb = 0; tb < 4; ++tb) {
+    ct[tb] = sC[16 * tb + i];
+    const float F = fast_exp2(ct[tb]);
+    Fm[tb] = (F * down_k) * down_v;
+    Fj[tb] = ((F * down_k) * down_k) * down_b;
+    Gi[tb] = ((((1.f - F) * Ip) * down_k) * down_k) * down_b;
+  }
+  f16x8 Lr[6];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    float cs[8];
+    *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
+    *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = 8 * g + j + 32 * ks;
+#pragma unroll
+      for (int tb = (ks ? 2 : 0); tb < 4; ++tb) {
+        const int t = 16 * tb + i;
+        Lr[lidx(tb, ks)][j] = (f16_t)((s <= t) ? fast_exp2(ct[tb] - cs[j]) : 0.f);
+      }
+    }
+  }
+  const float scale = ((a.scale * __builtin_amdgcn_exp2f((float)bexp.ev)) * down_k) * down_b;
+  const float scale_var = ((a.scale * down_k) * down_k) * down_b;
+
+  const int n_blocks = dk >> 4;
+  const float* cmu0 = a.chunk_mu + (((int64_t)cidx * H + h) * dv + r0) * dk + 4 * g;
+  const float* cI0 = a.chunk_I + (((int64_t)cidx * H + h) * dv + r0) * dk + 4 * g;
+  f32x4 mu0_n = *(const f32x4*)(cmu0 + (int64_t)w * dk), I0_n = *(const f32x4*)(cI0 + (int64_t)w * dk);
+#pragma unroll 1
+  for (int nb = 0; nb < n_blocks; ++nb) {
+    const int buf = nb & 1;
+    const bool more = nb + 1 < n_blocks;
+    f16x8 kA[2], kk[2];
+    float qD[4][4];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      kA[ks] = *(const f16x8*)&sK[(buf * 16 + i) * kKH + 8 * g + 32 * ks];
+      kk[ks] = *(const f16x8*)&sKK[(buf * 16 + i) * kKH + 8 * g + 32 * ks];
+    }
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+      const bf16x4 x = *(const bf16x4*)&sQ[(buf * kC + 16 * tb + i) * 16 + 4 * g];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) qD[tb][r] = (float)x[r];
+    }
+    if (more) request(nb + 1);
+    const float* cmu = cmu0 + 16 * nb;
+    const float* cI = cI0 + 16 * nb;
+#pragma unroll 1
+    for (int d = w; d < rn; d += 4) {
+      const f32x4 mu0 = mu0_n, I0 = I0_n;
+      {
+        // the state row of the next iteration: the wave's next row, or its first row of the next column block
+        const bool last = d + 4 >= rn;
+        const int64_t dn = last ? (int64_t)w * dk + (more ? 16 : 0) : (int64_t)(d + 4) * dk;
+        mu0_n = *(const f32x4*)(cmu + dn);
+        I0_n = *(const f32x4*)(cI + dn);
+      }
+      float* so = sO + d * kC + 16 * g + i;
+      float* sov = sOv + d * kC + 16 * g + i;
+      float prev = 0.f, prevv = 0.f;
+      if (nb) {
+        prev = *so;
+        if (HAS_VAR) prevv = *sov;
+      }
+      float M0[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) M0[r] = mu0[r] * I0[r];
+      f16x8 XM[2], XJ[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        XM[ks] = kA[ks] * *(const f16x8*)&sV[d * kVH + 8 * g + 32 * ks];
+        XJ[ks] = kk[ks] * *(const f16x8*)&sB[d * kVH + 8 * g + 32 * ks];
+      }
+      float p[4], pv[4];
+#pragma unroll
+      for (int tb = 0; tb < 4; ++tb) {
+        f32x4 accM = {0.f, 0.f, 0.f, 0.f};
+        f32x4 accI = {Gi[tb], Gi[tb], Gi[tb], Gi[tb]};
+        accM = mfma16h(XM[0], Lr[lidx(tb, 0)], accM);
+        accI = mfma16h(XJ[0], Lr[lidx(tb, 0)], accI);
+        if (tb >= 2) {
+          accM = mfma16h(XM[1], Lr[lidx(tb, 1)], accM);
+          accI = mfma16h(XJ[1], Lr[lidx(tb, 1)], accI);
+        }
+        float acc = 0.f, accv = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float Mf = fmaf(Fm[tb], M0[r], accM[r]);
+          const float If = fmaf(Fj[tb], I0[r], accI[r]);
+          const float rI = fast_rcp(If);
+          acc = fmaf(Mf * rI, qD[tb][r], acc);
+          if (HAS_VAR) accv = fmaf(qD[tb][r] * qD[tb][r], rI, accv);
+        }
+        p[tb] = acc;
+        pv[tb] = accv;
+      }
+      *so = prev + rows4_sum_x4(p[0], p[1], p[2], p[3]);
+      if (HAS_VAR) *sov = prevv + rows4_sum_x4(pv[0], pv[1], pv[2], pv[3]);
+    }
+    if (more) deposit(buf ^ 1);
+    // the other buffer is complete for the next column block (it was last read before the previous barrier); after
+    // the last block: the outputs are complete
+    __syncthreads();
+  }
+  // outputs: work item = (token ss, 4 value rows sq)
+  if (s_ok) {
+    const int n_groups = rn / kDG;
+    for (int dg = 0; dg < n_groups; ++dg) {
+      const int64_t off = ((int64_t)(t0 + ss) * H + h) * dv + r0 + dg * kDG + 4 * sq;
+      TIn* op = (TIn*)a.o + off;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) op[e] = from_f32<TIn>(sO[(dg * kDG + 4 * sq + e) * kC + ss] * scale);
+      if (HAS_VAR) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) store_rt(a.o_var, off + e, sOv[(dg * kDG + 4 * sq + e) * kC + ss] * scale_var, a.var_bf16);
+      }
+    }
+  }
+}
+
+// value rows per workgroup of chunk_out_rows_kernel: equal slices (multiples of 16) of at most 64 rows, 48 with o_var,
+// so that three workgroups fit the LDS of a compute unit
+static int out_rows_slice(int dv, bool var) {
+  const int cap = var ? 48 : 64;
+  const int n = (dv + cap - 1) / cap;
+  return ((dv / 16 + n - 1) / n) * 16;
+}
+static size_t out_rows_lds_bytes(int dv, bool var) {
+  const size_t dvs = out_rows_slice(dv, var);
+  return sizeof(float) * kC + 2 * sizeof(f16_t) * dvs * kVH + 4 * sizeof(f16_t) * 16 * kKH + 2 * sizeof(bf16_t) * kC * 16 +
+         sizeof(float) * dvs * kC * (var ? 2 : 1);
+}
+static int launch_out_rows(const ChunkArgs& a, hipStream_t s) {
+  const bool var = a.flags & PAL_FLAG_HAS_VAR;
+  const size_t lds = out_rows_lds_bytes(a.dv, var);
+  const int64_t blocks = (int64_t)a.total_chunks * a.H;
+  if (blocks > 0x7fffffff) return PAL_E_DIM;
+  if (lds > kMaxLds) return PAL_E_HEADDIM;
+  const int dvs = out_rows_slice(a.dv, var);
+  const dim3 grid((unsigned)blocks, (unsigned)((a.dv + dvs - 1) / dvs));
+  if (var) {
+    if (int rc = allow_lds((const void*)&chunk_out_rows_kernel<true>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_rows_kernel<true>), grid, dim3(256), lds, s, a, dvs);
+  } else {
+    if (int rc = allow_lds((const void*)&chunk_out_rows_kernel<false>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernChunkOut, s, (chunk_out_rows_kernel<false>), grid, dim3(256), lds, s, a, dvs);
+  }
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
 template <typename TIn, int NB, bool PREC>
 static int launch_out_nb_p(const ChunkArgs& a, hipStream_t s) {
   const bool var = a.flags & PAL_FLAG_HAS_VAR;
@@ -630,6 +870,13 @@ static int launch_out_nb(const ChunkArgs& a, hipStream_t s) {
 
 template <typename TIn>
 static int launch_out(const ChunkArgs& a, hipStream_t s) {
+  if constexpr (std::is_same_v<TIn, bf16_t>) {
+    // bf16 rows: the layout by value rows (chunk_out_rows_kernel) unless a workgroup of the layout by key columns is
+    // exactly two or four waves on at most 64 value rows (measured: 3-7 % faster there, 3-25 % slower elsewhere)
+    const int nbk = a.dk / 16;
+    const bool by_columns = a.dv <= 64 && (nbk == 2 || nbk == 4);
+    if (!by_columns && out_rows_lds_bytes(a.dv, a.flags & PAL_FLAG_HAS_VAR) <= kMaxLds) return launch_out_rows(a, s);
+  }
   switch (a.dk / 16) {
     case 1: return launch_out_nb<TIn, 1>(a, s);
     case 2: return launch_out_nb<TIn, 2>(a, s);

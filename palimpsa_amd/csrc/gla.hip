@@ -72,8 +72,9 @@ struct GlaTileArgs {
 //                   + sum_y Z^T[e,y] P^T[y,x]   A = Z^T rows (LDS, read with the token map above)
 //      so every state entry is read by exactly one wave of the workgroup.
 // EB = ceil(de / 64) column blocks per wave.
+// (second launch bound: at most 256 registers per lane, so matrix results stay in ordinary vector registers)
 template <typename TIn, int EB, bool REVERSE, bool STATE_T>
-__global__ __launch_bounds__(256) void gla_tile_kernel(GlaTileArgs A) {
+__global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
   extern __shared__ float smem[];
   const ChunkArgs& a = A.c;
   const int H = a.H, dc = A.dc, de = A.de;

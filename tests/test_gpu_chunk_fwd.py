@@ -291,3 +291,28 @@ def test_output_kernel_wave_layouts_with_uncertainty(gpu_device, dk, dv):
     assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_abs(ov, ov_ref) <= hp.BF16_OUT_ABS_TOL
     assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
+@pytest.mark.parametrize("dk,dv,var", [(112, 112, False), (64, 96, True), (96, 192, False), (48, 80, True),
+                                       (16, 64, False), (128, 128, True)])
+def test_output_kernel_row_layout_slices_packed(gpu_device, dk, dv, var):
+    """Head dims whose forward output kernel is laid out by value rows, with slices of unequal size (112 = 64 + 48,
+    80 = 48 + 32 with uncertainty), several slices (192 = 3 x 64), one column block (dk = 16) and eight, on a packed
+    batch with tiles of 1, 2, 63 and 64 tokens and an initial state per document."""
+    ck, _ = _ops()
+    H = 2
+    cu = [0, 1, 3, 66, 130, 257]
+    T, N = cu[-1], len(cu) - 1
+    inp = hp.rounded(po.make_inputs(1, T, H, dk, dv, seed=dk * 3 + dv), torch.bfloat16)
+    gen = torch.Generator().manual_seed(5)
+    mu0 = torch.randn(N, H, dv, dk, generator=gen) * 0.1
+    I0 = 1.0 + torch.rand(N, H, dv, dk, generator=gen)
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0, I0=I0, cu=cu, want_var=var)
+    d = hp.to_device(inp, gpu_device)
+    out, mu, I = _call(ck, d, initial_mu_state=mu0.to(gpu_device), initial_I_state=I0.to(gpu_device),
+                       output_final_state=True, output_uncertainty=var, cu_seqlens=torch.tensor(cu, device=gpu_device))
+    o, ov = out if var else (out, None)
+    assert hp.max_abs(o, o_ref) <= hp.BF16_OUT_ABS_TOL
+    if var:
+        assert hp.max_abs(ov, ov_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
