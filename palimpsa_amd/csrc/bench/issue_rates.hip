@@ -149,6 +149,57 @@ template <int MODE> __global__ void k(float* out, long long* cyc, float a, float
                         "v_cvt_pk_bf16_f32 %4, %1, %2\n v_mul_f32 %1, %1, %7\n v_fma_f32 %2, %2, %7, %8\n v_rcp_f32 %3, %3"
                          : "+v"(c0), "+v"(x1), "+v"(x2), "+v"(x3), "=v"(r0) : "v"(A), "v"(B), "v"(a), "v"(b));) )
       x0 += __uint_as_float(r0) * 1e-30f;
+    } else if (MODE == 32) {  // matrix instructions of two operand types in turn (bf16, f16, bf16, f16), independent
+      REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_f16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_f16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+    } else if (MODE == 33) {  // half of the waves issue bf16 matrix instructions, the other half f16
+      if ((threadIdx.x >> 6) & 4) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                          : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        REP4(asm volatile("v_mfma_f32_16x16x32_f16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_f16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_f16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_f16 %3, %4, %5, %3"
+                          : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      }
+    } else if (MODE == 34) {  // packed f16 multiply feeding a matrix instruction: 4 products + 1 matrix instruction, x4
+      REP4(asm volatile("v_pk_mul_f16 %1, %1, %5\n v_pk_mul_f16 %2, %2, %5\n v_pk_mul_f16 %3, %3, %5\n v_pk_mul_f16 %4, %4, %5\n v_mfma_f32_16x16x32_f16 %0, %6, %7, %0"
+                        : "+v"(c0), "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3) : "v"(a), "v"(A), "v"(B));)
+    } else if (MODE == 40) {  // one wave in four issues matrix instructions only (16), the other three v_rcp_f32 (64 each)
+      if (((threadIdx.x >> 6) >> 2) == 0) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        REP16(asm volatile("v_rcp_f32 %0, %0\n v_rcp_f32 %1, %1\n v_rcp_f32 %2, %2\n v_rcp_f32 %3, %3" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));)
+      }
+    } else if (MODE == 41) {  // one wave in four issues matrix instructions only (16), the other three v_cvt_pk_bf16_f32 (64 each)
+      if (((threadIdx.x >> 6) >> 2) == 0) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        unsigned r0, r1, r2, r3;
+        REP16(asm volatile("v_cvt_pk_bf16_f32 %0, %4, %5\n v_cvt_pk_bf16_f32 %1, %5, %6\n v_cvt_pk_bf16_f32 %2, %6, %7\n v_cvt_pk_bf16_f32 %3, %7, %4" : "=v"(r0), "=v"(r1), "=v"(r2), "=v"(r3) : "v"(x0), "v"(x1), "v"(x2), "v"(x3));)
+        x0 += __uint_as_float(r0 ^ r1 ^ r2 ^ r3) * 1e-30f;
+      }
+    } else if (MODE == 42) {  // one wave in four issues matrix instructions only (16), the other three v_pk_mul_f16 (64 each)
+      if (((threadIdx.x >> 6) >> 2) == 0) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        REP16(asm volatile("v_pk_mul_f16 %0, %0, %4\n v_pk_mul_f16 %1, %1, %4\n v_pk_mul_f16 %2, %2, %4\n v_pk_mul_f16 %3, %3, %4" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3) : "v"(a));)
+      }
+    } else if (MODE == 43) {  // one wave in four issues matrix instructions only (16), the other three v_and_b32 / v_lshlrev_b32 (64 each)
+      if (((threadIdx.x >> 6) >> 2) == 0) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        REP16(asm volatile("v_and_b32 %0, %0, %4\n v_lshlrev_b32 %1, 1, %1\n v_and_b32 %2, %2, %4\n v_lshlrev_b32 %3, 1, %3" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3) : "v"(a));)
+      }
+    } else if (MODE == 44) {  // one wave in four issues matrix instructions only (16), the other three v_permlane32_swap (64 each)
+      if (((threadIdx.x >> 6) >> 2) == 0) {
+        REP4(asm volatile("v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n v_mfma_f32_16x16x32_bf16 %1, %4, %5, %1\n v_mfma_f32_16x16x32_bf16 %2, %4, %5, %2\n v_mfma_f32_16x16x32_bf16 %3, %4, %5, %3"
+                        : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3) : "v"(A), "v"(B));)
+      } else {
+        REP16(asm volatile("v_permlane32_swap_b32 %0, %1\n v_permlane32_swap_b32 %2, %3\n v_permlane32_swap_b32 %0, %1\n v_permlane32_swap_b32 %2, %3" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));)
+      }
     } else if (MODE == 13) {  // ds_read_b128 dependent latency (pointer chase on zeroed lds)
       int p = addr;
       REP16(asm volatile("ds_read_b32 %0, %0\n s_waitcnt lgkmcnt(0)" : "+v"(p));)
@@ -217,6 +268,16 @@ int main() {
     run<28>("4 mfma back to back + 28 fma", wps, 128, out, cyc);
     run<30>("1 mfma + 7 mixed valu (per 8)", wps, 128, out, cyc);
     run<31>("7 mixed valu alone (per 7)", wps, 112, out, cyc);
+    run<32>("mfma bf16, f16 in turn, 4 indep", wps, 16, out, cyc);
+    if (wps >= 2) run<33>("half the waves mfma bf16, half f16", wps, 16, out, cyc);
+    run<34>("4 v_pk_mul_f16 + 1 mfma f16 (per 5)", wps, 20, out, cyc);
+    if (wps == 4) {
+      run<40>("1 wave mfma only, 3 waves rcp only", wps, 52, out, cyc);
+      run<41>("1 wave mfma only, 3 waves cvt_pk only", wps, 52, out, cyc);
+      run<42>("1 wave mfma only, 3 waves pk_mul_f16 only", wps, 52, out, cyc);
+      run<43>("1 wave mfma only, 3 waves and/shl only", wps, 52, out, cyc);
+      run<44>("1 wave mfma only, 3 waves permlane32_swap", wps, 52, out, cyc);
+    }
     if (wps == 4) run<27>("1 wave mfma only, 3 waves fma only", wps, 52, out, cyc);
   }
   return 0;
