@@ -46,7 +46,7 @@ CHUNK = 64
 # per launch at the headline shape, times 64 lanes, divided by tokens*H*dk*dv
 # (profiles/bench_c1.sq_counters_pmc.txt).  Like the traffic figures below they cannot be read from inside this
 # process and are stale once those kernels change.
-VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 31.7, "chunk_out_kernel": 8.2}
+VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 31.7, "chunk_out_kernel": 8.0}
 # HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
 # from inside this process, so the figures are carried here and are stale once those kernels change.
