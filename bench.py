@@ -218,7 +218,39 @@ def bench_decode(torch, dev, steps):
     ms_k, n_k = kern.get("recurrent_fwd_kernel", (float("nan"), 1))
     avg_ms = ms_k / max(n_k, 1)
     gbs_kernel = bytes_step / (avg_ms * 1e-3) / 1e9
+
+    # the same steps with the mean state kept in bf16 between steps (an optional cache format: 12 bytes per state
+    # entry and step instead of 16), through the bound step a server would use
+    from palimpsa_amd.ops.palimpsa import DecodeStep, mu_to_cache
+    dec = DecodeStep(B, H, d, d, dev, torch.bfloat16, mu_dtype=torch.bfloat16)
+    mu16, I16 = mu_to_cache(mu), I.clone()
+    bound = [dec] + [DecodeStep(B, H, d, d, dev, torch.bfloat16, mu_dtype=torch.bfloat16) for _ in range(ncyc - 1)]
+    for t, ds in enumerate(bound):
+        r = rows[t]
+        ds.bind(r["q"], r["k"], r["v"], r["b"], r["gt"], g, Ip, mu16, I16)
+    for t in range(8):
+        bound[t % ncyc].step()
+    torch.cuda.synchronize()
+    L.profile_enable(True)
+    t0 = time.perf_counter()
+    for t in range(steps):
+        bound[t % ncyc].step()
+    torch.cuda.synchronize()
+    elapsed16 = time.perf_counter() - t0
+    kern16 = L.profile_read()
+    L.profile_enable(False)
+    bytes16 = (12 * E + 2 * (2 * d + 2 * d) + 4 + 2 * d) * B * H
+    ms16, n16 = kern16.get("recurrent_fwd_kernel", (float("nan"), 1))
+    avg16 = ms16 / max(n16, 1)
+    bf16_mu = {
+        "workload": "c3 shape with the mean state kept in bf16 between steps (DecodeStep(mu_dtype=bfloat16)), I fp32",
+        "steps": steps, "tokens_per_s": B * steps / elapsed16, "ms_per_step": elapsed16 * 1e3 / steps,
+        "roofline": {"bound": "hbm", "kernel": "recurrent_fwd_kernel", "achieved": bytes16 / (avg16 * 1e-3) / 1e9,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": bytes16 / (avg16 * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                     "traffic": None, "algorithmic_bytes_per_launch": bytes16, "avg_launch_ms": avg16},
+    }
     return {
+        "bf16_mean_state": bf16_mu,
         "workload": "c3: single-token decode B=256 H=16 dk=dv=128 bf16 rows fp32 states",
         "steps": steps, "tokens_per_s": B * steps / elapsed, "ms_per_step": elapsed * 1e3 / steps,
         "hbm_gbs_wall": bytes_step * steps / elapsed / 1e9,

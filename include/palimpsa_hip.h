@@ -55,6 +55,13 @@ extern "C" {
 #define PAL_FLAG_STATES_ONE_PASS 512u    /* one pass per (sequence, head) that keeps the running state in
                                             registers, wherever it applies (bf16 rows)                       */
 
+/* pal_recurrent_fwd only (every other entry point answers PAL_E_STATE): init_mu and final_mu point to bf16 arrays of the
+ * same shape.  A cache format for decode, where the state is all the traffic: 12 instead of 16 bytes per state entry
+ * and step.  The precision state I stays fp32 (it accumulates small increments); mu is rounded to bf16 once per call,
+ * an error of 2^-9 relative per call that decays with the forgetting factor.  No counterpart in the reference
+ * (its states are fp32: fused_recurrent_palimpsa.py:84-96, :145-154). */
+#define PAL_FLAG_STATE_MU_BF16 2048u
+
 /* error codes (negative) */
 #define PAL_OK 0
 #define PAL_E_NULL -1        /* required pointer is NULL                      */

@@ -16,6 +16,7 @@ PAL_ABI_VERSION = 3
 PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
 PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS, PAL_FLAG_FP32_FAST = 256, 512, 1024
+PAL_FLAG_STATE_MU_BF16 = 2048   # pal_recurrent_fwd: mu kept in bf16 between calls (DecodeStep(mu_dtype=torch.bfloat16))
 PAL_CHUNK = 64
 
 PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5

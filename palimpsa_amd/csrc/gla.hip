@@ -343,6 +343,7 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   if (!t) return PAL_E_NULL;
   if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o || !t->chunk_I) return PAL_E_NULL;
   if (d->flags & PAL_FLAG_HAS_VAR) return PAL_E_STATE;   // no precision state, no output variance
+  if (d->flags & PAL_FLAG_STATE_MU_BF16) return PAL_E_STATE;
   if (d->n_qk_heads != 0 && d->n_qk_heads != d->n_heads) return PAL_E_DIM;   // shared q/k heads: Palimpsa entry points only
   if (((d->flags & PAL_FLAG_HAS_INIT) != 0) != (t->init_mu != nullptr)) return PAL_E_STATE;
   if (((d->flags & PAL_FLAG_STORE_FINAL) != 0) != (t->final_mu != nullptr)) return PAL_E_STATE;

@@ -129,6 +129,7 @@ extern "C" int pal_gla_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, v
   if (!t) return PAL_E_NULL;
   if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o) return PAL_E_NULL;
   if (d->flags & PAL_FLAG_HAS_VAR) return PAL_E_STATE;
+  if (d->flags & PAL_FLAG_STATE_MU_BF16) return PAL_E_STATE;
   if (((d->flags & PAL_FLAG_HAS_INIT) != 0) != (t->init_mu != nullptr)) return PAL_E_STATE;
   if (((d->flags & PAL_FLAG_STORE_FINAL) != 0) != (t->final_mu != nullptr)) return PAL_E_STATE;
   const bool varlen = d->flags & PAL_FLAG_VARLEN;

@@ -91,6 +91,7 @@ namespace pal {
 int check_fwd_common(const PalDims* d, const PalFwdTensors* t) {
   int rc = pal_validate_dims(d);
   if (rc) return rc;
+  if (d->flags & PAL_FLAG_STATE_MU_BF16) return PAL_E_STATE;   // pal_recurrent_fwd clears it before it comes here
   if (!t) return PAL_E_NULL;
   if (!t->q || !t->k || !t->v || !t->b || !t->gt || !t->g || !t->Ip || !t->o) return PAL_E_NULL;
   const bool has_init = d->flags & PAL_FLAG_HAS_INIT;

@@ -123,6 +123,32 @@ __device__ __forceinline__ void store_vec_stream(float* p, const float* in) {
   }
 }
 
+// the same for a bf16 array (a state kept in bf16): widened to fp32 on load, rounded to nearest even on store
+template <int VW>
+__device__ __forceinline__ void load_vec_stream(const bf16_t* p, float* out) {
+  if constexpr (VW == 4) {
+    const bf16x4 x = __builtin_bit_cast(bf16x4, __builtin_nontemporal_load((const f32x2*)p));
+    out[0] = (float)x[0]; out[1] = (float)x[1]; out[2] = (float)x[2]; out[3] = (float)x[3];
+  } else if constexpr (VW == 2) {
+    const bf16x2 x = __builtin_bit_cast(bf16x2, __builtin_nontemporal_load((const float*)p));
+    out[0] = (float)x[0]; out[1] = (float)x[1];
+  } else {
+    out[0] = (float)__builtin_bit_cast(bf16_t, __builtin_nontemporal_load((const unsigned short*)p));
+  }
+}
+template <int VW>
+__device__ __forceinline__ void store_vec_stream(bf16_t* p, const float* in) {
+  if constexpr (VW == 4) {
+    const bf16x4 x = {(bf16_t)in[0], (bf16_t)in[1], (bf16_t)in[2], (bf16_t)in[3]};
+    __builtin_nontemporal_store(__builtin_bit_cast(f32x2, x), (f32x2*)p);
+  } else if constexpr (VW == 2) {
+    const bf16x2 x = {(bf16_t)in[0], (bf16_t)in[1]};
+    __builtin_nontemporal_store(__builtin_bit_cast(float, x), (float*)p);
+  } else {
+    __builtin_nontemporal_store(__builtin_bit_cast(unsigned short, (bf16_t)in[0]), (unsigned short*)p);
+  }
+}
+
 // ------------------------------------------------------- cross-lane helpers
 // rotate within each row of 16 lanes (DPP row_ror:N)
 template <int N>

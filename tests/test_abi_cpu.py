@@ -121,6 +121,13 @@ def test_entry_points_reject_bad_arguments_without_touching_a_gpu(L):
                              None) == L.PAL_E_WORKSPACE
     assert lib.pal_chunk_bwd_workspace_bytes(_dims(L)) > 0
     assert lib.pal_chunk_bwd_workspace_bytes(_dims(L, dk=5)) == 0
+    # the bf16 cache format of the mean state belongs to pal_recurrent_fwd alone
+    mu16 = L.PAL_FLAG_STATE_MU_BF16
+    assert lib.pal_chunk_fwd(_dims(L, flags=L.PAL_FLAG_STORE_FINAL | mu16, total_chunks=2), _fwd_tensors(L, **ok_chunk),
+                             None) == L.PAL_E_STATE
+    assert lib.pal_chunk_bwd(_dims(L, flags=mu16), _fwd_tensors(L, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)), gr,
+                             None, 0, None) == L.PAL_E_STATE
+    assert lib.pal_recurrent_fwd(_dims(L, flags=mu16 | L.PAL_FLAG_HAS_INIT), _fwd_tensors(L), None) == L.PAL_E_STATE
 
 
 def test_error_codes_map_to_python_exceptions(L):

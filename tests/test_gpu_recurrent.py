@@ -313,3 +313,42 @@ def test_bound_decode_step_with_several_tokens_per_step(gpu_device):
     assert hp.max_rel(mu3, mu_ref) <= hp.FP32_REL_TOL and hp.max_rel(I3, I_ref) <= hp.FP32_REL_TOL
     with pytest.raises(ValueError):
         DecodeStep(B, H, dk, dv, dev, tokens=0)
+
+
+def test_decode_with_the_mean_state_kept_in_bf16(gpu_device):
+    """DecodeStep(mu_dtype=bfloat16): mu is rounded to bf16 once per step, I stays fp32.  Over 64 steps with a slow
+    (f ~ 0.98), a medium and a fast head the outputs stay within the bf16 output bar of the float64 oracle, and the
+    state within 2 % (max-norm) of the oracle's; the first step equals the fp32-state step exactly (same inputs
+    after mu_to_cache)."""
+    from palimpsa_amd.ops.palimpsa import DecodeStep, mu_from_cache, mu_to_cache
+    B, H, dk, dv, steps = 3, 3, 64, 32, 64
+    dev = gpu_device
+    inp = hp.rounded(po.make_inputs(B, steps, H, dk, dv, seed=71), torch.bfloat16)
+    inp["g"] = torch.tensor([0.04, 1.0, 8.0])
+    gen = torch.Generator().manual_seed(72)
+    mu0 = (torch.randn(B, H, dv, dk, generator=gen) * 0.1).to(torch.bfloat16).float()   # exactly representable
+    I0 = 1.0 + torch.rand(B, H, dv, dk, generator=gen)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(inp, mu0=mu0, I0=I0, dtype=torch.float64)
+    d = hp.to_device(inp, dev)
+    outs = {}
+    for name, mu_dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        dec = DecodeStep(B, H, dk, dv, dev, torch.bfloat16, mu_dtype=mu_dtype)
+        buf = {n: torch.empty_like(d[n][:, :1].contiguous()) for n in ("q", "k", "v", "b", "gt")}
+        mu = mu0.to(dev) if mu_dtype == torch.float32 else mu_to_cache(mu0.to(dev))
+        I = I0.to(dev).clone()
+        dec.bind(buf["q"], buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"], mu, I)
+        o_all = []
+        for t in range(steps):
+            for n in buf:
+                buf[n].copy_(d[n][:, t:t + 1])
+            o_all.append(dec.step().clone())
+        outs[name] = (torch.cat(o_all, dim=1), mu if mu_dtype == torch.float32 else mu_from_cache(mu), I)
+        with pytest.raises(ValueError):
+            dec.bind(buf["q"], buf["k"], buf["v"], buf["b"], buf["gt"], d["g"], d["Ip"],
+                     mu.float() if mu_dtype == torch.bfloat16 else mu.bfloat16(), I)
+    assert torch.equal(outs["bf16"][0][:, 0], outs["fp32"][0][:, 0])
+    for name in outs:
+        assert hp.max_abs(outs[name][0], o_ref) <= hp.BF16_OUT_ABS_TOL, name
+    assert hp.max_rel(outs["fp32"][1], mu_ref) <= 1e-4 and hp.max_rel(outs["fp32"][2], I_ref) <= 1e-4
+    assert hp.max_rel(outs["bf16"][1], mu_ref) <= 2e-2
+    assert hp.max_rel(outs["bf16"][2], I_ref) <= 1e-4          # I never sees the rounding of mu
