@@ -80,6 +80,10 @@ __global__ void recurrent_bwd_segoff_kernel(RecBwdArgs a) {
   }
 }
 
+// tokens whose rows are in flight in the token loops of the two kernels below (registers: 2 NPL + 5 per token)
+template <int NPL>
+constexpr int kRecBwdPrefetch = NPL <= 4 ? 3 : 2;
+
 // ------------------------------------------------------------ state checkpoints
 template <typename TIn, int NPL>
 __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
@@ -111,24 +115,46 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
   const TIn* kp = (const TIn*)a.k + (bos * a.Hq + h / (H / a.Hq)) * dk;
   const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv + drow;
   const TIn* bp = (const TIn*)a.b + (bos * H + h) * dv + drow;
-  for (int t = 0; t < len; ++t) {
-    if (t % S == 0) {
-      const int64_t co = (((int64_t)(segbase + t / S) * H + h) * dv + drow) * dk;
+  // the rows of PF tokens are in flight: a token is taken from its register set and the set reloaded at once with
+  // the token PF ahead (always issued, clamped to the last token: the same number of requests in every iteration)
+  constexpr int PF = kRecBwdPrefetch<NPL>;
+  float kb[PF][NPL], vb[PF], bb_[PF], gb[PF];
+  auto load_rows = [&](int t, float* kk, float& vv, float& bb, float& gg) {
 #pragma unroll
-      for (int iv = 0; iv < NV; ++iv) {
-        store_vec<VW>(a.ckM + co + Map::vec_start(j, iv), M + iv * VW);
-        store_vec<VW>(a.ckJ + co + Map::vec_start(j, iv), J + iv * VW);
+    for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
+    vv = to_f32(vp[(int64_t)t * H * dv]);
+    bb = to_f32(bp[(int64_t)t * H * dv]);
+    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+  };
+  if (len > 0) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) load_rows(min(u, len - 1), kb[u], vb[u], bb_[u], gb[u]);
+  }
+  for (int t0 = 0; t0 < len; t0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int t = t0 + u;
+      float kc[NPL];
+#pragma unroll
+      for (int e = 0; e < NPL; ++e) kc[e] = kb[u][e];
+      const float vv = vb[u], bb = bb_[u], gt = gb[u];
+      load_rows(min(t + PF, len - 1), kb[u], vb[u], bb_[u], gb[u]);
+      if (t < len) {
+        if (t % S == 0) {
+          const int64_t co = (((int64_t)(segbase + t / S) * H + h) * dv + drow) * dk;
+#pragma unroll
+          for (int iv = 0; iv < NV; ++iv) {
+            store_vec<VW>(a.ckM + co + Map::vec_start(j, iv), M + iv * VW);
+            store_vec<VW>(a.ckJ + co + Map::vec_start(j, iv), J + iv * VW);
+          }
+        }
+        const float f = fast_exp2(-gt * gh);
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) {
+          M[e] = fmaf(f, M[e], vv * kc[e]);
+          J[e] = fmaf(f, J[e], bb * kc[e] * kc[e]);
+        }
       }
-    }
-    float kc[NPL];
-#pragma unroll
-    for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
-    const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
-    const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
-#pragma unroll
-    for (int e = 0; e < NPL; ++e) {
-      M[e] = fmaf(f, M[e], vv * kc[e]);
-      J[e] = fmaf(f, J[e], bb * kc[e] * kc[e]);
     }
   }
 }
@@ -155,6 +181,26 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
   const TIn* vp = (const TIn*)a.v + vrow;
   const TIn* bp = (const TIn*)a.b + vrow;
   const TIn* dop = (const TIn*)a.d_o + vrow;
+  constexpr int PF = kRecBwdPrefetch<NPL>;
+  auto load_fwd_rows = [&](int t, float* kk, float& vv, float& bb, float& gg) {
+#pragma unroll
+    for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
+    vv = to_f32(vp[(int64_t)t * H * dv]);
+    bb = to_f32(bp[(int64_t)t * H * dv]);
+    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+  };
+  auto load_bwd_rows = [&](int t, float* kk, float* qq, float& vv, float& bb, float& dd, float& dvar, float& gg) {
+#pragma unroll
+    for (int iv = 0; iv < NV; ++iv) {
+      load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
+      load_vec<VW>(qp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), qq + iv * VW);
+    }
+    vv = to_f32(vp[(int64_t)t * H * dv]);
+    bb = to_f32(bp[(int64_t)t * H * dv]);
+    dd = to_f32(dop[(int64_t)t * H * dv]);
+    dvar = has_var ? load_rt(a.d_o_var, vrow + (int64_t)t * H * dv, a.var_bf16) : 0.f;
+    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+  };
   float dMc[NPL], dJc[NPL];   // f_{t+1} dM_{t+1}: what flows into token t from the future
 #pragma unroll
   for (int e = 0; e < NPL; ++e) { dMc[e] = 0.f; dJc[e] = 0.f; }
@@ -171,40 +217,54 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
         load_vec<VW>(a.ckJ + co + Map::vec_start(j, iv), J + iv * VW);
       }
     }
-    // states before every token of the segment
-    for (int jj = 0; jj < cnt; ++jj) {
-      const int t = ts + jj;
+    // states before every token of the segment (rows of PF tokens in flight, see recurrent_bwd_state_kernel)
+    {
+      float kb[PF][NPL], vb[PF], bb_[PF], gb[PF];
 #pragma unroll
-      for (int e = 0; e < NPL; ++e) {
-        stash[(jj * 2 * NPL + e) * 64 + lane] = M[e];
-        stash[(jj * 2 * NPL + NPL + e) * 64 + lane] = J[e];
-      }
-      if (jj + 1 < cnt) {
-        float kc[NPL];
+      for (int u = 0; u < PF; ++u) load_fwd_rows(ts + min(u, cnt - 1), kb[u], vb[u], bb_[u], gb[u]);
+      for (int j0 = 0; j0 < cnt; j0 += PF) {
 #pragma unroll
-        for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
-        const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
-        const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
+        for (int u = 0; u < PF; ++u) {
+          const int jj = j0 + u;
+          float kc[NPL];
 #pragma unroll
-        for (int e = 0; e < NPL; ++e) {
-          M[e] = fmaf(f, M[e], vv * kc[e]);
-          J[e] = fmaf(f, J[e], bb * kc[e] * kc[e]);
+          for (int e = 0; e < NPL; ++e) kc[e] = kb[u][e];
+          const float vv = vb[u], bb = bb_[u], gt = gb[u];
+          load_fwd_rows(ts + min(jj + PF, cnt - 1), kb[u], vb[u], bb_[u], gb[u]);
+          if (jj < cnt) {
+#pragma unroll
+            for (int e = 0; e < NPL; ++e) {
+              stash[(jj * 2 * NPL + e) * 64 + lane] = M[e];
+              stash[(jj * 2 * NPL + NPL + e) * 64 + lane] = J[e];
+            }
+            if (jj + 1 < cnt) {
+              const float f = fast_exp2(-gt * gh);
+#pragma unroll
+              for (int e = 0; e < NPL; ++e) {
+                M[e] = fmaf(f, M[e], vv * kc[e]);
+                J[e] = fmaf(f, J[e], bb * kc[e] * kc[e]);
+              }
+            }
+          }
         }
       }
     }
-    // reverse over the tokens of the segment
-    for (int jj = cnt - 1; jj >= 0; --jj) {
-      const int t = ts + jj;
+    // reverse over the tokens of the segment, rows of PF tokens in flight (token cnt-1-r in round r)
+    float rk[PF][NPL], rq[PF][NPL], rv[PF], rb[PF], rdo[PF], rdv[PF], rg[PF];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) load_bwd_rows(ts + max(cnt - 1 - u, 0), rk[u], rq[u], rv[u], rb[u], rdo[u], rdv[u], rg[u]);
+    for (int r0 = 0; r0 < cnt; r0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int jj = cnt - 1 - (r0 + u);
       float kc[NPL], qc[NPL];
 #pragma unroll
-      for (int iv = 0; iv < NV; ++iv) {
-        load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kc + iv * VW);
-        load_vec<VW>(qp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), qc + iv * VW);
-      }
-      const float vv = to_f32(vp[(int64_t)t * H * dv]), bb = to_f32(bp[(int64_t)t * H * dv]);
-      const float dov = scale * to_f32(dop[(int64_t)t * H * dv]);
-      const float dvv = has_var ? scale * load_rt(a.d_o_var, vrow + (int64_t)t * H * dv, a.var_bf16) : 0.f;
-      const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
+      for (int e = 0; e < NPL; ++e) { kc[e] = rk[u][e]; qc[e] = rq[u][e]; }
+      const float vv = rv[u], bb = rb[u], dov = scale * rdo[u], dvv = scale * rdv[u], gt = rg[u];
+      load_bwd_rows(ts + max(jj - PF, 0), rk[u], rq[u], rv[u], rb[u], rdo[u], rdv[u], rg[u]);
+      if (jj < 0) continue;
+      const int t = ts + jj;
+      const float f = fast_exp2(-gt * gh);
       float dqp[NPL], dkp[NPL];
       float dvs = 0.f, dbs = 0.f, dls = 0.f;
 #pragma unroll
@@ -254,6 +314,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
           store_vec<VW>(a.pdk + po + Map::vec_start(j, iv), dkp + iv * VW);
         }
       }
+    }
     }
   }
   // what reaches the initial state: dM_0 = f_1 dM_1

@@ -91,7 +91,12 @@ __device__ __forceinline__ void store_n_stream(T* p, const float* in) {
   }
 }
 
-template <typename TIn, int NPL, int RD, bool MU16>
+// PF = tokens whose rows are in flight.  PF = 1 (decode): the next token's rows are requested while the current one
+// is processed.  A long token-serial run is bound by the latency of those requests (0.3-0.6 us per token against
+// 0.1-0.2 us of arithmetic), so it keeps PF tokens in registers: a token is processed from its set and the set is
+// reloaded at once with the token PF ahead (always issued, clamped to the last token, so that the number of
+// requests in flight is the same in every iteration and the compiler can wait for exactly the oldest set).
+template <typename TIn, int NPL, int RD, bool MU16, int PF>
 __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
   using Map = NMap<NPL, MU16>;
   constexpr int VW = Map::VW;
@@ -160,7 +165,6 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
   const int64_t gt_base = bos * H + h;
   const int64_t var_base = (bos * H + h) * dv;
 
-  float kc[NPL], qc[NPL], vc[RD], bc[RD], gtc;
   auto load_token = [&](int t, float* kk_, float* qq_, float* vv_, float* bb_, float& gt_) {
     const int64_t off_k = (int64_t)t * Hq * dk;
     const int64_t off_v = (int64_t)t * H * dv;
@@ -176,13 +180,8 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
     }
     gt_ = load_gate(a.gt, gt_base + (int64_t)t * H, a.gate_bf16);
   };
-
-  if (T > 0) load_token(0, kc, qc, vc, bc, gtc);
-  for (int t = 0; t < T; ++t) {
-    float kn[NPL], qn[NPL], vn[RD], bn[RD], gtn = 0.f;
-    const bool more = (t + 1 < T);
-    if (more) load_token(t + 1, kn, qn, vn, bn, gtn);
-
+  // one token: state update and outputs from the token's rows
+  auto token = [&](int t, const float* kc, const float* qc, const float* vc, const float* bc, float gtc) {
     const float f = fast_exp2(-gtc * gh);
     float kk[NPL];
 #pragma unroll
@@ -205,12 +204,41 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
         if (j == 0) store_rt(a.o_var, var_base + (int64_t)t * H * dv + drow[rr], accv, a.var_bf16);
       }
     }
-    if (more) {
+  };
+
+  if constexpr (PF == 1) {
+    float kc[NPL], qc[NPL], vc[RD], bc[RD], gtc;
+    if (T > 0) load_token(0, kc, qc, vc, bc, gtc);
+    for (int t = 0; t < T; ++t) {
+      float kn[NPL], qn[NPL], vn[RD], bn[RD], gtn = 0.f;
+      const bool more = (t + 1 < T);
+      if (more) load_token(t + 1, kn, qn, vn, bn, gtn);
+      token(t, kc, qc, vc, bc, gtc);
+      if (more) {
 #pragma unroll
-      for (int e = 0; e < NPL; ++e) { kc[e] = kn[e]; qc[e] = qn[e]; }
+        for (int e = 0; e < NPL; ++e) { kc[e] = kn[e]; qc[e] = qn[e]; }
 #pragma unroll
-      for (int rr = 0; rr < RD; ++rr) { vc[rr] = vn[rr]; bc[rr] = bn[rr]; }
-      gtc = gtn;
+        for (int rr = 0; rr < RD; ++rr) { vc[rr] = vn[rr]; bc[rr] = bn[rr]; }
+        gtc = gtn;
+      }
+    }
+  } else if (T > 0) {
+    float kb[PF][NPL], qb[PF][NPL], vb[PF][RD], bb[PF][RD], gb[PF];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) load_token(min(u, T - 1), kb[u], qb[u], vb[u], bb[u], gb[u]);
+    for (int t0 = 0; t0 < T; t0 += PF) {
+#pragma unroll
+      for (int u = 0; u < PF; ++u) {
+        const int t = t0 + u;
+        float kc[NPL], qc[NPL], vc[RD], bc[RD];
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) { kc[e] = kb[u][e]; qc[e] = qb[u][e]; }
+#pragma unroll
+        for (int rr = 0; rr < RD; ++rr) { vc[rr] = vb[u][rr]; bc[rr] = bb[u][rr]; }
+        const float gtc = gb[u];
+        load_token(min(t + PF, T - 1), kb[u], qb[u], vb[u], bb[u], gb[u]);
+        if (t < T) token(t, kc, qc, vc, bc, gtc);
+      }
     }
   }
 
@@ -238,13 +266,18 @@ template <typename TIn, int NPL>
 static int launch_npl(const RecArgs& a, int rd, hipStream_t s) {
   const int64_t blocks = (int64_t)a.n_seqs * a.H * (a.dv / (4 * rd));
   if (blocks > 0x7fffffff) return PAL_E_DIM;
+  // tokens in flight of a long run: as many as the registers of a wave take without cutting the occupancy it needs
+  constexpr int PFL = NPL <= 4 ? 4 : (NPL <= 8 ? 3 : 2);
+  const bool serial = a.T > 4;
   if (a.flags & PAL_FLAG_STATE_MU_BF16) {
     // the bf16 cache format of mu is a decode format: the small-wave mapping only
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, true>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, true, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
   } else if (rd == 4) {
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 4, false>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 4, false, PFL>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+  } else if (serial) {
+    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, false, PFL>), dim3((unsigned)blocks), dim3(64), 0, s, a);
   } else {
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, false>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, false, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
   }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
