@@ -38,6 +38,18 @@ __device__ __forceinline__ float load_gate(const void* p, int64_t i, int is_bf16
   return is_bf16 ? (float)((const bf16_t*)p)[i] : ((const float*)p)[i];
 }
 
+// the same in two steps for loops that keep several requests in flight: now the aligned 32-bit word that holds the
+// element (one request of the same kind for both storage types, so that no wait is forced where the two would
+// meet), later the value from the word
+__device__ __forceinline__ unsigned load_gate_word(const void* p, int64_t i, int is_bf16) {
+  const int64_t byte = is_bf16 ? 2 * i : 4 * i;
+  return *(const unsigned*)((const char*)p + (byte & ~(int64_t)3));
+}
+__device__ __forceinline__ float gate_value(unsigned word, int64_t i, int is_bf16) {
+  const unsigned bits = is_bf16 ? ((i & 1) ? (word & 0xffff0000u) : (word << 16)) : word;
+  return __builtin_bit_cast(float, bits);
+}
+
 // store to an output whose element type is chosen at run time
 __device__ __forceinline__ void store_rt(void* p, int64_t i, float x, int is_bf16) {
   if (is_bf16) ((bf16_t*)p)[i] = (bf16_t)x;

@@ -96,7 +96,7 @@ __device__ __forceinline__ void store_n_stream(T* p, const float* in) {
 // 0.1-0.2 us of arithmetic), so it keeps PF tokens in registers: a token is processed from its set and the set is
 // reloaded at once with the token PF ahead (always issued, clamped to the last token, so that the number of
 // requests in flight is the same in every iteration and the compiler can wait for exactly the oldest set).
-template <typename TIn, int NPL, int RD, bool MU16, int PF>
+template <typename TIn, int NPL, int RD, bool MU16, int PF, bool HAS_VAR>
 __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
   using Map = NMap<NPL, MU16>;
   constexpr int VW = Map::VW;
@@ -124,7 +124,6 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
   const float gh = a.g[h] * kLog2e;
   const float Ip = a.Ip[h];
   const float scale = a.scale;
-  const bool has_var = a.flags & PAL_FLAG_HAS_VAR;
   constexpr bool mu16 = MU16;   // mu kept in bf16 between calls (a cache format of decode)
 
   int drow[RD];
@@ -156,33 +155,46 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
       for (int e = 0; e < NPL; ++e) { M[rr][e] = 0.f; J[rr][e] = 0.f; }
   }
 
+  // Addresses of a token's rows = a wave-uniform pointer that moves by one token at a time + a constant 32-bit lane
+  // offset, so that the per-token address work is a few scalar additions (a long token-serial run is bound by the
+  // number of instructions one wave issues per token).
   const int Hq = a.Hq, hq = h / (H / Hq);
-  const TIn* qp = (const TIn*)a.q + (bos * Hq + hq) * dk;
+  const int64_t step_k = (int64_t)Hq * dk, step_v = (int64_t)H * dv;
+  const TIn* qp = (const TIn*)a.q + (bos * Hq + hq) * dk;     // rows of the next token to request
   const TIn* kp = (const TIn*)a.k + (bos * Hq + hq) * dk;
   const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv;
   const TIn* bp = (const TIn*)a.b + (bos * H + h) * dv;
-  TIn* op = (TIn*)a.o + (bos * H + h) * dv;
-  const int64_t gt_base = bos * H + h;
-  const int64_t var_base = (bos * H + h) * dv;
+  int64_t gt_i = bos * H + h;
+  TIn* op = (TIn*)a.o + (bos * H + h) * dv;                   // output row of the token being processed
+  int64_t var_i = (bos * H + h) * dv;
+  int64_t go_i = gt_i;                                        // gate element of the token being processed
+  unsigned lane_k[NV], lane_v[RD];   // byte offsets: base pointer in scalar registers + 32-bit lane offset
+#pragma unroll
+  for (int iv = 0; iv < NV; ++iv) lane_k[iv] = (unsigned)Map::vec_start(j, iv) * (unsigned)sizeof(TIn);
+#pragma unroll
+  for (int rr = 0; rr < RD; ++rr) lane_v[rr] = (unsigned)drow[rr] * (unsigned)sizeof(TIn);
+  auto at = [](const TIn* base, unsigned bytes) { return (const TIn*)((const char*)base + bytes); };
 
-  auto load_token = [&](int t, float* kk_, float* qq_, float* vv_, float* bb_, float& gt_) {
-    const int64_t off_k = (int64_t)t * Hq * dk;
-    const int64_t off_v = (int64_t)t * H * dv;
+  // request the rows of the token the pointers stand at and move them on one token (callers never request beyond the
+  // last token of the sequence)
+  auto request = [&](float* kk_, float* qq_, float* vv_, float* bb_, unsigned& gt_) {
 #pragma unroll
     for (int iv = 0; iv < NV; ++iv) {
-      load_n<VW>(kp + off_k + Map::vec_start(j, iv), kk_ + iv * VW);
-      load_n<VW>(qp + off_k + Map::vec_start(j, iv), qq_ + iv * VW);
+      load_n<VW>(at(kp, lane_k[iv]), kk_ + iv * VW);
+      load_n<VW>(at(qp, lane_k[iv]), qq_ + iv * VW);
     }
 #pragma unroll
     for (int rr = 0; rr < RD; ++rr) {
-      vv_[rr] = to_f32(vp[off_v + drow[rr]]);
-      bb_[rr] = to_f32(bp[off_v + drow[rr]]);
+      vv_[rr] = to_f32(*at(vp, lane_v[rr]));
+      bb_[rr] = to_f32(*at(bp, lane_v[rr]));
     }
-    gt_ = load_gate(a.gt, gt_base + (int64_t)t * H, a.gate_bf16);
+    gt_ = load_gate_word(a.gt, gt_i, a.gate_bf16);
+    kp += step_k; qp += step_k; vp += step_v; bp += step_v; gt_i += H;
   };
   // one token: state update and outputs from the token's rows
-  auto token = [&](int t, const float* kc, const float* qc, const float* vc, const float* bc, float gtc) {
-    const float f = fast_exp2(-gtc * gh);
+  auto token = [&](const float* kc, const float* qc, const float* vc, const float* bc, unsigned gt_word) {
+    const float f = fast_exp2(-gate_value(gt_word, go_i, a.gate_bf16) * gh);
+    go_i += H;
     float kk[NPL];
 #pragma unroll
     for (int e = 0; e < NPL; ++e) kk[e] = kc[e] * kc[e];
@@ -195,25 +207,29 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
         J[rr][e] = fmaf(f, J[rr][e], bc[rr] * kk[e]);
         const float rI = fast_rcp(J[rr][e] + Ip);
         acc = fmaf(M[rr][e] * rI, qc[e], acc);
-        if (has_var) accv = fmaf(qc[e] * qc[e], rI, accv);
+        if constexpr (HAS_VAR) accv = fmaf(qc[e] * qc[e], rI, accv);
       }
       acc = row16_sum(acc) * scale;
-      if (j == 0) op[(int64_t)t * H * dv + drow[rr]] = from_f32<TIn>(acc);
-      if (has_var) {
+      if (j == 0) *(TIn*)((char*)op + lane_v[rr]) = from_f32<TIn>(acc);
+      if constexpr (HAS_VAR) {
         accv = row16_sum(accv) * scale;
-        if (j == 0) store_rt(a.o_var, var_base + (int64_t)t * H * dv + drow[rr], accv, a.var_bf16);
+        if (j == 0) store_rt(a.o_var, var_i + drow[rr], accv, a.var_bf16);
       }
     }
+    op += step_v;
+    var_i += step_v;
   };
 
   if constexpr (PF == 1) {
-    float kc[NPL], qc[NPL], vc[RD], bc[RD], gtc;
-    if (T > 0) load_token(0, kc, qc, vc, bc, gtc);
+    float kc[NPL], qc[NPL], vc[RD], bc[RD];
+    unsigned gtc = 0;
+    if (T > 0) request(kc, qc, vc, bc, gtc);
     for (int t = 0; t < T; ++t) {
-      float kn[NPL], qn[NPL], vn[RD], bn[RD], gtn = 0.f;
+      float kn[NPL], qn[NPL], vn[RD], bn[RD];
+      unsigned gtn = 0;
       const bool more = (t + 1 < T);
-      if (more) load_token(t + 1, kn, qn, vn, bn, gtn);
-      token(t, kc, qc, vc, bc, gtc);
+      if (more) request(kn, qn, vn, bn, gtn);
+      token(kc, qc, vc, bc, gtc);
       if (more) {
 #pragma unroll
         for (int e = 0; e < NPL; ++e) { kc[e] = kn[e]; qc[e] = qn[e]; }
@@ -222,22 +238,29 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(RecArgs a) {
         gtc = gtn;
       }
     }
-  } else if (T > 0) {
-    float kb[PF][NPL], qb[PF][NPL], vb[PF][RD], bb[PF][RD], gb[PF];
+  } else {
+    // token t lives in register set t mod PF; it is processed from there and the set requested again for token t + PF
+    float kb[PF][NPL], qb[PF][NPL], vb[PF][RD], bb[PF][RD];
+    unsigned gb[PF];
 #pragma unroll
-    for (int u = 0; u < PF; ++u) load_token(min(u, T - 1), kb[u], qb[u], vb[u], bb[u], gb[u]);
-    for (int t0 = 0; t0 < T; t0 += PF) {
+    for (int u = 0; u < PF; ++u)
+      if (u < T) request(kb[u], qb[u], vb[u], bb[u], gb[u]);
+    // groups of PF tokens that all have a token PF ahead of them: straight-line code, no per-token conditions
+    int t0 = 0;
+    for (; t0 + 2 * PF <= T; t0 += PF) {
 #pragma unroll
       for (int u = 0; u < PF; ++u) {
-        const int t = t0 + u;
-        float kc[NPL], qc[NPL], vc[RD], bc[RD];
+        token(kb[u], qb[u], vb[u], bb[u], gb[u]);
+        request(kb[u], qb[u], vb[u], bb[u], gb[u]);
+      }
+    }
+    // the last tokens (fewer than 2 PF): requests only while there is a token PF ahead
 #pragma unroll
-        for (int e = 0; e < NPL; ++e) { kc[e] = kb[u][e]; qc[e] = qb[u][e]; }
-#pragma unroll
-        for (int rr = 0; rr < RD; ++rr) { vc[rr] = vb[u][rr]; bc[rr] = bb[u][rr]; }
-        const float gtc = gb[u];
-        load_token(min(t + PF, T - 1), kb[u], qb[u], vb[u], bb[u], gb[u]);
-        if (t < T) token(t, kc, qc, vc, bc, gtc);
+    for (int u = 0; u < 2 * PF; ++u) {
+      const int t = t0 + u;
+      if (t < T) {
+        token(kb[u % PF], qb[u % PF], vb[u % PF], bb[u % PF], gb[u % PF]);
+        if (t + PF < T) request(kb[u % PF], qb[u % PF], vb[u % PF], bb[u % PF], gb[u % PF]);
       }
     }
   }
@@ -269,16 +292,23 @@ static int launch_npl(const RecArgs& a, int rd, hipStream_t s) {
   // tokens in flight of a long run: as many as the registers of a wave take without cutting the occupancy it needs
   constexpr int PFL = NPL <= 4 ? 4 : (NPL <= 8 ? 3 : 2);
   const bool serial = a.T > 4;
+  const bool var = a.flags & PAL_FLAG_HAS_VAR;
+#define PAL_REC_LAUNCH(RD_, MU_, PF_)                                                                                     \
+  do {                                                                                                                   \
+    if (var) PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, RD_, MU_, PF_, true>), dim3((unsigned)blocks), dim3(64), 0, s, a); \
+    else PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, RD_, MU_, PF_, false>), dim3((unsigned)blocks), dim3(64), 0, s, a); \
+  } while (0)
   if (a.flags & PAL_FLAG_STATE_MU_BF16) {
     // the bf16 cache format of mu is a decode format: the small-wave mapping only
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, true, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_REC_LAUNCH(1, true, 1);
   } else if (rd == 4) {
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 4, false, PFL>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_REC_LAUNCH(4, false, PFL);
   } else if (serial) {
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, false, PFL>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_REC_LAUNCH(1, false, PFL);
   } else {
-    PAL_TIMED_LAUNCH(kKernRecurrentFwd, s, (recurrent_fwd_kernel<TIn, NPL, 1, false, 1>), dim3((unsigned)blocks), dim3(64), 0, s, a);
+    PAL_REC_LAUNCH(1, false, 1);
   }
+#undef PAL_REC_LAUNCH
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
