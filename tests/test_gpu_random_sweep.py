@@ -25,7 +25,9 @@ def _case(seed):
     packed = rng.random() < 0.5
     if packed:
         n = rng.randint(1, 5)
-        lens = [rng.choice([1, 2, 17, 63, 64, 65, 100, 129, 200]) for _ in range(n)]
+        lens = [rng.choice([0, 1, 2, 17, 63, 64, 65, 100, 129, 200]) for _ in range(n)]
+        if sum(lens) == 0:
+            lens[-1] = 33
         cu = [0]
         for ln in lens:
             cu.append(cu[-1] + ln)
