@@ -340,3 +340,51 @@ def test_runs_on_the_callers_stream(gpu_device):
     for a, b_ in zip(ref, got):
         assert torch.equal(a, b_)
     assert torch.isfinite(total)
+
+
+def test_forward_and_backward_replay_in_a_graph(gpu_device):
+    """chunk_palimpsa forward + backward recorded into a HIP graph (the C ABI allocates nothing, synchronises nothing
+    and records no memset; the wrapper's buffers come from torch's capture-aware allocator): three replays on new
+    input values, with eager work and synchronisations in between, each equal to the eager result."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    dev = gpu_device
+    B, T, H, dk, dv = 2, 200, 2, 64, 64
+    names = ("q", "k", "v", "b", "gt", "g", "Ip")
+
+    def fresh(seed):
+        inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=seed), torch.bfloat16)
+        do = torch.randn(B, T, H, dv, generator=torch.Generator().manual_seed(seed + 1)).to(torch.bfloat16)
+        return hp.to_device(inp, dev), do.to(dev)
+
+    def eager(d, do):
+        leaves = [d[n].clone().requires_grad_(True) for n in names]
+        o = chunk_palimpsa(*leaves, chunk_size=64)
+        return (o.detach(),) + torch.autograd.grad((o.float() * do.float()).sum(), leaves)
+
+    d0, do0 = fresh(400)
+    static = [d0[n].clone().requires_grad_(True) for n in names]
+    static_do = do0.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                                    # warm-up on the capture stream
+            o = chunk_palimpsa(*static, chunk_size=64)
+            torch.autograd.grad((o.float() * static_do.float()).sum(), static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g = chunk_palimpsa(*static, chunk_size=64)
+        grads_g = torch.autograd.grad((o_g.float() * static_do.float()).sum(), static)
+    for seed in (410, 420, 430):
+        d, do = fresh(seed)
+        ref = eager(d, do)                                    # eager work between the replays
+        with torch.no_grad():
+            for x, n in zip(static, names):
+                x.copy_(d[n])
+            static_do.copy_(do)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (o_g,) + tuple(grads_g)
+        for a_, b_, n in zip(got, ref, ("o",) + names):
+            assert torch.equal(a_, b_), (seed, n)
