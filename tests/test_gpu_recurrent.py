@@ -279,10 +279,13 @@ def test_bound_decode_step_matches_entry_point_and_replays_in_a_graph(gpu_device
         DecodeStep(B, H, 40, dv, dev)
 
 
-def test_bound_decode_step_with_several_tokens_per_step(gpu_device):
-    """A bound step over blocks of 3 tokens equals the same tokens one at a time (state in place)."""
+@pytest.mark.parametrize("k", [3, 5, 7, 8, 13])
+def test_bound_decode_step_with_several_tokens_per_step(gpu_device, k):
+    """A bound step over blocks of k tokens equals the same tokens one at a time (state in place); k <= 4 takes the
+    decode form of the kernel, longer blocks the form that keeps the rows of several tokens in flight (its group and
+    tail loops at every remainder)."""
     from palimpsa_amd.ops.palimpsa import DecodeStep
-    B, H, dk, dv, blocks, k = 4, 2, 32, 48, 3, 3
+    B, H, dk, dv, blocks = 4, 2, 32, 48, 3
     dev = gpu_device
     inp = hp.rounded(po.make_inputs(B, blocks * k, H, dk, dv, seed=71), torch.bfloat16)
     d = hp.to_device(inp, dev)
