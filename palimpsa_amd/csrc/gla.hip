@@ -336,6 +336,307 @@ static int launch_gla_tile_dt(const GlaTileArgs& A, int dtype, GlaRole role, hip
   return dtype == PAL_DTYPE_BF16 ? launch_gla_tile<bf16_t>(A, role, s) : launch_gla_tile<float>(A, role, s);
 }
 
+// ------------------------------------------------------------------ the three input gradients in one kernel
+// For head dims up to 64 and bf16 rows the tiles of q, k, v, dO of a (tile, head) and its two states fit into LDS
+// together (76 KB, two workgroups per compute unit), so one workgroup forms dq, dv and dk in turn with the products
+// of gla_tile_kernel (same roles, same operand maps) from one copy of the rows: 48 KB read and 24 KB written per
+// (tile, head) instead of 3 x 41 KB moved by three launches, and the tile states are read as 16-byte pieces and
+// transposed on their way out of LDS instead of by 2-byte requests to memory.  The rows W of the two dot
+// products (q for q.dq, k for k.dk) come from the same tiles.
+struct GlaBwdTileArgs {
+  ChunkArgs c;                  // T, H, tiles, gate (gt, g), scale, dk, dv
+  const void *q, *k, *v, *d_o;  // rows [token][H][dk | dv]
+  const bf16_t *S, *G;          // tile-start states and gradients of the tile-end states, [tile][H][dv][dk]
+  void *dq, *dk, *dv;
+  float *qdq, *kdk;             // [H][tokens]
+  int64_t n_tokens;
+};
+
+constexpr int kFR = 72;   // row stride (bf16) of every tile of the fused kernel (rows of up to 64 entries)
+
+// Eight waves per workgroup (four per SIMD with two workgroups on a compute unit): a role's scores are formed by two
+// waves per token block (one per half of the score operand), its output by two waves per block of 16 columns (token
+// blocks {0, 2} and {1, 3}: the same number of matrix instructions in both causal directions).
+// DKC, DVC: the head dims when they are known at compile time (loops unrolled, index arithmetic folded), else 0.
+template <typename TIn, int DKC, int DVC>
+__global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) {
+  static_assert(sizeof(TIn) == 2, "bf16 rows");
+  extern __shared__ float smem[];
+  const ChunkArgs& a = A.c;
+  const int H = a.H, dk = DKC ? DKC : a.dk, dv = DVC ? DVC : a.dv;
+  float* sC = smem;                          // [64] running log2 decay inside the tile
+  float* sDot = sC + kC;                     // [8][64] partial dot products of the waves
+  bf16_t* sQ = (bf16_t*)(sDot + 8 * kC);     // row tiles [64 tokens][kFR], zero beyond the tile's tokens and widths
+  bf16_t* sK = sQ + kC * kFR;
+  bf16_t* sV = sK + kC * kFR;
+  bf16_t* sDo = sV + kC * kFR;
+  bf16_t* sS = sDo + kC * kFR;               // state tiles [64 value rows][kFR], zero beyond dv x dk
+  bf16_t* sG = sS + kC * kFR;
+  bf16_t* sZT = sG + kC * kFR;               // [64 columns][kVT]: the mixed rows of the current role, token index fastest
+  bf16x8* sP = (bf16x8*)(sZT + kC * kVT);    // [4 token blocks][2][64 lanes] score operands; then the output tile [64][kFR]
+  TIn* sOut = (TIn*)sP;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // A workgroup walks over (tile, head) items; the rows and states of the next item are requested into registers
+  // before the products of the current one start, so that their latency is covered by that work.
+  // Waves 0-3: tokens 2 sp, 2 sp + 1, columns [8 c8, 8 c8 + 8) of q and k and two rows of S; waves 4-7: of v, dO and G.
+  const int sp = (tid & 255) >> 3, c8 = tid & 7;
+  const bool upper = w >= 4;
+  const int64_t n_items = (int64_t)a.total_chunks * H;
+  bf16x8 ra[2], rb[2], rc[2];
+  unsigned gate_n = 0u;   // the token's gate as stored (wave 0)
+  float gh_n = 0.f;       // the head's decay rate g (wave 0)
+  // (tile, head) of an item and the tile's place in the token axis.  With a tile table the two words are requested
+  // one item before they are needed (meta_request) and range-checked when they are (meta_finish, as chunk_lookup).
+  struct Meta { int cidx, h, t0, clen; };
+  // A load from an address that is the same in every lane is turned into a scalar value right behind the load, which
+  // makes the wave wait for it there (and for every request issued before it).  The loads that are meant to stay in
+  // flight get an offset of zero that the compiler cannot see through; their values are made scalar where they are used.
+  int lane_zero = 0;
+  asm volatile("" : "+v"(lane_zero));
+  int tab_t0 = 0, tab_clen = 0;   // words of the tile table for the item after the next (written by loads only)
+  int cidx_nn = 0, h_nn = 0;
+  auto meta_request = [&](int64_t item) {
+    // the item is the same for every lane
+    cidx_nn = __builtin_amdgcn_readfirstlane((int)(item / H));
+    h_nn = __builtin_amdgcn_readfirstlane((int)(item - (int64_t)cidx_nn * H));
+    if (a.chunk_table) {
+      const int32_t* row = a.chunk_table + 4 * (int64_t)cidx_nn;
+      tab_t0 = row[1 + lane_zero];
+      tab_clen = row[2 + lane_zero];
+    }
+  };
+  auto meta_finish = [&](Meta& m) {
+    m.cidx = cidx_nn;
+    m.h = h_nn;
+    if (a.chunk_table) {
+      m.t0 = min(max(__builtin_amdgcn_readfirstlane(tab_t0), 0), a.T - 1);
+      m.clen = min(max(__builtin_amdgcn_readfirstlane(tab_clen), 0), min(kC, a.T - m.t0));
+    } else {
+      const int per = (a.T + kC - 1) / kC;
+      const int seq = m.cidx / per, cis = m.cidx - seq * per;
+      m.t0 = seq * a.T + cis * kC;
+      m.clen = min(kC, a.T - cis * kC);
+    }
+  };
+  auto request = [&](const Meta& m) {
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const TIn* pa = (const TIn*)(upper ? A.v : A.q);
+    const TIn* pb = (const TIn*)(upper ? A.d_o : A.k);
+    const bf16_t* pc = upper ? A.G : A.S;
+    const int d = upper ? dv : dk;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int s = 2 * sp + u;
+      const bool on = s < m.clen && 8 * c8 < d;
+      const int64_t row = ((int64_t)(m.t0 + (on ? s : 0)) * H + m.h) * d + (on ? 8 * c8 : 0);
+      ra[u] = on ? *(const bf16x8*)(pa + row) : zero;
+      rb[u] = on ? *(const bf16x8*)(pb + row) : zero;
+      const bool ons = s < dv && 8 * c8 < dk;
+      const int64_t so = ((int64_t)m.cidx * H + m.h) * dv * dk + (int64_t)(ons ? s : 0) * dk + (ons ? 8 * c8 : 0);
+      rc[u] = ons ? *(const bf16x8*)(pc + so) : zero;
+    }
+    if (w == 0) {
+      if (lane < m.clen) gate_n = load_gate_word(a.gt, (int64_t)(m.t0 + lane) * H + m.h, a.gate_bf16);
+      gh_n = a.g[m.h + lane_zero];
+    }
+  };
+  int64_t item = blockIdx.x;
+  const int64_t stride = gridDim.x;
+  if (item >= n_items) return;
+  Meta m_next;
+  meta_request(item);
+  meta_finish(m_next);
+  request(m_next);
+  if (item + stride < n_items) meta_request(item + stride);
+  for (;;) {
+  // the requested item becomes the current one: its tiles go to LDS (every read of the previous item's is behind a barrier)
+  const int h = m_next.h, t0 = m_next.t0, clen = m_next.clen;
+  if (w == 0) {
+    const float gt = (lane < clen) ? gate_value(gate_n, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
+    sC[lane] = wave_inclusive_scan(-gt * (gh_n * kLog2e), lane);
+  }
+  {
+    bf16_t* ta = upper ? sV : sQ;
+    bf16_t* tb = upper ? sDo : sK;
+    bf16_t* tc = upper ? sG : sS;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int o = (2 * sp + u) * kFR + 8 * c8;
+      *(bf16x8*)&ta[o] = ra[u];
+      *(bf16x8*)&tb[o] = rb[u];
+      *(bf16x8*)&tc[o] = rc[u];
+    }
+    if (!upper) {   // first role (dq) mixes the rows of k: token pair sp, one 32-bit word per column
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *(bf16x2*)&sZT[(8 * c8 + e) * kVT + 2 * sp] = bf16x2{rb[0][e], rb[1][e]};
+    }
+  }
+  __syncthreads();
+  const bool more = item + stride < n_items;
+  if (more) {
+    meta_finish(m_next);
+    request(m_next);
+    if (item + 2 * stride < n_items) meta_request(item + 2 * stride);
+  }
+
+  const float scale = a.scale;
+  // One role of gla_tile_kernel on the tiles in LDS.  sX, sY: rows of the scores (width dc); sSt: state tile read
+  // straight (rows = output columns) or transposed; sW: rows of the dot product or null; zn: rows the NEXT role mixes.
+  auto role = [&](auto rev_c, auto st_c, const bf16_t* sX, const bf16_t* sY, const bf16_t* sSt, const bf16_t* sW,
+                  const bf16_t* zn, int dc, int de, void* out, float* dot_out) {
+    constexpr bool REVERSE = decltype(rev_c)::value, STATE_T = decltype(st_c)::value;
+    const int KS = (dc + 31) >> 5, n_eb = de >> 4;
+    auto x_operand = [&](int xb, int ks) { return *(const bf16x8*)(sX + (16 * xb + i) * kFR + 8 * g + 32 * ks); };
+    // ---- scores of token block w / 2 against the blocks yb = 2 p + (w & 1) on its causal side: one half of each of
+    //      the block's two score operands
+    {
+      const int tb = w >> 1, half = w & 1;
+      f32x4 accS[2];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) accS[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 Xo = x_operand(tb, ks);
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const int yb = 2 * p + half;
+          if (REVERSE ? yb >= tb : yb <= tb)
+            accS[p] = mfma16(*(const bf16x8*)(sY + (16 * yb + i) * kFR + 8 * g + 32 * ks), Xo, accS[p]);
+        }
+      }
+      const float cx = sC[16 * tb + i];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const int yb = 2 * p + half;
+        const f32x4 cy = *(const f32x4*)&sC[16 * yb + 4 * g];
+        float val[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const bool side = REVERSE ? yb >= tb : yb <= tb;
+          const bool live = side && (yb != tb || (REVERSE ? 4 * g + r >= i : 4 * g + r <= i));
+          val[r] = live ? accS[p][r] * fast_exp2(REVERSE ? cy[r] - cx : cx - cy[r]) : 0.f;
+        }
+        store_vec<4>((bf16_t*)&sP[(tb * 2 + p) * 64 + lane] + 4 * half, val);
+      }
+    }
+    __syncthreads();
+    // ---- output columns [16 (w / 2), 16 (w / 2) + 16) for the token blocks xh, xh + 2 (xh = w & 1)
+    const int eb = min(w >> 1, n_eb - 1);          // a wave past the last block repeats it (not stored)
+    const bool valid = (w >> 1) < n_eb;
+    const int xh = w & 1;
+    f32x4 acc[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < KS; ++ks) {
+      bf16x8 Sa;
+      if constexpr (STATE_T) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) Sa[j] = sSt[(32 * ks + 8 * g + j) * kFR + 16 * eb + i];
+      } else {
+        Sa = *(const bf16x8*)(sSt + (16 * eb + i) * kFR + 32 * ks + 8 * g);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) acc[u] = mfma16(Sa, x_operand(xh + 2 * u, ks), acc[u]);
+    }
+    const bf16_t* zrow = sZT + (16 * eb + i) * kVT + 4 * g;
+    bf16x8 Za[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const bf16x4 lo = *(const bf16x4*)(zrow + 32 * p), hi = *(const bf16x4*)(zrow + 32 * p + 16);
+      Za[p] = bf16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+    float dot[2] = {0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int xb = xh + 2 * u;
+      const float cx = sC[16 * xb + i];
+      const float wx = fast_exp2(REVERSE ? sC[kC - 1] - cx : cx);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[u][r] *= wx;
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+        if ((REVERSE ? 2 * p + 1 >= xb : 2 * p <= xb)) acc[u] = mfma16(Za[p], sP[(xb * 2 + p) * 64 + lane], acc[u]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[u][r] *= scale;
+      if (sW && valid) {
+        const bf16x4 wv = *(const bf16x4*)(sW + (16 * xb + i) * kFR + 16 * eb + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dot[u] = fmaf((float)wv[r], acc[u][r], dot[u]);
+      }
+    }
+    __syncthreads();   // every wave has its scores and mixed rows: the two areas are free
+    if (sW) {
+      // lanes of row g get the sum over the four rows of argument g: token block g of this wave, or zero
+      const float d0 = dot[0], d1 = dot[1];
+      sDot[w * kC + lane] = rows4_sum_x4(xh ? 0.f : d0, xh ? d0 : 0.f, xh ? 0.f : d1, xh ? d1 : 0.f);   // lane = token
+    }
+    if (valid) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        store_vec<4>(sOut + (16 * (xh + 2 * u) + i) * kFR + 16 * eb + 4 * g, (const float*)&acc[u]);
+    }
+    if (zn) {
+      // token pair zp, columns [8 zc + 4 ze, 8 zc + 4 ze + 4) of the next role's mixed rows
+      const int zp = tid >> 4, zc = (tid >> 1) & 7, ze = tid & 1;
+      const bf16x4 z0 = *(const bf16x4*)(zn + (2 * zp) * kFR + 8 * zc + 4 * ze);
+      const bf16x4 z1 = *(const bf16x4*)(zn + (2 * zp + 1) * kFR + 8 * zc + 4 * ze);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) *(bf16x2*)&sZT[(8 * zc + 4 * ze + e) * kVT + 2 * zp] = bf16x2{z0[e], z1[e]};
+    }
+    __syncthreads();
+    if (sW && w == 0 && lane < clen) {
+      float tot = 0.f;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) tot += sDot[x * kC + lane];
+      dot_out[(int64_t)h * A.n_tokens + t0 + lane] = tot;
+    }
+    {
+      const int per_row = de >> 3;
+      TIn* obase = (TIn*)out + ((int64_t)t0 * H + h) * de;
+      for (int idx = tid; idx < clen * per_row; idx += 512) {
+        const int x = idx / per_row, c = idx - x * per_row;
+        *(f32x4*)(obase + (int64_t)x * H * de + 8 * c) = *(const f32x4*)(sOut + x * kFR + 8 * c);
+      }
+    }
+    __syncthreads();   // the output tile has been read: the next role may write its scores
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  // dq: X = dO, Y = v, mixes k, tile-start state transposed, q . dq on the side; then the rows of dO for dv
+  role(F_{}, T_{}, sDo, sV, sS, sQ, sDo, dv, dk, A.dq, A.qdq);
+  // dv: X = k, Y = q, mixes dO, gradient of the tile-end state, reverse; then the rows of q for dk
+  role(T_{}, F_{}, sK, sQ, sG, (const bf16_t*)nullptr, sQ, dk, dv, A.dv, (float*)nullptr);
+  // dk: X = v, Y = dO, mixes q, gradient of the tile-end state transposed, reverse, k . dk on the side
+  role(T_{}, T_{}, sV, sDo, sG, sK, (const bf16_t*)nullptr, dv, dk, A.dk, A.kdk);
+  if (!more) break;
+  item += stride;
+  }
+}
+
+static bool gla_bwd_tile_applies(const PalDims* d) {
+  return d->dtype == PAL_DTYPE_BF16 && d->dk <= 64 && d->dv <= 64;
+}
+
+static int launch_gla_bwd_tile(const GlaBwdTileArgs& A, hipStream_t s) {
+  const size_t lds = sizeof(float) * (kC + 8 * kC) + sizeof(bf16_t) * (size_t)kC * (6 * kFR + kVT + kFR);
+  const int64_t items = (int64_t)A.c.total_chunks * A.c.H;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      cus <= 0)
+    cus = 256;
+  const int64_t resident = 2 * (int64_t)cus;   // two workgroups per compute unit, each walks its items
+  const int64_t blocks = items < resident ? items : resident;
+  if (A.c.dk == 64 && A.c.dv == 64) {
+    if (int rc = allow_lds((const void*)&gla_bwd_tile_kernel<bf16_t, 64, 64>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernGlaBwdTile, s, (gla_bwd_tile_kernel<bf16_t, 64, 64>), dim3((unsigned)blocks), dim3(512), lds, s, A);
+  } else {
+    if (int rc = allow_lds((const void*)&gla_bwd_tile_kernel<bf16_t, 0, 0>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernGlaBwdTile, s, (gla_bwd_tile_kernel<bf16_t, 0, 0>), dim3((unsigned)blocks), dim3(512), lds, s, A);
+  }
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
 // argument checks shared by the forward and the backward entry points
 static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   int rc = pal_validate_dims(d);
@@ -571,6 +872,15 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
     PAL_HIP_LAUNCH_CHECK();
     }
   }
+  if (gla_bwd_tile_applies(d)) {
+    GlaBwdTileArgs F{};
+    F.c = a;
+    F.q = t->q; F.k = t->k; F.v = t->v; F.d_o = gr->d_o;
+    F.S = (const bf16_t*)t->chunk_I; F.G = g_tiles;
+    F.dq = gr->dq; F.dk = gr->dk; F.dv = gr->dv; F.qdq = qdq; F.kdk = kdk;
+    F.n_tokens = (int64_t)d->batch * d->seq_len;
+    if (int rc = launch_gla_bwd_tile(F, s)) return rc;
+  } else {
   GlaTileArgs A{};
   A.c = a;
   A.n_tokens = (int64_t)d->batch * d->seq_len;
@@ -586,6 +896,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   A.X = t->v; A.Y = gr->d_o; A.Z = t->q; A.St = g_tiles; A.out = gr->dk; A.W = t->k; A.dot = kdk;
   A.dc = d->dv; A.de = d->dk;
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDk, s)) return rc;
+  }
   {
     const int64_t blocks = (int64_t)d->n_seqs * d->n_heads;
     PAL_TIMED_LAUNCH(kKernGlaBwdGate, s, gla_bwd_gate_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, qdq, kdk, gr->dgt,

@@ -29,6 +29,7 @@ enum KernelId {
   kKernGlaRecurrentFwd,
   kKernChunkStates,
   kKernGlaBwdStates,
+  kKernGlaBwdTile,
   kKernCount
 };
 

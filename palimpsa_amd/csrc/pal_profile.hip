@@ -53,7 +53,7 @@ static const char* kNames[kKernCount] = {
     "chunk_bwd_head_reduce_kernel", "recurrent_bwd_state_kernel", "recurrent_bwd_kernel", "gla_out_kernel",
     "gla_dq_kernel", "gla_dv_kernel", "gla_dk_kernel", "gla_bwd_scan_kernel", "gla_bwd_gate_kernel",
     "prologue_fwd_kernel", "prologue_bwd_kernel", "epilogue_fwd_kernel", "epilogue_bwd_kernel",
-    "gla_recurrent_fwd_kernel", "chunk_states_kernel", "gla_bwd_states_kernel"};
+    "gla_recurrent_fwd_kernel", "chunk_states_kernel", "gla_bwd_states_kernel", "gla_bwd_tile_kernel"};
 
 }  // namespace pal
 

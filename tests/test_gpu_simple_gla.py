@@ -570,3 +570,43 @@ def test_packed_pretraining_batch_full_size(gpu_device):
     o_p.backward(do.to(dev))
     for name, x, r in zip(("q", "k", "v", "g"), leaves, ref):
         assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
+
+
+def test_backward_packed_batch_walked_by_resident_workgroups(gpu_device):
+    """Head dims up to 64 take the kernel that forms dq, dk, dv from one copy of the rows; its workgroups walk over
+    several (tile, head) items each and request the tile table two items ahead.  8192 tokens in ragged documents
+    (tiles of 1 to 64 tokens, 2000 items): gradients against the Palimpsa kernels on b = 0, Ip = 1 and, for three
+    documents, against the closed form."""
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    H, dk, dv = 12, 64, 48
+    lens, tot, j = [], 0, 0
+    while tot < 8192:
+        ln = min(1 + (j * 977) % 700, 8192 - tot)
+        lens.append(ln)
+        tot += ln
+        j += 1
+    cu = [0]
+    for ln in lens:
+        cu.append(cu[-1] + ln)
+    q, k, v, g, _ = _inputs(1, cu[-1], H, dk, dv, 95)
+    gen = torch.Generator().manual_seed(96)
+    do = torch.randn(1, cu[-1], H, dv, generator=gen).bfloat16()
+    dev = gpu_device
+    cu_d = torch.tensor(cu, device=dev, dtype=torch.int32)
+    leaves = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    o, _ = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3], cu_seqlens=cu_d)
+    o.backward(do.to(dev))
+    ref = [x.to(dev).clone().requires_grad_(True) for x in (q, k, v, g)]
+    ones = torch.ones(H, device=dev)
+    o_p = chunk_palimpsa(ref[0], ref[1], ref[2], torch.zeros_like(ref[2]), -ref[3], ones, ones, cu_seqlens=cu_d)
+    o_p.backward(do.to(dev))
+    for name, x, r in zip(("q", "k", "v", "g"), leaves, ref):
+        assert hp.max_rel(x.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
+    for jdoc in (0, len(lens) // 2, len(lens) - 1):
+        sl = slice(cu[jdoc], cu[jdoc + 1])
+        rl = [x[:, sl].double().clone().requires_grad_(True) for x in (q, k, v, g)]
+        o_ref, _ = _closed_form(*rl, dk ** -0.5)
+        (o_ref * do[:, sl].double()).sum().backward()
+        for name, x, r in zip(("q", "k", "v", "g"), leaves, rl):
+            assert hp.max_rel(x.grad[:, sl], r.grad) <= hp.BF16_GRAD_NORM_TOL, (jdoc, name)
