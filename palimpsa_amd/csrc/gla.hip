@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
   const ChunkArgs& a = A.c;
   const int H = a.H, dc = A.dc, de = A.de;
   const int KS = (dc + 31) >> 5;      // contraction steps of the scores and of the state term
-  const int dcp = 32 * KS + 8;        // row stride (bf16) of the Y tile
+  const int dcp = 32 * KS + 16;       // row stride (bf16) of the X and Y tiles: 32 bytes more than a multiple of 64 (no bank conflicts)
   float* sC = smem;                   // [64] running log2 decay inside the tile
   float* sDot = sC + kC;              // [4][64] partial dot products of the waves
   bf16x8* sP = (bf16x8*)(sDot + 4 * kC);   // [4 token blocks][2][64 lanes] score operands
@@ -299,7 +299,7 @@ template <typename TIn, int EB, bool REVERSE, bool STATE_T>
 static int launch_gla_tile_eb(const GlaTileArgs& A, int kern_id, hipStream_t s) {
   const int KS = (A.dc + 31) / 32;
   const size_t lds_head = sizeof(float) * (kC + 4 * kC);
-  const size_t lds_stage = 16 * 4 * 2 * 64 + sizeof(bf16_t) * (2 * (size_t)kC * (32 * KS + 8) + (size_t)A.de * kVT);
+  const size_t lds_stage = 16 * 4 * 2 * 64 + sizeof(bf16_t) * (2 * (size_t)kC * (32 * KS + 16) + (size_t)A.de * kVT);
   const size_t lds_out = (size_t)kC * (A.de * sizeof(TIn) + 16);   // the output tile reuses the staging area
   const size_t lds = lds_head + (lds_stage > lds_out ? lds_stage : lds_out);
   const int64_t blocks = (int64_t)A.c.total_chunks * A.c.H;
@@ -352,7 +352,17 @@ struct GlaBwdTileArgs {
   int64_t n_tokens;
 };
 
-constexpr int kFR = 72;   // row stride (bf16) of every tile of the fused kernel (rows of up to 64 entries)
+constexpr int kFR = 80;   // row stride (bf16) of the row and state tiles of the fused kernel (rows of up to 64 entries):
+                          // 16-byte reads by lanes (row i, piece g) are free of bank conflicts when the rows are
+                          // 32 bytes more than a multiple of 64 bytes apart (measured; 144-byte rows cost twice the time)
+constexpr int kFZ = 68;   // row stride (bf16) of its transposed tile and of its output tile: both are accessed in 8-byte
+                          // pieces by 16 lanes on 16 rows at a time, which 34 words per row spread over the 32 banks
+// Place of entry (row, col) in a state tile.  The tile is read along its rows (16-byte pieces) by one role and along
+// its columns (2-byte pieces, eight rows apart between the lane groups) by the others; eight rows are a multiple of
+// the 32 LDS banks apart, so the groups of 16 columns are exchanged between the groups of eight rows.
+constexpr int kFS = 72;   // row stride (bf16) of the state tiles (read along rows by one role only; 80 would not leave room for
+                          // two workgroups per compute unit)
+__device__ __forceinline__ int state_tile_at(int row, int col) { return row * kFS + (col ^ (((row >> 3) & 3) << 4)); }
 
 // Eight waves per workgroup (four per SIMD with two workgroups on a compute unit): a role's scores are formed by two
 // waves per token block (one per half of the score operand), its output by two waves per block of 16 columns (token
@@ -370,10 +380,10 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
   bf16_t* sK = sQ + kC * kFR;
   bf16_t* sV = sK + kC * kFR;
   bf16_t* sDo = sV + kC * kFR;
-  bf16_t* sS = sDo + kC * kFR;               // state tiles [64 value rows][kFR], zero beyond dv x dk
-  bf16_t* sG = sS + kC * kFR;
-  bf16_t* sZT = sG + kC * kFR;               // [64 columns][kVT]: the mixed rows of the current role, token index fastest
-  bf16x8* sP = (bf16x8*)(sZT + kC * kVT);    // [4 token blocks][2][64 lanes] score operands; then the output tile [64][kFR]
+  bf16_t* sS = sDo + kC * kFR;               // state tiles [64 value rows][kFS], zero beyond dv x dk
+  bf16_t* sG = sS + kC * kFS;
+  bf16_t* sZT = sG + kC * kFS;               // [64 columns][kFZ]: the mixed rows of the current role, token index fastest
+  bf16x8* sP = (bf16x8*)(sZT + kC * kFZ);    // [4 token blocks][2][64 lanes] score operands; then the output tile [64][kFZ]
   TIn* sOut = (TIn*)sP;
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -465,11 +475,11 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
       const int o = (2 * sp + u) * kFR + 8 * c8;
       *(bf16x8*)&ta[o] = ra[u];
       *(bf16x8*)&tb[o] = rb[u];
-      *(bf16x8*)&tc[o] = rc[u];
+      *(bf16x8*)&tc[state_tile_at(2 * sp + u, 8 * c8)] = rc[u];
     }
     if (!upper) {   // first role (dq) mixes the rows of k: token pair sp, one 32-bit word per column
 #pragma unroll
-      for (int e = 0; e < 8; ++e) *(bf16x2*)&sZT[(8 * c8 + e) * kVT + 2 * sp] = bf16x2{rb[0][e], rb[1][e]};
+      for (int e = 0; e < 8; ++e) *(bf16x2*)&sZT[(8 * c8 + e) * kFZ + 2 * sp] = bf16x2{rb[0][e], rb[1][e]};
     }
   }
   __syncthreads();
@@ -531,14 +541,14 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
       bf16x8 Sa;
       if constexpr (STATE_T) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) Sa[j] = sSt[(32 * ks + 8 * g + j) * kFR + 16 * eb + i];
+        for (int j = 0; j < 8; ++j) Sa[j] = sSt[state_tile_at(32 * ks + 8 * g + j, 16 * eb + i)];
       } else {
-        Sa = *(const bf16x8*)(sSt + (16 * eb + i) * kFR + 32 * ks + 8 * g);
+        Sa = *(const bf16x8*)(sSt + state_tile_at(16 * eb + i, 32 * ks + 8 * g));
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u) acc[u] = mfma16(Sa, x_operand(xh + 2 * u, ks), acc[u]);
     }
-    const bf16_t* zrow = sZT + (16 * eb + i) * kVT + 4 * g;
+    const bf16_t* zrow = sZT + (16 * eb + i) * kFZ + 4 * g;
     bf16x8 Za[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -573,7 +583,7 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
     if (valid) {
 #pragma unroll
       for (int u = 0; u < 2; ++u)
-        store_vec<4>(sOut + (16 * (xh + 2 * u) + i) * kFR + 16 * eb + 4 * g, (const float*)&acc[u]);
+        store_vec<4>(sOut + (16 * (xh + 2 * u) + i) * kFZ + 16 * eb + 4 * g, (const float*)&acc[u]);
     }
     if (zn) {
       // token pair zp, columns [8 zc + 4 ze, 8 zc + 4 ze + 4) of the next role's mixed rows
@@ -581,7 +591,7 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
       const bf16x4 z0 = *(const bf16x4*)(zn + (2 * zp) * kFR + 8 * zc + 4 * ze);
       const bf16x4 z1 = *(const bf16x4*)(zn + (2 * zp + 1) * kFR + 8 * zc + 4 * ze);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) *(bf16x2*)&sZT[(8 * zc + 4 * ze + e) * kVT + 2 * zp] = bf16x2{z0[e], z1[e]};
+      for (int e = 0; e < 4; ++e) *(bf16x2*)&sZT[(8 * zc + 4 * ze + e) * kFZ + 2 * zp] = bf16x2{z0[e], z1[e]};
     }
     __syncthreads();
     if (sW && w == 0 && lane < clen) {
@@ -595,7 +605,8 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
       TIn* obase = (TIn*)out + ((int64_t)t0 * H + h) * de;
       for (int idx = tid; idx < clen * per_row; idx += 512) {
         const int x = idx / per_row, c = idx - x * per_row;
-        *(f32x4*)(obase + (int64_t)x * H * de + 8 * c) = *(const f32x4*)(sOut + x * kFR + 8 * c);
+        const bf16x4 lo = *(const bf16x4*)(sOut + x * kFZ + 8 * c), hi = *(const bf16x4*)(sOut + x * kFZ + 8 * c + 4);
+        *(bf16x8*)(obase + (int64_t)x * H * de + 8 * c) = bf16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
     }
     __syncthreads();   // the output tile has been read: the next role may write its scores
@@ -618,7 +629,7 @@ static bool gla_bwd_tile_applies(const PalDims* d) {
 }
 
 static int launch_gla_bwd_tile(const GlaBwdTileArgs& A, hipStream_t s) {
-  const size_t lds = sizeof(float) * (kC + 8 * kC) + sizeof(bf16_t) * (size_t)kC * (6 * kFR + kVT + kFR);
+  const size_t lds = sizeof(float) * (kC + 8 * kC) + sizeof(bf16_t) * (size_t)kC * (4 * kFR + 2 * kFS + kFZ + 72);
   const int64_t items = (int64_t)A.c.total_chunks * A.c.H;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
