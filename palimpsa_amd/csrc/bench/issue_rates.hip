@@ -229,6 +229,80 @@ template <int MODE> void run(const char* name, int wps, int n_instr_per_iter, fl
   fflush(stdout);
 }
 
+// ---- LDS access patterns: LDS cycles per wave64 instruction when all 16 waves of a compute unit issue the same kind of
+// access with a given lane -> byte address map (bank conflicts show as multiples of the contiguous case)
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+enum LdsOp { kRead128, kRead64, kReadU16, kWrite32, kWrite64 };
+template <int OP> __global__ void lds_pattern_kernel(float* out, const int* addr_of_lane) {
+  extern __shared__ float lds[];
+  for (int i = threadIdx.x; i < 16384; i += blockDim.x) lds[i] = 0.f;
+  __syncthreads();
+  const int addr = addr_of_lane[threadIdx.x & 63];
+  float acc = 0.f;
+  for (int it = 0; it < ITER / 2; ++it) {
+    if (OP == kRead128) {
+      f32x4 r0, r1, r2, r3;
+      asm volatile("ds_read_b128 %0, %4\n ds_read_b128 %1, %4 offset:16384\n ds_read_b128 %2, %4 offset:32768\n ds_read_b128 %3, %4 offset:49152\n s_waitcnt lgkmcnt(0)"
+                   : "=v"(r0), "=v"(r1), "=v"(r2), "=v"(r3) : "v"(addr));
+      acc += r0[0] + r1[1] + r2[2] + r3[3];
+    } else if (OP == kRead64) {
+      f32x2 r0, r1, r2, r3;
+      asm volatile("ds_read_b64 %0, %4\n ds_read_b64 %1, %4 offset:16384\n ds_read_b64 %2, %4 offset:32768\n ds_read_b64 %3, %4 offset:49152\n s_waitcnt lgkmcnt(0)"
+                   : "=v"(r0), "=v"(r1), "=v"(r2), "=v"(r3) : "v"(addr));
+      acc += r0[0] + r1[1] + r2[0] + r3[1];
+    } else if (OP == kReadU16) {
+      float r0, r1, r2, r3;
+      asm volatile("ds_read_u16 %0, %4\n ds_read_u16 %1, %4 offset:16384\n ds_read_u16 %2, %4 offset:32768\n ds_read_u16 %3, %4 offset:49152\n s_waitcnt lgkmcnt(0)"
+                   : "=v"(r0), "=v"(r1), "=v"(r2), "=v"(r3) : "v"(addr));
+      acc += r0 + r1 + r2 + r3;
+    } else if (OP == kWrite32) {
+      asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %1 offset:16384\n ds_write_b32 %0, %1 offset:32768\n ds_write_b32 %0, %1 offset:49152\n s_waitcnt lgkmcnt(0)"
+                   :: "v"(addr), "v"(acc));
+    } else {
+      f32x2 v = {acc, acc};
+      asm volatile("ds_write_b64 %0, %1\n ds_write_b64 %0, %1 offset:16384\n ds_write_b64 %0, %1 offset:32768\n ds_write_b64 %0, %1 offset:49152\n s_waitcnt lgkmcnt(0)"
+                   :: "v"(addr), "v"(v));
+    }
+  }
+  out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+template <int OP> void run_lds(const char* name, int (*addr)(int), float* out, int* table) {
+  int h[64];
+  for (int l = 0; l < 64; ++l) h[l] = addr(l);
+  HIP_OK(hipMemcpy(table, h, sizeof(h), hipMemcpyHostToDevice));
+  HIP_OK(hipFuncSetAttribute((const void*)lds_pattern_kernel<OP>, hipFuncAttributeMaxDynamicSharedMemorySize, 66 * 1024));
+  hipEvent_t e0, e1; HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+  lds_pattern_kernel<OP><<<256, 1024, 66 * 1024>>>(out, table);
+  HIP_OK(hipEventRecord(e0));
+  lds_pattern_kernel<OP><<<256, 1024, 66 * 1024>>>(out, table);
+  HIP_OK(hipEventRecord(e1)); HIP_OK(hipEventSynchronize(e1));
+  float ms; HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  printf("%-78s %6.2f LDS cycles per wave instruction\n", name, ms * 1e-3 * g_ghz * 1e9 / ((double)(ITER / 2) * 4 * 16));
+  fflush(stdout);
+}
+#define LDS_ROWS(OP, S, PIECE) \
+  run_lds<OP>(#OP " rows " #S " bytes apart: (lane & 15) * " #S " + (lane >> 4) * " #PIECE, [](int l) { return (l & 15) * S + (l >> 4) * PIECE; }, out, table)
+static void lds_patterns(float* out) {
+  int* table;
+  HIP_OK(hipMalloc(&table, 64 * sizeof(int)));
+  printf("LDS access patterns, 16 waves per compute unit\n");
+  run_lds<kRead128>("kRead128 contiguous: lane * 16", [](int l) { return l * 16; }, out, table);
+  LDS_ROWS(kRead128, 96, 16); LDS_ROWS(kRead128, 144, 16); LDS_ROWS(kRead128, 160, 16); LDS_ROWS(kRead128, 176, 16);
+  LDS_ROWS(kRead128, 224, 16); LDS_ROWS(kRead128, 272, 16); LDS_ROWS(kRead128, 288, 16); LDS_ROWS(kRead128, 544, 16);
+  run_lds<kRead64>("kRead64 contiguous: lane * 8", [](int l) { return l * 8; }, out, table);
+  LDS_ROWS(kRead64, 136, 8); LDS_ROWS(kRead64, 144, 8); LDS_ROWS(kRead64, 160, 8); LDS_ROWS(kRead64, 176, 8);
+  run_lds<kReadU16>("kReadU16 contiguous: lane * 2", [](int l) { return l * 2; }, out, table);
+  run_lds<kReadU16>("kReadU16 columns of rows 144 bytes apart, lane groups 8 rows apart", [](int l) { return 8 * (l >> 4) * 144 + (l & 15) * 2; }, out, table);
+  run_lds<kReadU16>("kReadU16 the same with the 32-byte groups of a row exchanged per lane group", [](int l) { return 8 * (l >> 4) * 144 + (((l & 15) ^ ((l >> 4) << 4)) * 2); }, out, table);
+  run_lds<kWrite32>("kWrite32 contiguous: lane * 4", [](int l) { return l * 4; }, out, table);
+  run_lds<kWrite32>("kWrite32 transposing: column 8 (lane & 7), word lane >> 3, columns 144 bytes apart", [](int l) { return 8 * (l & 7) * 144 + (l >> 3) * 4; }, out, table);
+  run_lds<kWrite32>("kWrite32 transposing: column 8 (lane & 7), word lane >> 3, columns 136 bytes apart", [](int l) { return 8 * (l & 7) * 136 + (l >> 3) * 4; }, out, table);
+  run_lds<kWrite32>("kWrite32 transposing: column 8 (lane & 7), word lane >> 3, columns 140 bytes apart", [](int l) { return 8 * (l & 7) * 140 + (l >> 3) * 4; }, out, table);
+  run_lds<kWrite64>("kWrite64 contiguous: lane * 8", [](int l) { return l * 8; }, out, table);
+  LDS_ROWS(kWrite64, 136, 8); LDS_ROWS(kWrite64, 144, 8); LDS_ROWS(kWrite64, 160, 8);
+  HIP_OK(hipFree(table));
+}
+
 int main() {
   int khz = 0;
   HIP_OK(hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, 0));
@@ -280,5 +354,6 @@ int main() {
     }
     if (wps == 4) run<27>("1 wave mfma only, 3 waves fma only", wps, 52, out, cyc);
   }
+  lds_patterns(out);
   return 0;
 }
