@@ -610,3 +610,48 @@ def test_backward_packed_batch_walked_by_resident_workgroups(gpu_device):
         (o_ref * do[:, sl].double()).sum().backward()
         for name, x, r in zip(("q", "k", "v", "g"), leaves, rl):
             assert hp.max_rel(x.grad[:, sl], r.grad) <= hp.BF16_GRAD_NORM_TOL, (jdoc, name)
+
+
+def test_forward_and_backward_replay_in_a_graph(gpu_device):
+    """chunk_simple_gla forward + backward recorded into a HIP graph (head dims 64: the backward tile kernel with
+    resident workgroups): three replays on new values, with eager work in between, each equal to the eager result."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla
+    dev = gpu_device
+    B, T, H, d = 2, 300, 3, 64
+
+    def fresh(seed):
+        q, k, v, g, _ = _inputs(B, T, H, d, d, seed)
+        do = torch.randn(B, T, H, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16()
+        return [x.to(dev) for x in (q, k, v, g)], do.to(dev)
+
+    def eager(xs, do):
+        leaves = [x.clone().requires_grad_(True) for x in xs]
+        o, _ = chunk_simple_gla(q=leaves[0], k=leaves[1], v=leaves[2], g=leaves[3])
+        return (o.detach(),) + torch.autograd.grad(o, leaves, do)
+
+    xs0, do0 = fresh(500)
+    static = [x.clone().requires_grad_(True) for x in xs0]
+    static_do = do0.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            o, _ = chunk_simple_gla(q=static[0], k=static[1], v=static[2], g=static[3])
+            torch.autograd.grad(o, static, static_do)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g, _ = chunk_simple_gla(q=static[0], k=static[1], v=static[2], g=static[3])
+        grads_g = torch.autograd.grad(o_g, static, static_do)
+    for seed in (510, 520, 530):
+        xs, do = fresh(seed)
+        ref = eager(xs, do)
+        with torch.no_grad():
+            for x, y in zip(static, xs):
+                x.copy_(y)
+            static_do.copy_(do)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a_, b_, n in zip((o_g,) + tuple(grads_g), ref, "oqkvg"):
+            assert torch.equal(a_, b_), (seed, n)
