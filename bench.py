@@ -480,7 +480,7 @@ def bench_c2(torch, dev, steps, warmup):
     E, th = d * d, T * H
     roof = mfma_roofline("chunk_bwd_local_kernel", kernels, 4 * (CHUNK + 1) * E * th, th * E,
                          "flops = 4(C+1)*dk*dv per token-head; step_frac uses (6C+14)*dk*dv; dk = 96 runs the tile kernel "
-                         "in two passes of three column blocks")
+                         "in three passes of two column blocks (two workgroups per compute unit)")
     roof["step_frac"] = (6 * CHUNK + 14) * E * th / (ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
     return {"workload": f"c2: packed varlen chunked fwd+bwd, {len(cu) - 1} documents, 32768 tokens, H=16 dk=dv=96 bf16",
             "documents": len(cu) - 1, "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_median": med,
