@@ -118,13 +118,16 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
   // the rows of PF tokens are in flight: a token is taken from its register set and the set reloaded at once with
   // the token PF ahead (always issued, clamped to the last token: the same number of requests in every iteration)
   constexpr int PF = kRecBwdPrefetch<NPL>;
-  float kb[PF][NPL], vb[PF], bb_[PF], gb[PF];
-  auto load_rows = [&](int t, float* kk, float& vv, float& bb, float& gg) {
+  // (the gate is requested as the aligned word that holds it and decoded when the token is taken up: one kind of
+  //  request for both storage types, so that no wait is forced where the two would meet)
+  float kb[PF][NPL], vb[PF], bb_[PF];
+  unsigned gb[PF];
+  auto load_rows = [&](int t, float* kk, float& vv, float& bb, unsigned& gg) {
 #pragma unroll
     for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
     vv = to_f32(vp[(int64_t)t * H * dv]);
     bb = to_f32(bp[(int64_t)t * H * dv]);
-    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+    gg = load_gate_word(a.gt, (bos + t) * H + h, a.gate_bf16);
   };
   if (len > 0) {
 #pragma unroll
@@ -137,9 +140,11 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
       float kc[NPL];
 #pragma unroll
       for (int e = 0; e < NPL; ++e) kc[e] = kb[u][e];
-      const float vv = vb[u], bb = bb_[u], gt = gb[u];
+      const float vv = vb[u], bb = bb_[u];
+      const unsigned gw = gb[u];
       load_rows(min(t + PF, len - 1), kb[u], vb[u], bb_[u], gb[u]);
       if (t < len) {
+        const float gt = gate_value(gw, (bos + t) * H + h, a.gate_bf16);
         if (t % S == 0) {
           const int64_t co = (((int64_t)(segbase + t / S) * H + h) * dv + drow) * dk;
 #pragma unroll
@@ -160,7 +165,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_state_kernel(RecBwdArgs a) {
 }
 
 // ------------------------------------------------------------------- backward
-template <typename TIn, int NPL>
+template <typename TIn, int NPL, bool HAS_VAR>
 __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
   using Map = NMapB<NPL>;
   constexpr int VW = Map::VW, NV = Map::NV;
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
   rec_seq(a, n, bos, len, segbase);
   const float gval = a.g[h];
   const float gh = gval * kLog2e, Ip = a.Ip[h], scale = a.scale;
-  const bool has_var = a.flags & PAL_FLAG_HAS_VAR;
+  constexpr bool has_var = HAS_VAR;
   const int drow = tile * 4 + grp;
   const TIn* qp = (const TIn*)a.q + (bos * a.Hq + h / (H / a.Hq)) * dk;
   const TIn* kp = (const TIn*)a.k + (bos * a.Hq + h / (H / a.Hq)) * dk;
@@ -182,14 +187,17 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
   const TIn* bp = (const TIn*)a.b + vrow;
   const TIn* dop = (const TIn*)a.d_o + vrow;
   constexpr int PF = kRecBwdPrefetch<NPL>;
-  auto load_fwd_rows = [&](int t, float* kk, float& vv, float& bb, float& gg) {
+  // gates and the gradient of the uncertainty output (element types chosen at run time) are requested as the aligned
+  // word that holds them and decoded when the token is taken up: one kind of request for both storage types, so that
+  // the rows of the tokens ahead stay in flight (a type branch at the request would be waited for on the spot)
+  auto load_fwd_rows = [&](int t, float* kk, float& vv, float& bb, unsigned& gg) {
 #pragma unroll
     for (int iv = 0; iv < NV; ++iv) load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
     vv = to_f32(vp[(int64_t)t * H * dv]);
     bb = to_f32(bp[(int64_t)t * H * dv]);
-    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+    gg = load_gate_word(a.gt, (bos + t) * H + h, a.gate_bf16);
   };
-  auto load_bwd_rows = [&](int t, float* kk, float* qq, float& vv, float& bb, float& dd, float& dvar, float& gg) {
+  auto load_bwd_rows = [&](int t, float* kk, float* qq, float& vv, float& bb, float& dd, unsigned& dvar, unsigned& gg) {
 #pragma unroll
     for (int iv = 0; iv < NV; ++iv) {
       load_vec<VW>(kp + (int64_t)t * a.Hq * dk + Map::vec_start(j, iv), kk + iv * VW);
@@ -198,8 +206,9 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
     vv = to_f32(vp[(int64_t)t * H * dv]);
     bb = to_f32(bp[(int64_t)t * H * dv]);
     dd = to_f32(dop[(int64_t)t * H * dv]);
-    dvar = has_var ? load_rt(a.d_o_var, vrow + (int64_t)t * H * dv, a.var_bf16) : 0.f;
-    gg = load_gate(a.gt, (bos + t) * H + h, a.gate_bf16);
+    dvar = 0u;
+    if constexpr (HAS_VAR) dvar = load_gate_word(a.d_o_var, vrow + (int64_t)t * H * dv, a.var_bf16);
+    gg = load_gate_word(a.gt, (bos + t) * H + h, a.gate_bf16);
   };
   float dMc[NPL], dJc[NPL];   // f_{t+1} dM_{t+1}: what flows into token t from the future
 #pragma unroll
@@ -219,7 +228,8 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
     }
     // states before every token of the segment (rows of PF tokens in flight, see recurrent_bwd_state_kernel)
     {
-      float kb[PF][NPL], vb[PF], bb_[PF], gb[PF];
+      float kb[PF][NPL], vb[PF], bb_[PF];
+      unsigned gb[PF];
 #pragma unroll
       for (int u = 0; u < PF; ++u) load_fwd_rows(ts + min(u, cnt - 1), kb[u], vb[u], bb_[u], gb[u]);
       for (int j0 = 0; j0 < cnt; j0 += PF) {
@@ -229,7 +239,8 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
           float kc[NPL];
 #pragma unroll
           for (int e = 0; e < NPL; ++e) kc[e] = kb[u][e];
-          const float vv = vb[u], bb = bb_[u], gt = gb[u];
+          const float vv = vb[u], bb = bb_[u];
+          const float gt = gate_value(gb[u], (bos + ts + min(jj, cnt - 1)) * H + h, a.gate_bf16);
           load_fwd_rows(ts + min(jj + PF, cnt - 1), kb[u], vb[u], bb_[u], gb[u]);
           if (jj < cnt) {
 #pragma unroll
@@ -250,7 +261,8 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
       }
     }
     // reverse over the tokens of the segment, rows of PF tokens in flight (token cnt-1-r in round r)
-    float rk[PF][NPL], rq[PF][NPL], rv[PF], rb[PF], rdo[PF], rdv[PF], rg[PF];
+    float rk[PF][NPL], rq[PF][NPL], rv[PF], rb[PF], rdo[PF];
+    unsigned rdv[PF], rg[PF];
 #pragma unroll
     for (int u = 0; u < PF; ++u) load_bwd_rows(ts + max(cnt - 1 - u, 0), rk[u], rq[u], rv[u], rb[u], rdo[u], rdv[u], rg[u]);
     for (int r0 = 0; r0 < cnt; r0 += PF) {
@@ -260,7 +272,11 @@ __global__ __launch_bounds__(64) void recurrent_bwd_kernel(RecBwdArgs a) {
       float kc[NPL], qc[NPL];
 #pragma unroll
       for (int e = 0; e < NPL; ++e) { kc[e] = rk[u][e]; qc[e] = rq[u][e]; }
-      const float vv = rv[u], bb = rb[u], dov = scale * rdo[u], dvv = scale * rdv[u], gt = rg[u];
+      const float vv = rv[u], bb = rb[u], dov = scale * rdo[u];
+      const int tl = ts + max(jj, 0);                       // the token this register set was requested for
+      const float gt = gate_value(rg[u], (bos + tl) * H + h, a.gate_bf16);
+      float dvv = 0.f;
+      if constexpr (HAS_VAR) dvv = scale * gate_value(rdv[u], vrow + (int64_t)tl * H * dv, a.var_bf16);
       load_bwd_rows(ts + max(jj - PF, 0), rk[u], rq[u], rv[u], rb[u], rdo[u], rdv[u], rg[u]);
       if (jj < 0) continue;
       const int t = ts + jj;
@@ -454,8 +470,13 @@ static int launch_rec_bwd(const RecBwdArgs& a, hipStream_t s) {
   PAL_TIMED_LAUNCH(kKernRecurrentBwdFwdPass, s, (recurrent_bwd_state_kernel<TIn, NPL>), dim3((unsigned)blocks), dim3(64), 0, s, a);
   PAL_HIP_LAUNCH_CHECK();
   const size_t lds = (size_t)a.S * 2 * NPL * 64 * sizeof(float);
-  if (int rc = allow_lds((const void*)&recurrent_bwd_kernel<TIn, NPL>, lds)) return rc;
-  PAL_TIMED_LAUNCH(kKernRecurrentBwd, s, (recurrent_bwd_kernel<TIn, NPL>), dim3((unsigned)blocks), dim3(64), lds, s, a);
+  if (a.flags & PAL_FLAG_HAS_VAR) {
+    if (int rc = allow_lds((const void*)&recurrent_bwd_kernel<TIn, NPL, true>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernRecurrentBwd, s, (recurrent_bwd_kernel<TIn, NPL, true>), dim3((unsigned)blocks), dim3(64), lds, s, a);
+  } else {
+    if (int rc = allow_lds((const void*)&recurrent_bwd_kernel<TIn, NPL, false>, lds)) return rc;
+    PAL_TIMED_LAUNCH(kKernRecurrentBwd, s, (recurrent_bwd_kernel<TIn, NPL, false>), dim3((unsigned)blocks), dim3(64), lds, s, a);
+  }
   PAL_HIP_LAUNCH_CHECK();
   return PAL_OK;
 }
