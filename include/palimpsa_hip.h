@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PAL_ABI_VERSION 3
+#define PAL_ABI_VERSION 4
 
 /* element types of tensors handed over the boundary */
 #define PAL_DTYPE_F32 0
@@ -261,6 +261,11 @@ typedef struct PalGlueDims {
   int32_t dtype;        /* PAL_DTYPE_* of every row tensor                     */
   float eps;            /* prologue: clamp of the L2 norm (F.normalize, 1e-12);
                            epilogue: eps of the RMS norm                       */
+  float dt_min, dt_max; /* prologue in the MetaMamba2 form (bs_raw NULL): bounds of the clamp on
+                           softplus(dt_raw + dt_bias) (layers/meta_mamba2.py:284, time_step_limit) */
+  int32_t norm_over_heads; /* epilogue: 0 = RMS norm over dv per head, gate after it (layers/palimpsa.py:337-343);
+                           1 = gate first, RMS norm over all H*dv entries of a token with weight [H*dv] and
+                           rstd [tokens] (layers/meta_mamba2.py:355-363); H*dv <= 4096 */
 } PalGlueDims;
 
 typedef struct PalPrologueTensors {
@@ -288,7 +293,11 @@ typedef struct PalPrologueGrads {
  *   q, k = l2norm(q_raw), l2norm(k_raw), heads repeated H/Hqk times
  *   bs = sigmoid(bs_raw) rounded to dtype;  v = x * bs
  *   b = sigmoid(b_raw) * softplus(b_scale) * bs          (when b_raw given)
- *   gt = softplus(dt_raw + dt_bias)                      (fp32)            */
+ *   gt = softplus(dt_raw + dt_bias)                      (fp32)
+ * With bs_raw NULL the call is the MetaMamba2 layer's (layers/meta_mamba2.py:283-299):
+ *   gt = clamp(softplus(dt_raw + dt_bias), dt_min, dt_max);  v = x * gt;  b = sigmoid(b_raw) * softplus(b_scale) * gt
+ * and q_raw, k_raw, q, k may all be NULL (that layer hands its B, C rows to the operator as they are,
+ * shared heads through PalDims.n_qk_heads); dbs_raw, and with them dq, dk, dq_raw, dk_raw, are then unused. */
 int pal_prologue_fwd(const PalGlueDims *dims, const PalPrologueTensors *t, void *stream);
 /* Its backward.  workspace: pal_prologue_bwd_workspace_bytes(dims) bytes of
  * device memory for the per-head partial sums of ddt_bias / db_scale. */
@@ -315,7 +324,10 @@ typedef struct PalEpilogueGrads {
 
 /* y = rmsnorm(o + x*D) * weight * gate*sigmoid(gate)   (layers/palimpsa.py:337-343;
  * the gated norm is fla.modules.FusedRMSNormGated, a dependency outside the
- * reference tree: RMS norm over dv, then a swish gate). */
+ * reference tree: RMS norm over dv, then a swish gate).
+ * With dims->norm_over_heads: y = rmsnorm_{H*dv}((o + x*D) * gate*sigmoid(gate)) * weight
+ * (layers/meta_mamba2.py:355-363; fla.modules.layernorm_gated.RMSNormGated with norm_before_gate=False,
+ * restated from its published behaviour), weight [H*dv], rstd [tokens]. */
 int pal_epilogue_fwd(const PalGlueDims *dims, const PalEpilogueTensors *t, void *stream);
 size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims *dims);
 int pal_epilogue_bwd(const PalGlueDims *dims, const PalEpilogueTensors *t, const PalEpilogueGrads *gr,

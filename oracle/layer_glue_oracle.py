@@ -17,6 +17,15 @@ What it restates (citations are into the reference repository):
   third-party code itself.  What the mathematics fixes is pinned in tests/test_layer_glue_oracle_cpu.py:
   the ungated case against ``torch.nn.functional.rms_norm``, the gate against ``F.silu``, unit norms and
   head repetition of q/k, and ``torch.autograd.gradcheck`` of both functions in float64.
+* ``mamba_prologue``: palimpsa/layers/meta_mamba2.py:283-299 —
+  ``dt = clamp(softplus(dt.float() + dt_bias), *time_step_limit)`` (:283-284), ``dx = (x * dt).to(x.dtype)`` (:294),
+  ``b = (sigmoid(b_raw) * softplus(b_scale) * dt).to(h.dtype)`` (:296-299); same torch routines as those lines.
+* ``mamba_epilogue``: palimpsa/layers/meta_mamba2.py:355-363 — ``o + x * D`` (:356), heads flattened (:359) and
+  ``RMSNormGated(intermediate_size, eps, norm_before_gate=False)(o, gate)`` (:363; built at :130-132), again a module of
+  flash-linear-attention (fla.modules.layernorm_gated, the Mamba2 norm): with ``norm_before_gate=False`` it is
+  ``rms_norm(x * silu(z)) * weight`` over the whole last dim.  Restated from that published behaviour, **parity unpinned**
+  against the third-party code; pinned in the same test file against ``F.rms_norm`` on the gated input, by
+  the clamp's limits and by ``gradcheck``.
 """
 from __future__ import annotations
 
@@ -55,3 +64,28 @@ def epilogue(o, x, D, gate, weight, eps, compute=torch.float64):
         g = gate.to(compute)
         y = y * g * torch.sigmoid(g)
     return y
+
+
+def mamba_prologue(x, dt_raw, dt_bias, b_raw=None, b_scale=None, dt_limit=(0.0, float("inf")), compute=torch.float64):
+    """Returns (v, b | None, dt) in ``compute`` precision."""
+    dt = F.softplus(dt_raw.to(compute) + dt_bias.to(compute))
+    dt = torch.clamp(dt, dt_limit[0], dt_limit[1])
+    v = x.to(compute) * dt.unsqueeze(-1)
+    b = None
+    if b_raw is not None:
+        b = torch.sigmoid(b_raw.to(compute)) * F.softplus(b_scale.to(compute)).view(-1, 1)
+        b = b * dt.unsqueeze(-1)
+    return v, b, dt
+
+
+def mamba_epilogue(o, x, D, gate, weight, eps, compute=torch.float64):
+    """rmsnorm over all heads of ((o + x * D) * gate * sigmoid(gate)) * weight; o [..., H, dv] -> [..., H, dv]."""
+    r = o.to(compute)
+    if x is not None:
+        r = r + x.to(compute).reshape(r.shape) * D.to(compute).view(-1, 1)
+    flat = r.flatten(-2)
+    if gate is not None:
+        g = gate.to(compute).reshape(flat.shape)
+        flat = flat * g * torch.sigmoid(g)
+    rstd = torch.rsqrt(flat.pow(2).mean(-1, keepdim=True) + eps)
+    return (flat * rstd * weight.to(compute).reshape(-1)).reshape(r.shape)

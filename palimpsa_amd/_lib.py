@@ -12,7 +12,7 @@ from typing import Optional
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libpalimpsa_hip.so")
 
-PAL_ABI_VERSION = 3
+PAL_ABI_VERSION = 4
 PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
 PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS, PAL_FLAG_FP32_FAST = 256, 512, 1024
@@ -49,7 +49,8 @@ class PalBwdTensors(C.Structure):
 
 
 class PalGlueDims(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in ("tokens", "n_heads", "n_qk_heads", "dk", "dv", "dtype")] + [("eps", C.c_float)]
+    _fields_ = ([(n, C.c_int32) for n in ("tokens", "n_heads", "n_qk_heads", "dk", "dv", "dtype")] +
+                [("eps", C.c_float), ("dt_min", C.c_float), ("dt_max", C.c_float), ("norm_over_heads", C.c_int32)])
 
 
 class PalPrologueTensors(C.Structure):

@@ -2,6 +2,10 @@
 //   prologue (palimpsa/layers/palimpsa.py:266-279): L2-normalised q, k (heads repeated), v = x * bs,
 //     b = sigmoid(b_raw) * softplus(b_scale) * bs, gt = softplus(dt_raw + dt_bias);
 //   epilogue (:337-343): y = rmsnorm(o + x * D) * weight * swish(gate).
+// and of the reference's other caller of the operator (palimpsa/layers/meta_mamba2.py):
+//   prologue (:283-299): dt = clamp(softplus(dt_raw + dt_bias)), v = x * dt, b = sigmoid(b_raw) * softplus(b_scale) * dt
+//     (q = C and k = B go to the operator as they are, shared heads through its n_qk_heads);
+//   epilogue (:355-363): y = rmsnorm over all heads of a token of ((o + x * D) * swish(gate)) * weight.
 // All of it is bound by HBM: every row is read once and written once.  A row of d elements is handled
 // by a group of GL lanes (the power of two >= d/8), eight consecutive elements per lane (16-byte
 // accesses for bf16 rows); a workgroup of 256 threads owns one head and a range of tokens, so that the
@@ -73,12 +77,15 @@ struct PrologueArgs {
   float* part;          // backward: [H][n_token_blocks][2] partial sums (ddt_bias, db_scale)
   int tokens, H, Hqk, dk, dv, GLk, GLv, tok_per_block;
   float eps;
+  int mamba;            // the multiplier of x and b is gt itself, clamped to [dt_min, dt_max] (no bs_raw)
+  int task0;            // first task of the grid's z axis (2 when there are no q, k rows)
+  float dt_min, dt_max;
 };
 
 // grid (token blocks, heads, 3): z = 0 rows of q, z = 1 rows of k (heads of q_raw / k_raw), z = 2 rows of v, b and gt
 template <typename T>
 __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
-  const int tid = threadIdx.x, task = blockIdx.z, h = blockIdx.y;
+  const int tid = threadIdx.x, task = blockIdx.z + A.task0, h = blockIdx.y;
   const int tok0 = blockIdx.x * A.tok_per_block;
   const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
   if (task < 2) {
@@ -109,8 +116,14 @@ __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
     const float bias = A.t.dt_bias[h];
     for (int tok = tok0 + slot; tok < tok1; tok += rows) {
       const int64_t th = (int64_t)tok * A.H + h;
-      const float bs = round_to<T>(sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th])));
-      if (l == 0) A.t.gt[th] = softplusf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias);
+      float gtv = softplusf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias), bs;
+      if (A.mamba) {
+        gtv = fminf(fmaxf(gtv, A.dt_min), A.dt_max);
+        bs = gtv;
+      } else {
+        bs = round_to<T>(sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th])));
+      }
+      if (l == 0) A.t.gt[th] = gtv;
       if (!on) continue;
       float x[8];
       load8((const T*)A.t.x + th * d + 8 * l, x);
@@ -131,7 +144,7 @@ __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
 template <typename T>
 __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
   __shared__ float sRed[4][2];
-  const int tid = threadIdx.x, task = blockIdx.z, h = blockIdx.y;
+  const int tid = threadIdx.x, task = blockIdx.z + A.task0, h = blockIdx.y;
   const int tok0 = blockIdx.x * A.tok_per_block;
   const int tok1 = min(A.tokens, tok0 + A.tok_per_block);
   if (task < 2) {
@@ -179,8 +192,17 @@ __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
     float acc_dt = 0.f, acc_bs = 0.f;   // this thread's share of ddt_bias[h] and of sum db * sigmoid(b_raw) * bs
     for (int tok = tok0 + slot; tok < tok1; tok += rows) {
       const int64_t th = (int64_t)tok * A.H + h;
-      const float sg = sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th]));
-      const float bs = round_to<T>(sg);
+      const float pre = to_f32(((const T*)A.t.dt_raw)[th]) + bias;
+      float sg = 0.f, bs;
+      bool pass = true;     // mamba: the clamp lets the gradient through (bounds included, as torch.clamp)
+      if (A.mamba) {
+        const float spd = softplusf_(pre);
+        pass = spd >= A.dt_min && spd <= A.dt_max;
+        bs = fminf(fmaxf(spd, A.dt_min), A.dt_max);
+      } else {
+        sg = sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th]));
+        bs = round_to<T>(sg);
+      }
       float dbs = 0.f, dsp = 0.f;
       if (on) {
         float x[8], gv[8];
@@ -205,8 +227,14 @@ __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
       }
       dbs = group_sum(fmaf(dsp, sp, dbs), GL);   // d/d bs of v = x bs and b = s sp bs
       if (l == 0) {
-        ((T*)A.g.dbs_raw)[th] = from_f32<T>(dbs * sg * (1.f - sg));
-        const float ddt = A.g.dgt[th] * sigmoidf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias);
+        float ddt;
+        if (A.mamba) {
+          // gt is an output and the multiplier of x and b
+          ddt = pass ? (A.g.dgt[th] + dbs) * sigmoidf_(pre) : 0.f;
+        } else {
+          ((T*)A.g.dbs_raw)[th] = from_f32<T>(dbs * sg * (1.f - sg));
+          ddt = A.g.dgt[th] * sigmoidf_(pre);
+        }
         ((T*)A.g.ddt_raw)[th] = from_f32<T>(ddt);
         acc_dt += ddt;
       }
@@ -400,6 +428,196 @@ __global__ void epilogue_bwd_reduce_kernel(EpilogueArgs A, int n_blocks) {
   }
 }
 
+// ------------------------------------------------------------------ epilogue over all heads of a token
+// y = rmsnorm_{H dv}((o + x D) swish(gate)) weight  (palimpsa/layers/meta_mamba2.py:355-363: the gate is applied before
+// a norm that runs over the whole token).  One wave per token, 512 elements per pass (eight per lane, inside one head
+// since dv is a multiple of 8); a wave takes kHeadsIter tokens in turn and the four waves of a workgroup add their sums
+// over tokens (dweight, dD of the backward) in LDS, so that a workgroup leaves one partial row per 16 tokens.
+constexpr int kHeadsIter = 4;      // tokens per wave (a workgroup of four waves takes 16)
+constexpr int kHeadsMaxCh = 8;     // passes of 512 elements: H dv <= 4096
+
+template <typename T>
+__global__ __launch_bounds__(256) void epilogue_heads_fwd_kernel(EpilogueArgs A) {
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int dv = A.dv, HD = A.H * dv, nch = (HD + 511) >> 9;
+  const float inv_n = 1.f / (float)HD;
+  for (int it = 0; it < kHeadsIter; ++it) {
+    const int tok = ((int)blockIdx.x * 4 + w) * kHeadsIter + it;
+    if (tok >= A.tokens) break;
+    const int64_t row = (int64_t)tok * HD;
+    float r[kHeadsMaxCh][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kHeadsMaxCh; ++c) {
+      const int e0 = 512 * c + 8 * lane;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[c][e] = 0.f;
+      if (c < nch && e0 < HD) {
+        load8((const T*)A.t.o + row + e0, r[c]);
+        if (A.t.x) {
+          float x[8];
+          load8((const T*)A.t.x + row + e0, x);
+          const float Dh = A.t.D[e0 / dv];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) r[c][e] = fmaf(x[e], Dh, r[c][e]);
+        }
+        if (A.t.gate) {
+          float z[8];
+          load8((const T*)A.t.gate + row + e0, z);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) r[c][e] *= z[e] * sigmoidf_(z[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(r[c][e], r[c][e], ss);
+      }
+    }
+    ss = wave_sum(ss);
+    const float rstd = rsqrtf(ss * inv_n + A.eps);
+    if (lane == 0) A.t.rstd[tok] = rstd;
+#pragma unroll
+    for (int c = 0; c < kHeadsMaxCh; ++c) {
+      const int e0 = 512 * c + 8 * lane;
+      if (c < nch && e0 < HD) {
+        float wv[8], y[8];
+        load8(A.t.weight + e0, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = r[c][e] * rstd * wv[e];
+        store8((T*)A.t.y + row + e0, y);
+      }
+    }
+  }
+}
+
+// r = u s, u = o + x D, s = swish(gate);  n = r rstd;  y = n w;  g = dy w;  dr = rstd (g - n mean(g n));
+// du = dr s (= d_o), dx = du D, dgate = dr u s', dD[h] += du . x, dweight += dy n.
+// Two passes over the token's rows (the second finds them in the cache): the mean first, then the gradients.
+// part_w: [workgroups][H dv] partial dweight, part_D: [workgroups][H dv / 8] partial dD (one slot per eight elements).
+template <typename T>
+__global__ __launch_bounds__(256) void epilogue_heads_bwd_kernel(EpilogueArgs A) {
+  extern __shared__ float sPartial[];   // [4 waves][H dv + H dv / 8]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int dv = A.dv, HD = A.H * dv, nch = (HD + 511) >> 9;
+  const float inv_n = 1.f / (float)HD;
+  const int64_t wave_id = (int64_t)blockIdx.x * 4 + w;
+  float dw[kHeadsMaxCh][8], accD[kHeadsMaxCh];
+#pragma unroll
+  for (int c = 0; c < kHeadsMaxCh; ++c) {
+    accD[c] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dw[c][e] = 0.f;
+  }
+  // u, swish(gate) and its derivative, x of eight elements of a token
+  auto fetch = [&](int64_t row, int e0, float* u, float* sw, float* dsw, float* x, float& Dh) {
+    load8((const T*)A.t.o + row + e0, u);
+    Dh = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sw[e] = 1.f; dsw[e] = 0.f; x[e] = 0.f; }
+    if (A.t.x) {
+      load8((const T*)A.t.x + row + e0, x);
+      Dh = A.t.D[e0 / dv];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = fmaf(x[e], Dh, u[e]);
+    }
+    if (A.t.gate) {
+      float z[8];
+      load8((const T*)A.t.gate + row + e0, z);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float sg = sigmoidf_(z[e]);
+        sw[e] = z[e] * sg;
+        dsw[e] = sg * (1.f + z[e] * (1.f - sg));
+      }
+    }
+  };
+  for (int it = 0; it < kHeadsIter; ++it) {
+    const int tok = (int)wave_id * kHeadsIter + it;
+    if (tok >= A.tokens) break;
+    const int64_t row = (int64_t)tok * HD;
+    const float rstd = A.t.rstd[tok];
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < kHeadsMaxCh; ++c) {
+      const int e0 = 512 * c + 8 * lane;
+      if (c < nch && e0 < HD) {
+        float u[8], sw[8], dsw[8], x[8], gy[8], wv[8], Dh;
+        fetch(row, e0, u, sw, dsw, x, Dh);
+        load8((const T*)A.g.dy + row + e0, gy);
+        load8(A.t.weight + e0, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot = fmaf(gy[e] * wv[e], u[e] * sw[e] * rstd, dot);
+      }
+    }
+    dot = wave_sum(dot) * inv_n;
+#pragma unroll
+    for (int c = 0; c < kHeadsMaxCh; ++c) {
+      const int e0 = 512 * c + 8 * lane;
+      if (c < nch && e0 < HD) {
+        float u[8], sw[8], dsw[8], x[8], gy[8], wv[8], Dh;
+        fetch(row, e0, u, sw, dsw, x, Dh);
+        load8((const T*)A.g.dy + row + e0, gy);
+        load8(A.t.weight + e0, wv);
+        float du[8], dz[8], dx[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float n = u[e] * sw[e] * rstd;
+          const float dr = rstd * (gy[e] * wv[e] - n * dot);
+          du[e] = dr * sw[e];
+          dz[e] = dr * u[e] * dsw[e];
+          dx[e] = du[e] * Dh;
+          accD[c] = fmaf(du[e], x[e], accD[c]);
+          dw[c][e] = fmaf(gy[e], n, dw[c][e]);
+        }
+        store8((T*)A.g.d_o + row + e0, du);
+        if (A.t.x) store8((T*)A.g.dx + row + e0, dx);
+        if (A.t.gate) store8((T*)A.g.dgate + row + e0, dz);
+      }
+    }
+  }
+  const int per_wave = HD + (HD >> 3);
+#pragma unroll
+  for (int c = 0; c < kHeadsMaxCh; ++c) {
+    const int e0 = 512 * c + 8 * lane;
+    if (c < nch && e0 < HD) {
+      float* pw = sPartial + w * per_wave + e0;
+      *(f32x4*)pw = f32x4{dw[c][0], dw[c][1], dw[c][2], dw[c][3]};
+      *(f32x4*)(pw + 4) = f32x4{dw[c][4], dw[c][5], dw[c][6], dw[c][7]};
+      sPartial[w * per_wave + HD + (e0 >> 3)] = accD[c];
+    }
+  }
+  __syncthreads();
+  // the four waves' rows in wave order (a wave without tokens holds zeros)
+  for (int e = tid; e < per_wave; e += 256) {
+    const float tot = (sPartial[e] + sPartial[per_wave + e]) + (sPartial[2 * per_wave + e] + sPartial[3 * per_wave + e]);
+    if (e < HD) A.part_w[(int64_t)blockIdx.x * HD + e] = tot;
+    else A.part_D[(int64_t)blockIdx.x * (HD >> 3) + (e - HD)] = tot;
+  }
+}
+
+// dweight[e] (blocks 0 .. H dv / 64 - 1: one lane per column, the waves' rows added in order) and dD[h] (one wave per head)
+__global__ __launch_bounds__(64) void epilogue_heads_reduce_kernel(EpilogueArgs A, int n_waves /* partial rows */) {
+  const int lane = threadIdx.x;
+  const int dv = A.dv, HD = A.H * dv, n_wblocks = (HD + 63) / 64;
+  if ((int)blockIdx.x < n_wblocks) {
+    const int e = blockIdx.x * 64 + lane;
+    if (e < HD) {
+      float s = 0.f;
+      for (int j = 0; j < n_waves; ++j) s += A.part_w[(int64_t)j * HD + e];
+      A.g.dweight[e] = s;
+    }
+  } else if (A.t.x) {
+    const int h = blockIdx.x - n_wblocks, per = dv >> 3;
+    float s = 0.f;
+    for (int64_t j = lane; j < (int64_t)n_waves * per; j += 64) {
+      const int64_t wv = j / per, slot = j - wv * per;
+      s += A.part_D[wv * (HD >> 3) + (int64_t)h * per + slot];
+    }
+    s = wave_sum(s);
+    if (lane == 0) A.g.dD[h] = s;
+  }
+}
+
+static int heads_waves(const PalGlueDims* d) { return (d->tokens + kHeadsIter - 1) / kHeadsIter; }
+
 static int check_glue_dims(const PalGlueDims* d) {
   if (!d) return PAL_E_NULL;
   if (d->tokens <= 0 || d->n_heads <= 0 || d->n_qk_heads <= 0 || d->n_heads % d->n_qk_heads != 0) return PAL_E_DIM;
@@ -407,14 +625,19 @@ static int check_glue_dims(const PalGlueDims* d) {
   if (d->dk < 8 || d->dk > 256 || d->dk % 8 || d->dv < 8 || d->dv > 256 || d->dv % 8) return PAL_E_HEADDIM;
   if (d->dtype != PAL_DTYPE_BF16 && d->dtype != PAL_DTYPE_F32) return PAL_E_DTYPE;
   if (!(d->eps >= 0.f)) return PAL_E_DIM;
+  if (d->norm_over_heads && (int64_t)d->n_heads * d->dv > 512 * kHeadsMaxCh) return PAL_E_DIM;
+  if (!(d->dt_min <= d->dt_max)) return PAL_E_DIM;   // also refuses NaN bounds
   return PAL_OK;
 }
 
 static int check_prologue(const PalGlueDims* d, const PalPrologueTensors* t) {
   if (int rc = check_glue_dims(d)) return rc;
   if (!t) return PAL_E_NULL;
-  if (!t->q_raw || !t->k_raw || !t->x || !t->dt_raw || !t->bs_raw || !t->dt_bias || !t->q || !t->k || !t->v || !t->gt)
-    return PAL_E_NULL;
+  if (!t->x || !t->dt_raw || !t->dt_bias || !t->v || !t->gt) return PAL_E_NULL;
+  // q, k rows: all four tensors or none (the MetaMamba2 form hands its B, C rows to the operator as they are)
+  const int n_qk = (t->q_raw != nullptr) + (t->k_raw != nullptr) + (t->q != nullptr) + (t->k != nullptr);
+  if (n_qk != 0 && n_qk != 4) return PAL_E_NULL;
+  if (t->bs_raw && n_qk == 0) return PAL_E_NULL;     // the Palimpsa layer's form always has them
   if ((t->b_raw != nullptr) != (t->b != nullptr)) return PAL_E_STATE;
   if (t->b_raw && !t->b_scale) return PAL_E_NULL;
   const void* ptrs[] = {t->q_raw, t->k_raw, t->x, t->b_raw, t->q, t->k, t->v, t->b};
@@ -430,6 +653,9 @@ static void fill_prologue(PrologueArgs& A, const PalGlueDims* d, const PalProlog
   A.GLk = g.GLk; A.GLv = g.GLv; A.tok_per_block = g.tok_per_block;
   A.eps = d->eps;
   A.part = nullptr;
+  A.mamba = t->bs_raw == nullptr;
+  A.task0 = t->q_raw ? 0 : 2;
+  A.dt_min = d->dt_min; A.dt_max = d->dt_max;
 }
 
 static int check_epilogue(const PalGlueDims* d, const PalEpilogueTensors* t) {
@@ -462,7 +688,7 @@ extern "C" int pal_prologue_fwd(const PalGlueDims* d, const PalPrologueTensors* 
   PrologueArgs A{};
   fill_prologue(A, d, t);
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((d->tokens + A.tok_per_block - 1) / A.tok_per_block, d->n_heads, 3);
+  const dim3 grid((d->tokens + A.tok_per_block - 1) / A.tok_per_block, d->n_heads, 3 - A.task0);
   if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernPrologueFwd, s, prologue_fwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
   else PAL_TIMED_LAUNCH(kKernPrologueFwd, s, prologue_fwd_kernel<float>, grid, dim3(256), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
@@ -482,9 +708,9 @@ extern "C" int pal_prologue_bwd(const PalGlueDims* d, const PalPrologueTensors* 
   using namespace pal;
   if (int rc = check_prologue(d, t)) return rc;
   if (!gr) return PAL_E_NULL;
-  if (!gr->dq || !gr->dk || !gr->dv || !gr->dgt || !gr->dq_raw || !gr->dk_raw || !gr->dx || !gr->ddt_raw ||
-      !gr->dbs_raw || !gr->ddt_bias)
-    return PAL_E_NULL;
+  if (!gr->dv || !gr->dgt || !gr->dx || !gr->ddt_raw || !gr->ddt_bias) return PAL_E_NULL;
+  if (t->q_raw && (!gr->dq || !gr->dk || !gr->dq_raw || !gr->dk_raw)) return PAL_E_NULL;
+  if (t->bs_raw && !gr->dbs_raw) return PAL_E_NULL;
   if (t->b_raw && (!gr->db || !gr->db_raw || !gr->db_scale)) return PAL_E_NULL;
   const void* ptrs[] = {gr->dq, gr->dk, gr->dv, gr->db, gr->dq_raw, gr->dk_raw, gr->dx, gr->db_raw, workspace};
   for (const void* p : ptrs)
@@ -496,7 +722,7 @@ extern "C" int pal_prologue_bwd(const PalGlueDims* d, const PalPrologueTensors* 
   A.part = (float*)workspace;
   hipStream_t s = (hipStream_t)stream;
   const int nb = (d->tokens + A.tok_per_block - 1) / A.tok_per_block;
-  const dim3 grid(nb, d->n_heads, 3);
+  const dim3 grid(nb, d->n_heads, 3 - A.task0);
   if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernPrologueBwd, s, prologue_bwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
   else PAL_TIMED_LAUNCH(kKernPrologueBwd, s, prologue_bwd_kernel<float>, grid, dim3(256), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
@@ -511,6 +737,13 @@ extern "C" int pal_epilogue_fwd(const PalGlueDims* d, const PalEpilogueTensors* 
   EpilogueArgs A{};
   fill_epilogue(A, d, t);
   hipStream_t s = (hipStream_t)stream;
+  if (d->norm_over_heads) {
+    const dim3 hgrid((heads_waves(d) + 3) / 4);
+    if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_heads_fwd_kernel<bf16_t>, hgrid, dim3(256), 0, s, A);
+    else PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_heads_fwd_kernel<float>, hgrid, dim3(256), 0, s, A);
+    PAL_HIP_LAUNCH_CHECK();
+    return PAL_OK;
+  }
   const dim3 grid((d->tokens + A.tok_per_block - 1) / A.tok_per_block, d->n_heads);
   if (d->dtype == PAL_DTYPE_BF16) PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_fwd_kernel<bf16_t>, grid, dim3(256), 0, s, A);
   else PAL_TIMED_LAUNCH(kKernEpilogueFwd, s, epilogue_fwd_kernel<float>, grid, dim3(256), 0, s, A);
@@ -521,6 +754,10 @@ extern "C" int pal_epilogue_fwd(const PalGlueDims* d, const PalEpilogueTensors* 
 extern "C" size_t pal_epilogue_bwd_workspace_bytes(const PalGlueDims* d) {
   using namespace pal;
   if (check_glue_dims(d) != PAL_OK) return 0;
+  if (d->norm_over_heads) {
+    const size_t HD = (size_t)d->n_heads * d->dv, nblk = (size_t)((heads_waves(d) + 3) / 4);
+    return up256(sizeof(float) * nblk * HD) + up256(sizeof(float) * nblk * (HD / 8));
+  }
   const GlueGeom g = glue_geom(d);
   const int tpb = (256 / g.GLv) * kGlueIter;
   const size_t nb = (d->tokens + tpb - 1) / tpb;
@@ -542,6 +779,25 @@ extern "C" int pal_epilogue_bwd(const PalGlueDims* d, const PalEpilogueTensors* 
   EpilogueArgs A{};
   fill_epilogue(A, d, t);
   A.g = *gr;
+  if (d->norm_over_heads) {
+    const int nblk = (heads_waves(d) + 3) / 4;
+    const size_t HD = (size_t)d->n_heads * d->dv;
+    A.part_w = (float*)workspace;
+    A.part_D = (float*)((char*)workspace + up256(sizeof(float) * (size_t)nblk * HD));
+    hipStream_t hs = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * 4 * (HD + HD / 8);
+    if (d->dtype == PAL_DTYPE_BF16) {
+      if (int rc = allow_lds((const void*)&epilogue_heads_bwd_kernel<bf16_t>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, epilogue_heads_bwd_kernel<bf16_t>, dim3(nblk), dim3(256), lds, hs, A);
+    } else {
+      if (int rc = allow_lds((const void*)&epilogue_heads_bwd_kernel<float>, lds)) return rc;
+      PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, epilogue_heads_bwd_kernel<float>, dim3(nblk), dim3(256), lds, hs, A);
+    }
+    PAL_HIP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(epilogue_heads_reduce_kernel, dim3((unsigned)((HD + 63) / 64 + d->n_heads)), dim3(64), 0, hs, A, nblk);
+    PAL_HIP_LAUNCH_CHECK();
+    return PAL_OK;
+  }
   const int nb = (d->tokens + A.tok_per_block - 1) / A.tok_per_block;
   A.part_w = (float*)workspace;
   A.part_D = (float*)((char*)workspace + up256(sizeof(float) * (size_t)nb * d->n_heads * d->dv));

@@ -253,6 +253,22 @@ def test_layer_glue_entry_points_reject_bad_arguments(L):
     assert lib.pal_epilogue_bwd(gd(), et(), eg, None, 0, None) == L.PAL_E_WORKSPACE
     assert lib.pal_epilogue_bwd_workspace_bytes(gd()) > 0
 
+    # the MetaMamba2 layer's form: no bs_raw (the multiplier is the clamped time step), q/k rows all present or all absent
+    mamba = dict(bs_raw=None, q_raw=None, k_raw=None, q=None, k=None)
+    assert lib.pal_prologue_fwd(gd(dt_min=0.5, dt_max=0.1), pt(**mamba), None) == L.PAL_E_DIM      # bounds out of order
+    assert lib.pal_prologue_fwd(gd(dt_min=float("nan")), pt(**mamba), None) == L.PAL_E_DIM
+    assert lib.pal_prologue_fwd(gd(), pt(**dict(mamba, k=_fake(0x7000))), None) == L.PAL_E_NULL    # one of the four q/k tensors
+    assert lib.pal_prologue_fwd(gd(), pt(q_raw=None, k_raw=None, q=None, k=None), None) == L.PAL_E_NULL   # bs_raw needs q, k
+    assert lib.pal_prologue_fwd(gd(), pt(**dict(mamba, gt=None)), None) == L.PAL_E_NULL
+    gm = L.PalPrologueGrads(**{n: _fake(0x1000 * (i + 30)) for i, n in enumerate(gnames)
+                               if n not in ("dq", "dk", "dq_raw", "dk_raw", "dbs_raw")})
+    assert lib.pal_prologue_bwd(gd(dt_max=1.0), pt(**mamba), gm, None, 0, None) == L.PAL_E_WORKSPACE   # arguments accepted
+    assert lib.pal_prologue_bwd(gd(), pt(), gm, None, 0, None) == L.PAL_E_NULL                     # the layer form needs them
+    # norm over all heads of a token: up to 4096 entries
+    assert lib.pal_epilogue_fwd(gd(norm_over_heads=1, n_heads=32, n_qk_heads=32, dv=256), et(), None) == L.PAL_E_DIM
+    assert lib.pal_epilogue_bwd(gd(norm_over_heads=1), et(), eg, None, 0, None) == L.PAL_E_WORKSPACE
+    assert lib.pal_epilogue_bwd_workspace_bytes(gd(norm_over_heads=1, tokens=1600)) == 100 * 4 * (256 + 32)   # one row per 16 tokens
+
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     """Without the built library the package raises ImportError with the build instruction; nothing is computed."""

@@ -243,3 +243,141 @@ def test_full_size_headline_shape(gpu_device):
     assert hp.max_abs(y.float(), y_ref.detach()) <= hp.BF16_OUT_ABS_TOL * max(1.0, y_ref.abs().max().item())
     for name, t, r in zip(("o", "x", "D", "gate", "weight"), lv, rv):
         assert hp.max_rel(t.grad, r.grad) <= hp.BF16_GRAD_NORM_TOL, name
+
+
+# ------------------------------------------------------------------ the MetaMamba2 layer's form of the same kernels
+MAMBA_SHAPES = [
+    ((2, 70), 12, 64, torch.bfloat16),      # 768 entries per token: two passes of the wave, the second half full
+    ((1, 33), 6, 48, torch.bfloat16),       # 288 entries: one partial pass
+    ((3, 17), 16, 192, torch.bfloat16),     # 3072 entries
+    ((5,), 2, 256, torch.bfloat16),
+    ((2, 40), 4, 64, torch.float32),
+    ((2, 300), 16, 96, torch.bfloat16),     # more tokens than one workgroup takes
+]
+
+
+@pytest.mark.parametrize("lead,H,dv,dtype", MAMBA_SHAPES)
+@pytest.mark.parametrize("with_b,limit", [(True, (0.0, float("inf"))), (True, (0.05, 0.4)), (False, (0.05, 0.4))])
+def test_mamba_prologue_forward_backward(gpu_device, lead, H, dv, dtype, with_b, limit):
+    from palimpsa_amd.ops.layer_glue import metamamba2_inputs
+    a = _inputs(lead, 1, H, 8, dv, 10, dtype)
+    names = ("x", "dt_raw", "dt_bias", "b_raw", "b_scale")
+    if not with_b:
+        a["b_raw"] = a["b_scale"] = None
+    dev = gpu_device
+    leaves = {n: (None if a[n] is None else a[n].to(dev).clone().requires_grad_(True)) for n in names}
+    outs = metamamba2_inputs(**leaves, dt_limit=limit)
+    ref_leaves = {n: (None if a[n] is None else a[n].double().clone().requires_grad_(True)) for n in names}
+    refs = lo.mamba_prologue(**ref_leaves, dt_limit=limit)
+    out_tol, grad_tol = (hp.BF16_OUT_ABS_TOL, hp.BF16_GRAD_NORM_TOL) if dtype == torch.bfloat16 else (1e-4, 1e-4)
+    gen = torch.Generator().manual_seed(11)
+    loss, loss_ref = 0.0, 0.0
+    for name, y, r in zip(("v", "b", "dt"), outs, refs):
+        if r is None:
+            assert y is None
+            continue
+        assert y.shape == r.shape and y.dtype == (torch.float32 if name == "dt" else dtype), name
+        assert hp.max_abs(y.float(), r) <= out_tol * max(1.0, r.abs().max().item()), name
+        wgt = torch.randn(r.shape, generator=gen).to(y.dtype)
+        loss = loss + (y.float() * wgt.to(dev).float()).sum()
+        loss_ref = loss_ref + (r * wgt.double()).sum()
+    # the clamp is live in the bounded cases: some time steps on either side
+    if limit[1] < 1.0:
+        assert (refs[2] == limit[0]).any() and (refs[2] == limit[1]).any() and ((refs[2] > limit[0]) & (refs[2] < limit[1])).any()
+    loss.backward()
+    loss_ref.backward()
+    for n in names:
+        if a[n] is None:
+            continue
+        g, r = leaves[n].grad, ref_leaves[n].grad
+        assert g.shape == r.shape and g.dtype == leaves[n].dtype, n
+        err = hp.max_rel(g, r)
+        assert err <= grad_tol, (n, err)
+
+
+@pytest.mark.parametrize("lead,H,dv,dtype", MAMBA_SHAPES)
+@pytest.mark.parametrize("residual,gated", [(True, True), (False, True), (True, False), (False, False)])
+def test_mamba_epilogue_forward_backward(gpu_device, lead, H, dv, dtype, residual, gated):
+    from palimpsa_amd.ops.layer_glue import metamamba2_output_norm
+    gen = torch.Generator().manual_seed(12)
+    o = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+    x = torch.randn(*lead, H, dv, generator=gen).to(dtype) if residual else None
+    D = torch.randn(H, generator=gen) if residual else None
+    gate = torch.randn(*lead, H * dv, generator=gen).to(dtype) if gated else None      # the layer's gate is [.., H dv]
+    w = 1.0 + 0.2 * torch.randn(H * dv, generator=gen)
+    dy = torch.randn(*lead, H, dv, generator=gen).to(dtype)
+    dev = gpu_device
+    names = ("o", "x", "D", "gate", "w")
+    vals = dict(o=o, x=x, D=D, gate=gate, w=w)
+    leaves = {n: (None if vals[n] is None else vals[n].to(dev).clone().requires_grad_(True)) for n in names}
+    y = metamamba2_output_norm(leaves["o"], leaves["x"], leaves["D"], leaves["gate"], leaves["w"], 1e-5)
+    ref_leaves = {n: (None if vals[n] is None else vals[n].double().clone().requires_grad_(True)) for n in names}
+    y_ref = lo.mamba_epilogue(ref_leaves["o"], ref_leaves["x"], ref_leaves["D"], ref_leaves["gate"], ref_leaves["w"], 1e-5)
+    out_tol, grad_tol = (hp.BF16_OUT_ABS_TOL, hp.BF16_GRAD_NORM_TOL) if dtype == torch.bfloat16 else (1e-4, 1e-4)
+    assert y.shape == o.shape and y.dtype == dtype
+    assert hp.max_abs(y.float(), y_ref.detach()) <= out_tol * max(1.0, y_ref.abs().max().item())
+    y.backward(dy.to(dev))
+    y_ref.backward(dy.double())
+    for n in names:
+        if vals[n] is None:
+            continue
+        g, r = leaves[n].grad, ref_leaves[n].grad
+        assert g.shape == r.shape and g.dtype == leaves[n].dtype, n
+        err = hp.max_rel(g, r)
+        assert err <= grad_tol, (n, err)
+
+
+def test_mamba_glue_is_reproducible_and_rejects_wide_tokens(gpu_device):
+    from palimpsa_amd.ops.layer_glue import metamamba2_inputs, metamamba2_output_norm
+    dev = gpu_device
+    a = _inputs((3, 500), 1, 12, 8, 64, 13, torch.bfloat16)
+
+    def run():
+        lv = {n: a[n].to(dev).clone().requires_grad_(True) for n in ("x", "dt_raw", "dt_bias", "b_raw", "b_scale")}
+        D = torch.ones(12, device=dev, requires_grad=True)
+        w = torch.ones(768, device=dev, requires_grad=True)
+        v, b, dt = metamamba2_inputs(**lv, dt_limit=(0.0, 0.5))
+        y = metamamba2_output_norm(v * b, lv["x"], D, v, w)
+        (y.float() ** 2).sum().backward()
+        return [y.detach(), dt.detach()] + [t.grad for t in lv.values()] + [D.grad, w.grad]
+
+    for p, q in zip(run(), run()):
+        assert torch.isfinite(p.float()).all() and torch.equal(p, q)      # sums over tokens are taken in a fixed order
+    with pytest.raises(ValueError):
+        metamamba2_output_norm(torch.zeros(2, 32, 256, device=dev), None, None, None, torch.ones(32 * 256, device=dev))
+
+
+def test_mamba_layer_slice_end_to_end(gpu_device):
+    """MetaMamba2.forward between its convolution and out_proj (layers/meta_mamba2.py:276-363): inputs from the
+    projections, the operator with scale = 1 and B, C rows of two groups shared by eight heads, residual + gated norm
+    over the token; forward and all gradients against the oracles chained the same way."""
+    from oracle import palimpsa_oracle as po
+    from palimpsa_amd.ops.layer_glue import metamamba2_inputs, metamamba2_output_norm
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+    dev = gpu_device
+    B, T, H, G, dk, dv = 2, 130, 8, 2, 64, 32
+    gen = torch.Generator().manual_seed(14)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    vals = dict(C=(0.5 * r(B, T, G, dk)).bfloat16(), Bm=(0.5 * r(B, T, G, dk)).bfloat16(), x=r(B, T, H, dv).bfloat16(),
+                dt_raw=(r(B, T, H) - 1.0).bfloat16(), dt_bias=0.3 * r(H), b_raw=r(B, T, H, dv).bfloat16(), b_scale=r(H) + 1.0,
+                A_log=torch.log(torch.arange(1, H + 1).float()), Ip_log=0.2 * r(H), D=1.0 + 0.1 * r(H),
+                gate=r(B, T, H * dv).bfloat16(), w=1.0 + 0.1 * r(H * dv))
+    dy = r(B, T, H, dv).bfloat16()
+
+    lv = {n: t.to(dev).clone().requires_grad_(True) for n, t in vals.items()}
+    v, b, dt = metamamba2_inputs(lv["x"], lv["dt_raw"], lv["dt_bias"], lv["b_raw"], lv["b_scale"], dt_limit=(0.0, 2.0))
+    o = chunk_palimpsa(lv["C"], lv["Bm"], v, b, dt, lv["A_log"].exp(), lv["Ip_log"].exp(), scale=1.0, chunk_size=16)
+    y = metamamba2_output_norm(o, lv["x"], lv["D"], lv["gate"], lv["w"], 1e-5)
+    y.backward(dy.to(dev))
+
+    rl = {n: t.double().clone().requires_grad_(True) for n, t in vals.items()}
+    v_r, b_r, dt_r = lo.mamba_prologue(rl["x"], rl["dt_raw"], rl["dt_bias"], rl["b_raw"], rl["b_scale"], dt_limit=(0.0, 2.0))
+    rep = H // G
+    o_r = po.palimpsa_recurrence(rl["C"].repeat_interleave(rep, dim=2), rl["Bm"].repeat_interleave(rep, dim=2), v_r, b_r,
+                                 dt_r, rl["A_log"].exp(), rl["Ip_log"].exp(), scale=1.0, compute_dtype=torch.float64)[0]
+    y_r = lo.mamba_epilogue(o_r, rl["x"], rl["D"], rl["gate"], rl["w"], 1e-5)
+    y_r.backward(dy.double())
+    assert hp.max_abs(y.float(), y_r.detach()) <= hp.BF16_OUT_ABS_TOL * max(1.0, y_r.abs().max().item())
+    for n in vals:
+        err = hp.max_rel(lv[n].grad, rl[n].grad)
+        assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)

@@ -74,3 +74,45 @@ def test_gradcheck_of_both_functions():
     D = torch.randn(2, generator=gen, dtype=torch.float64).requires_grad_(True)
     w = torch.randn(8, generator=gen, dtype=torch.float64).requires_grad_(True)
     assert torch.autograd.gradcheck(lambda o, x, g, D, w: lo.epilogue(o, x, D, g, w, 1e-5), ts + [D, w], atol=1e-8)
+
+
+def test_mamba_prologue_clamp_and_products():
+    a = _inputs((2, 9), 1, 4, 8, 16, 5)
+    v, b, dt = lo.mamba_prologue(a["x"], a["dt_raw"], a["dt_bias"], a["b_raw"], a["b_scale"], dt_limit=(0.3, 1.2))
+    sp = F.softplus(a["dt_raw"] + a["dt_bias"])
+    assert dt.min() >= 0.3 and dt.max() <= 1.2
+    inside = (sp > 0.3) & (sp < 1.2)
+    assert inside.any() and (~inside).any()
+    assert torch.equal(dt[inside], sp[inside])
+    assert torch.allclose(v, a["x"] * dt[..., None], atol=1e-12)
+    assert torch.allclose(b / dt[..., None] / F.softplus(a["b_scale"]).view(-1, 1), torch.sigmoid(a["b_raw"]), atol=1e-12)
+    # the layer's default limits leave softplus as it is
+    assert torch.equal(lo.mamba_prologue(a["x"], a["dt_raw"], a["dt_bias"])[2], sp)
+    assert lo.mamba_prologue(a["x"], a["dt_raw"], a["dt_bias"])[1] is None
+
+
+def test_mamba_epilogue_reduces_to_library_routines():
+    gen = torch.Generator().manual_seed(6)
+    o = torch.randn(3, 5, 4, 24, generator=gen, dtype=torch.float64)
+    x = torch.randn(3, 5, 4, 24, generator=gen, dtype=torch.float64)
+    g = torch.randn(3, 5, 96, generator=gen, dtype=torch.float64)
+    D = torch.randn(4, generator=gen, dtype=torch.float64)
+    w = torch.randn(96, generator=gen, dtype=torch.float64)
+    eps = 1e-5
+    r = (o + x * D.view(4, 1)).flatten(-2)
+    assert torch.allclose(lo.mamba_epilogue(o, None, None, None, w, eps).flatten(-2), F.rms_norm(o.flatten(-2), (96,), w, eps), atol=1e-12)
+    assert torch.allclose(lo.mamba_epilogue(o, x, D, g, w, eps).flatten(-2), F.rms_norm(r * F.silu(g), (96,), w, eps), atol=1e-12)
+    # the mean square runs over all heads of a token: scaling one head changes the others' outputs
+    o2 = o.clone()
+    o2[..., 0, :] *= 3.0
+    assert not torch.allclose(lo.mamba_epilogue(o2, None, None, None, w, eps)[..., 1, :], lo.mamba_epilogue(o, None, None, None, w, eps)[..., 1, :])
+
+
+def test_mamba_glue_gradcheck():
+    a = _inputs((3,), 1, 2, 8, 8, 7)
+    leaves = [a[n].clone().requires_grad_(True) for n in ("x", "dt_raw", "dt_bias", "b_raw", "b_scale")]
+    assert torch.autograd.gradcheck(lambda *t: lo.mamba_prologue(*t, dt_limit=(0.0, 50.0)), leaves, atol=1e-8)
+    gen = torch.Generator().manual_seed(8)
+    mk = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float64).requires_grad_(True)
+    o, x, g, D, w = mk(3, 2, 8), mk(3, 2, 8), mk(3, 2, 8), mk(2), mk(16)
+    assert torch.autograd.gradcheck(lambda *t: lo.mamba_epilogue(*t, 1e-5), (o, x, D, g, w), atol=1e-8)
