@@ -17,6 +17,7 @@ One JSON line is printed; it also carries
                 headline shape, its tile kernel against the HBM peak
   extra.layer_slice  fused prologue -> chunk_palimpsa -> fused epilogue, forward+backward, on the headline shape
                 (the layer between its projections and o_proj), the prologue backward against the HBM peak
+  extra.mamba_layer_slice  the same for the reference's other caller (MetaMamba2.forward) on its 170M shape
   extra.c0      config 0 (fp32 recurrent forward, B=2 T=256 H=4 d=32), with the CPU port beside it
   extra.c2      config 2 (packed 32768 tokens, lognormal documents, H=16 d=96, chunked forward+backward)
   extra.c4      config 4 (one sequence of 65536 tokens, H=16 d=128, chunked forward with initial and final state)
@@ -426,6 +427,65 @@ def bench_layer_slice(torch, dev, steps, warmup):
                          "algorithmic_bytes_per_launch": bytes_pb, "avg_launch_ms": avg_pb}}
 
 
+def bench_mamba_layer_slice(torch, dev, steps, warmup):
+    """What MetaMamba2.forward does between its convolution and out_proj (layers/meta_mamba2.py:283-363) on the shape
+    of the reference's meta_mamba2_170M configuration (16 heads, head_dim 96, state_size 48, 16 groups): time step,
+    x dt and b dt, the operator with scale 1 on the raw B, C rows, residual and gated norm over the token; fwd+bwd."""
+    from palimpsa_amd import _lib as L
+    from palimpsa_amd.ops.layer_glue import metamamba2_inputs, metamamba2_output_norm
+    from palimpsa_amd.ops.palimpsa import chunk_palimpsa
+
+    B, T, H, G, dk, dv = 8, 2048, 16, 16, 48, 96
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    r = lambda *shape: torch.randn(*shape, generator=gen)
+    bf = torch.bfloat16
+    leaves = dict(C=(0.5 * r(B, T, G, dk)).to(bf), Bm=(0.5 * r(B, T, G, dk)).to(bf), x=r(B, T, H, dv).to(bf),
+                  dt_raw=(r(B, T, H) - 1.0).to(bf), dt_bias=torch.ones(H), b_raw=r(B, T, H, dv).to(bf), b_scale=torch.ones(H),
+                  gate=r(B, T, H * dv).to(bf), weight=torch.ones(H * dv), D=torch.ones(H),
+                  A_log=torch.log(torch.arange(1, H + 1).float()))
+    leaves = {n: v.to(dev).requires_grad_(True) for n, v in leaves.items()}
+    Ip = torch.ones(H, device=dev)
+    dy = r(B, T, H, dv).to(dev, bf)
+
+    def step():
+        for x in leaves.values():
+            x.grad = None
+        v, b, dt = metamamba2_inputs(leaves["x"], leaves["dt_raw"], leaves["dt_bias"], leaves["b_raw"], leaves["b_scale"])
+        o = chunk_palimpsa(leaves["C"], leaves["Bm"], v, b, dt, leaves["A_log"].exp(), Ip, scale=1.0, chunk_size=CHUNK)
+        y = metamamba2_output_norm(o, leaves["x"], leaves["D"], leaves["gate"], leaves["weight"], 1e-5)
+        y.backward(dy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    L.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    kern = L.profile_read()
+    L.profile_enable(False)
+    rows = B * T * H
+    # algorithmic bytes of the epilogue backward: o, x, gate, dy in; d_o, dx, dgate out (bf16 rows)
+    bytes_eb = rows * dv * 2 * 7
+    ms_eb, n_eb = kern.get("epilogue_bwd_kernel", (float("nan"), 1))
+    avg_eb = ms_eb / max(n_eb, 1)
+    achieved = bytes_eb / (avg_eb * 1e-3) / 1e9
+    glue = ("prologue_fwd_kernel", "prologue_bwd_kernel", "epilogue_fwd_kernel", "epilogue_bwd_kernel")
+    return {"workload": "metamamba2 prologue -> chunk_palimpsa (scale 1) -> epilogue over the token, fwd+bwd, "
+                        "B=8 T=2048 H=16 dk=48 dv=96 bf16 (meta_mamba2_170M)",
+            "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms,
+            "glue_kernel_ms_per_step": sum(kern[k][0] for k in glue if k in kern) / steps,
+            "kernels": {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()},
+            "roofline": {"bound": "hbm", "kernel": "epilogue_bwd_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "algorithmic_bytes_per_launch": bytes_eb, "avg_launch_ms": avg_eb}}
+
+
 def bench_c0(torch, dev, steps, warmup, with_cpu):
     """Config 0: fp32 token-serial forward, B=2 T=256 H=4 dk=dv=32, final states returned."""
     from palimpsa_amd.ops.palimpsa import fused_recurrent_palimpsa
@@ -630,6 +690,7 @@ def main():
         extra["simple_gla"] = bench_simple_gla(torch, dev, args.steps, args.warmup)
     if not args.no_layer_slice:
         extra["layer_slice"] = bench_layer_slice(torch, dev, args.steps, args.warmup)
+        extra["mamba_layer_slice"] = bench_mamba_layer_slice(torch, dev, max(args.steps // 2, 1), args.warmup)
     if not args.no_configs:
         short = max(5, min(args.steps, 20))     # 8-10 ms per step
         extra["c0"] = bench_c0(torch, dev, args.steps, args.warmup, not args.no_cpu_baseline)
