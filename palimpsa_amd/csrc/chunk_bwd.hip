@@ -79,8 +79,10 @@ __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2
 // PREC (fp32 rows): every operand is carried as two bf16 halves and every product takes three matrix instructions
 // (split_bf16 / mfma16_split); the LDS slots hold 16 operands instead of 8 and a wave may use 256 registers
 // (two waves per SIMD), so at most 2 column blocks are in flight.
+// Three column blocks (dk = 48) are 12 waves, three per SIMD and one workgroup per compute unit (its LDS): that
+// instance may use 168 registers.
 template <typename TIn, int NB, bool HAS_VAR, bool MULTI, bool PREC>
-__global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(PREC ? 2 : 4)))
+__global__ __launch_bounds__(4 * NB * 64) __attribute__((amdgpu_waves_per_eu(PREC ? 2 : (NB == 3 ? 3 : 4))))
 void chunk_bwd_local_roles_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
