@@ -57,6 +57,8 @@ struct BwdArgs {
 
 constexpr int kVS2 = 68;
 constexpr int kDG2 = 16;
+// local pass: second producer one value row behind the first (see the kernel)
+__host__ __device__ constexpr bool local_lag(int NB, bool prec) { return !prec && NB != 2; }
 
 __device__ __forceinline__ constexpr int lidx2(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
 __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2 * sb + p : 4 + (sb - 2); }
@@ -94,9 +96,18 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
   float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
   float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [2*NB] sums of dJloc (padded to 16 floats)
-  float* sMJ = sRed + NB * kC + 16;      // [NB][2 slots][2][16] tile-start M_0, J_0 of the row in flight
+  // LAG: the second producer runs one value row behind the first and takes the operands of tokens 0..31 from the
+  // first one's slot instead of forming them again (it is the longest role of a row); the consumers follow two rows
+  // behind.  The first producer's half of a slot is then alive for three rows, the second one's for two:
+  //   sX  [NB][3 x {P^M_0, P^J_0, X^M_0, X^J_0} | 2 x {P^M_1, P^J_1, X^M_1, X^J_1}][64 lanes],  sMJ [NB][4 slots][2][16].
+  // Not with two column blocks per workgroup (two such workgroups share a compute unit's LDS) nor with split operands.
+  constexpr bool LAG = local_lag(NB, PREC);
+  constexpr int LAGC = LAG ? 2 : 1;        // rows the consumers run behind the first producer
+  float* sMJ = sRed + NB * kC + 16;      // [NB][2 (LAG: 4) slots][2][16] tile-start M_0, J_0 of the rows in flight
   constexpr int OPN = PREC ? 16 : 8;       // operands per slot (PREC: the lo halves follow the 8 hi halves)
-  bf16x8* sX = (bf16x8*)(sMJ + NB * 64);   // [NB][2 slots][OPN operands][64 lanes]
+  bf16x8* sX = (bf16x8*)(sMJ + NB * (LAG ? 128 : 64));   // [NB][2 slots][OPN operands][64 lanes] (LAG: see above)
+  // [NB][16 rows][4][M 0..3, J 0..3] first column of dM^loc, dJ^loc of a group of value rows (the carry to the previous tile)
+  float* sCar = (float*)(sX + NB * (LAG ? 20 : 2 * OPN) * 64);
   const int tid = threadIdx.x;
   int lane = tid & 63, i = lane & 15, g = lane >> 4;   // re-derived per pass from an opaque copy, see below
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: role branches are scalar
@@ -110,6 +121,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   const float Ip = a.Ip[h];
   const float gh = a.g[h] * kLog2e;
   const float scale = a.scale;
+  const bool fold = !PREC && a.init_mu == nullptr;
 
   if (wave == 0) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
@@ -168,8 +180,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   auto iter_tail = [&](int it) {
     if ((it & 15) == 8 && (it >> 4) + 1 < n_groups) stage((it >> 4) + 1);
     __syncthreads();
-    if (it >= 1 && ((it - 1) & 15) == 15) {
-      const int dg = (it - 1) >> 4;
+    if (it >= LAGC && ((it - LAGC) & 15) == 15) {
+      const int dg = (it - LAGC) >> 4;
       if (st_on && st_s < clen) {
         unsigned off = st_off;
         asm volatile("" : "+v"(off));
@@ -193,16 +205,36 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         store_vec<4>(dvo, sv);
         store_vec<4>(dbo, sb_);
       }
+      // carry handed to the previous tile, f_first * dM^loc at the first token: thread = (column block, row, quad of columns)
+      if (tid < n_act * 64) {
+        const int w = tid >> 6, row = (tid >> 2) & 15, q4 = tid & 3;
+        const float f_first = fast_exp2(sC[0]);
+        const f32x4 cm = *(const f32x4*)&sCar[tid * 8], cj = *(const f32x4*)&sCar[tid * 8 + 4];
+        const float rm[4] = {f_first * cm[0], f_first * cm[1], f_first * cm[2], f_first * cm[3]};
+        const float rj[4] = {f_first * cj[0], f_first * cj[1], f_first * cj[2], f_first * cj[3]};
+        const int64_t co = tile_off + (int64_t)(dg * kDG2 + row) * dk + 16 * (pass * NB + w) + 4 * q4;
+        store_vec<4>((TIn*)A.wDM + co, rm);
+        store_vec<4>((TIn*)A.wDJ + co, rj);
+      }
       __syncthreads();
     }
   };
 
   // ------------------------------------------------------------------ producers
-  auto producer = [&](auto hfc) {
+  // FOLD (bf16 operands, no initial state): the tile-start state rides in the operand of the tile's first token,
+  // X'_0 = X_0 + f_0 (M_0, J_0), since F_t = L[t,0] f_0: the prefix product then yields M_t, J_t without the
+  // two multiply-adds per state entry.  The state is rounded to bf16 there like every other operand; a J_0 below
+  // zero (an initial state with I_0 < Ip) would cancel against Ip, so launches with an initial state keep the fp32 form.
+  auto producer = [&](auto hfc, auto foldc) {
     constexpr int HF = decltype(hfc)::value;   // token blocks 2HF, 2HF+1 (index tl)
+    constexpr bool FOLD = decltype(foldc)::value;
     bf16x8 Lop[HF ? 4 : 2];   // forward operand L[t,s], s <= t: HF=0 [tl], HF=1 [2tl+ks]
     bf16x8 Lol[PREC ? (HF ? 4 : 2) : 1];   // PREC: its lo halves
     float kk[HF ? 16 : 8];    // k in operand layout (n = i, s = 8g+j+32ks)
+    // its square, kept where the registers are there for it (measured: 5 % of the kernel at dk = 64; with several
+    // passes over the tile the loop spills and is 1-2 % slower, there the square is formed per value row)
+    constexpr bool KK2 = !MULTI && NB != 3;
+    float kk2[KK2 ? (HF ? 16 : 8) : 1];
     float qq[8];              // q in result layout (t = 16tb+4g+r, n = i)
     float dq[8];
     float sigacc = 0.f;
@@ -223,6 +255,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           const bool ok = s < clen;
           const float kv = to_f32((kp + (int64_t)(ok ? s : 0) * rs)[i]);
           kk[ks * 8 + j] = ok ? kv : 0.f;
+          if constexpr (KK2) kk2[ks * 8 + j] = kk[ks * 8 + j] * kk[ks * 8 + j];
 #pragma unroll
           for (int tl = 0; tl < 2; ++tl) {
             const int t = 16 * (2 * HF + tl) + i;
@@ -248,14 +281,17 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     const float* cmu = a.chunk_mu + tile_off + 16 * nb;
     const float* cI = a.chunk_I + tile_off + 16 * nb;
     float mu_n = cmu[i], I_n = cI[i];
+    const float f0m = (FOLD && g == 0) ? fast_exp2(sC[0]) : 0.f;   // lanes that hold token 0 of the operands
 
     // The producer of token blocks 2-3 has the longest iteration (both operand halves, twice the matrix instructions):
     // the other three waves of its SIMD finish a row earlier and would leave it to issue alone at half rate, so it
     // gets the issue slots first (measured: 1 % of the kernel; raising both producers or the consumers costs 3-10 %).
     if (HF) __builtin_amdgcn_s_setprio(3);
-    for (int it = 0; it <= dv; ++it) {
-      if (it < dv) {
-        const int d = it, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+    constexpr int LAGP = (LAG && HF) ? 1 : 0;   // rows this producer runs behind the first one
+    int b3 = 0;                                 // LAG: d mod 3, the first producer's slot of the row
+    for (int it = 0; it < dv + LAGC; ++it) {
+      if (it >= LAGP && it - LAGP < dv) {
+        const int d = it - LAGP, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
@@ -267,14 +303,22 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           I_n = (cI + dn)[i];
         }
         const float M0 = mu0 * I0, J0 = I0 - Ip;
+        const float fM = f0m * M0, fJ = f0m * J0;
         if (!HF && g == 0) {
-          sMJ[(nbl * 2 + (d & 1)) * 32 + i] = M0;
-          sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + i] = J0;
+          float* mj = sMJ + (LAG ? nbl * 4 + (d & 3) : nbl * 2 + (d & 1)) * 32;
+          mj[i] = M0;
+          mj[16 + i] = J0;
         }
         bf16x8 XM[HF + 1], XJ[HF + 1];
         bf16x8 XMl[PREC ? HF + 1 : 1], XJl[PREC ? HF + 1 : 1];
 #pragma unroll
         for (int ks = 0; ks <= HF; ++ks) {
+          if (LAG && HF && ks == 0) {   // tokens 0..31: as the first producer left them a row ago
+            const bf16x8* p0 = sX + (nbl * 20 + 4 * b3) * 64 + lane;
+            XM[0] = p0[2 * 64];
+            XJ[0] = p0[3 * 64];
+            continue;
+          }
           const f32x4 v0 = *(const f32x4*)&sV[8 * g + 32 * ks];
           const f32x4 v1 = *(const f32x4*)&sV[8 * g + 32 * ks + 4];
           const f32x4 b0 = *(const f32x4*)&sB[8 * g + 32 * ks];
@@ -296,8 +340,11 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
             const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
             const float ka = kk[ks * 8 + j], kb = kk[ks * 8 + j + 1];
-            const bf16x2 pm = pack2(ka * va, kb * vb);
-            const bf16x2 pj = pack2((ka * ba) * ka, (kb * bb) * kb);
+            const bool tok0 = FOLD && ks == 0 && j == 0;
+            const bf16x2 pm = pack2(tok0 ? fmaf(ka, va, fM) : ka * va, kb * vb);
+            const float kab = KK2 ? kk2[ks * 8 + j] : ka * ba, kbb = KK2 ? kk2[ks * 8 + j + 1] : kb * bb;
+            const float ja = KK2 ? ba : ka, jb = KK2 ? bb : kb;
+            const bf16x2 pj = pack2(tok0 ? fmaf(kab, ja, fJ) : kab * ja, kbb * jb);
             XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
             XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
           }
@@ -325,15 +372,16 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             accI = mfma16(Lop[2 * tl + HF], XJ[HF], accI);
           }
           }
-          const f32x4 Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
+          f32x4 Fv = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (!FOLD) Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
           const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
           f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
           if (HAS_VAR) dvv = *(const f32x4*)&sDov[16 * tb + 4 * g];
           float dMl[4], dJl[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float Mf = fmaf(Fv[r], M0, accM[r]);
-            const float If = fmaf(Fv[r], J0, accI[r]);
+            const float Mf = FOLD ? accM[r] : fmaf(Fv[r], M0, accM[r]);
+            const float If = FOLD ? accI[r] : fmaf(Fv[r], J0, accI[r]);
             const float rI = fast_rcp(If);
             const float mu = Mf * rI;
             const float q = qq[tl * 4 + r];
@@ -346,7 +394,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
               dJl[r] = fmaf(-w, rI, dJl[r]);
               dq[tl * 4 + r] = fmaf(2.f * wq, rI, dq[tl * 4 + r]);
             }
-            sigacc += dJl[r];
+            if constexpr (PREC) sigacc += dJl[r];
           }
           const int o4 = tl * 4;
           if constexpr (PREC) {
@@ -355,10 +403,19 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           } else {
           const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
           const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
+          // the sum of dJloc (for dIp) from the packed pairs: one instruction per two entries
+          const bf16x2 one2 = {(bf16_t)1.f, (bf16_t)1.f};
+          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j0, one2, sigacc, false);
+          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j1, one2, sigacc, false);
           PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
           PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
           }
         }
+        if constexpr (LAG) {
+          bf16x8* mine = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;
+          mine[0] = PM; mine[64] = PJ; mine[2 * 64] = XM[HF]; mine[3 * 64] = XJ[HF];
+          b3 = (b3 == 2) ? 0 : b3 + 1;
+        } else {
         bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
         if constexpr (PREC) {
           bf16x8 PMl, PJl;
@@ -369,6 +426,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         }
         slot[(0 + HF) * 64] = PM; slot[(2 + HF) * 64] = PJ;
         slot[(4 + HF) * 64] = XM[HF]; slot[(6 + HF) * 64] = XJ[HF];
+        }
       }
       iter_tail(it);
     }
@@ -387,8 +445,9 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   };
 
   // ------------------------------------------------------------------ consumers
-  auto consumer = [&](auto hfc) {
+  auto consumer = [&](auto hfc, auto foldc) {
     constexpr int HF = decltype(hfc)::value;   // column-token blocks 2HF, 2HF+1 (index sl)
+    constexpr bool FOLD = decltype(foldc)::value;   // the operands of token 0 carry f_0 (M_0, J_0), see the producers
     bf16x8 Lop[6];    // reverse operand, HF=0 [2sl+p], HF=1 [sl] (p=1); strictly-lower operand, HF=0 [4+sl], HF=1 [2+2sl+ks]
     bf16x8 Lol[PREC ? 6 : 1];   // PREC: its lo halves
     float kr[8];      // k in result layout (s = 16sb+i, n = 4g+r)
@@ -411,7 +470,11 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
           for (int sl = 0; sl < 2; ++sl) {
             const int t = 16 * (2 * HF + sl) + i;
-            const float lv = (s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
+            float lv = (s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
+            // the last contraction slot of the wave's range (token 31 / 63) is never below a column token of the
+            // wave: it carries the tile-start state instead, with the decay F_t from the start of the tile
+            // (FOLD: the product has the state already, through token 0, for every column token but token 0 itself)
+            if (!PREC && ks == HF && g == 3 && j == 7) lv = (FOLD && t != 0) ? 0.f : fast_exp2(ct[sl]);
             const bf16_t lh = (bf16_t)lv;
             Lop[HF ? 2 + 2 * sl + ks : 4 + sl][j] = lh;
             if constexpr (PREC) Lol[HF ? 2 + 2 * sl + ks : 4 + sl][j] = (bf16_t)(lv - (float)lh);
@@ -447,33 +510,48 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         Fs[sl] = sF[16 * (2 * HF + sl) + i];
       }
     }
-    const float f_first = fast_exp2(sC[0]);
     // the carries between tiles are kept in the dtype of the rows: bf16 rows feed them to the matrix cores in bf16
-    // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers
-    TIn* wDM = (TIn*)A.wDM + tile_off + 16 * nb;
-    TIn* wDJ = (TIn*)A.wDJ + tile_off + 16 * nb;
+    // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers.  The consumer of the
+    // first column token parks them per group of value rows; the flush of the group scales and stores them.
+    float* car = sCar + ((nbl * kDG2) * 4 + g) * 8;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
     float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
 
-    for (int it = 0; it <= dv; ++it) {
-      if (it >= 1) {
-        const int d = it - 1, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+    int b3 = 0;   // LAG: d mod 3
+    for (int it = 0; it < dv + LAGC; ++it) {
+      if (it >= LAGC) {
+        const int d = it - LAGC, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
+        const bf16x8* p0 = sX + (nbl * 20 + 4 * b3) * 64 + lane;              // LAG: the first producer's operands
+        const bf16x8* p1 = sX + (nbl * 20 + 12 + 4 * (d & 1)) * 64 + lane;    //      the second producer's
+        const float* mj = sMJ + (LAG ? nbl * 4 + (d & 3) : nbl * 2 + (d & 1)) * 32;
+        if constexpr (LAG) b3 = (b3 == 2) ? 0 : b3 + 1;
         // HF=0 (column tokens 0..31): reverse needs both P halves, strictly-lower only X_0;
         // HF=1 (column tokens 32..63): reverse needs P_1 only, strictly-lower both X halves
-        const bf16x8 PM1 = slot[1 * 64], PJ1 = slot[3 * 64], XM0 = slot[4 * 64], XJ0 = slot[6 * 64];
-        const bf16x8 Ma = slot[(HF ? 5 : 0) * 64];   // HF=0: P^M_0, HF=1: X^M_1
-        const bf16x8 Ja = slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
+        const bf16x8 PM1 = LAG ? p1[0] : slot[1 * 64], PJ1 = LAG ? p1[64] : slot[3 * 64];
+        bf16x8 XM0 = LAG ? p0[2 * 64] : slot[4 * 64], XJ0 = LAG ? p0[3 * 64] : slot[6 * 64];
+        bf16x8 Ma = LAG ? (HF ? p1[2 * 64] : p0[0]) : slot[(HF ? 5 : 0) * 64];    // HF=0: P^M_0, HF=1: X^M_1
+        bf16x8 Ja = LAG ? (HF ? p1[3 * 64] : p0[64]) : slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
         bf16x8 PM1l, PJ1l, XM0l, XJ0l, Mal, Jal;     // PREC: the lo halves of the six
         if constexpr (PREC) {
           PM1l = slot[(8 + 1) * 64]; PJ1l = slot[(8 + 3) * 64]; XM0l = slot[(8 + 4) * 64]; XJ0l = slot[(8 + 6) * 64];
           Mal = slot[(8 + (HF ? 5 : 0)) * 64];
           Jal = slot[(8 + (HF ? 7 : 2)) * 64];
         }
-        const f32x4 M0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 4 * g];
-        const f32x4 J0T = *(const f32x4*)&sMJ[(nbl * 2 + (d & 1)) * 32 + 16 + 4 * g];
+        f32x4 M0T, J0T;
+        if constexpr (PREC) {
+          M0T = *(const f32x4*)&mj[4 * g];
+          J0T = *(const f32x4*)&mj[16 + 4 * g];
+        } else if (!(FOLD && HF)) {
+          // tile-start state of the row as the virtual token of the strictly-lower product: element 7 of the lanes
+          // g = 3 of its last operand (token 31 / 63 of the contraction, which no column token of this wave uses)
+          const bf16x2 mj2 = pack2(mj[i], mj[16 + i]);
+          if (g == 3) {
+            if (HF) { Ma[7] = mj2[0]; Ja[7] = mj2[1]; } else { XM0[7] = mj2[0]; XJ0[7] = mj2[1]; }
+          }
+        }
         float dvp[2], dbp[2];
 #pragma unroll
         for (int sl = 0; sl < 2; ++sl) {
@@ -522,8 +600,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             dbs = fmaf(aJ[r] * kv, kv, dbs);
             dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
             dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
-            const float Ss = fmaf(Fs[sl], M0T[r], sM[r]);
-            const float SJ = fmaf(Fs[sl], J0T[r], sJ[r]);
+            const float Ss = PREC ? fmaf(Fs[sl], M0T[r], sM[r]) : sM[r];
+            const float SJ = PREC ? fmaf(Fs[sl], J0T[r], sJ[r]) : sJ[r];
             gm = fmaf(aM[r], Ss, gm);
             gm = fmaf(aJ[r], SJ, gm);
           }
@@ -531,11 +609,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           dvp[sl] = dvs;
           dbp[sl] = dbs;
           if (!HF && sl == 0 && i == 0) {
-            // carry handed to the previous tile: f_first * dM^loc at the first token
-            const f32x4 rm = {f_first * aM[0], f_first * aM[1], f_first * aM[2], f_first * aM[3]};
-            const f32x4 rj = {f_first * aJ[0], f_first * aJ[1], f_first * aJ[2], f_first * aJ[3]};
-            store_vec<4>(wDM + (int64_t)d * dk + 4 * g, (const float*)&rm);
-            store_vec<4>(wDJ + (int64_t)d * dk + 4 * g, (const float*)&rj);
+            *(f32x4*)&car[dd * 32] = aM;
+            *(f32x4*)&car[dd * 32 + 4] = aJ;
           }
         }
         pw[dd * kC] = rows4_sum_x4(dvp[0], dvp[1], dbp[0], dbp[1]);
@@ -572,11 +647,18 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     stage(0);
     __syncthreads();
     if (MULTI && nbl >= n_act) {
-      for (int it = 0; it <= dv; ++it) iter_tail(it);
-    } else if (role == 0) producer(std::integral_constant<int, 0>{});
-    else if (role == 1) producer(std::integral_constant<int, 1>{});
-    else if (role == 2) consumer(std::integral_constant<int, 0>{});
-    else consumer(std::integral_constant<int, 1>{});
+      for (int it = 0; it < dv + LAGC; ++it) iter_tail(it);
+    } else if (fold) {
+      if constexpr (!PREC) {
+        if (role == 0) producer(std::integral_constant<int, 0>{}, std::true_type{});
+        else if (role == 1) producer(std::integral_constant<int, 1>{}, std::true_type{});
+        else if (role == 2) consumer(std::integral_constant<int, 0>{}, std::true_type{});
+        else consumer(std::integral_constant<int, 1>{}, std::true_type{});
+      }
+    } else if (role == 0) producer(std::integral_constant<int, 0>{}, std::false_type{});
+    else if (role == 1) producer(std::integral_constant<int, 1>{}, std::false_type{});
+    else if (role == 2) consumer(std::integral_constant<int, 0>{}, std::false_type{});
+    else consumer(std::integral_constant<int, 1>{}, std::false_type{});
     __syncthreads();
     if (tid < kC) {
 #pragma unroll
@@ -1112,8 +1194,10 @@ struct BwdPlan {
 };
 
 static size_t local_lds_bytes(int NB, bool var, bool prec) {
-  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 + NB * 64) +
-         (size_t)NB * 2 * (prec ? 16 : 8) * 64 * 16;
+  const bool lag = local_lag(NB, prec);
+  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 +
+                          NB * (lag ? 128 : 64) + NB * kDG2 * 32) +
+         (size_t)NB * (lag ? 20 : 2 * (prec ? 16 : 8)) * 64 * 16;
 }
 
 // prec: the fp32-accurate variants (fp32 rows without PAL_FLAG_FP32_FAST)
