@@ -82,7 +82,11 @@ __device__ __forceinline__ void seq_lookup(const ChunkArgs& a, int n, int& bos, 
 // is an absolute error far below that of the bf16 rows).  The sums then hold M 2^-(ek+ev) and J 2^-(2ek+eb); the
 // tile-start state enters with the same factors and mu = M / I is put right once per output by 2^(ev-ek-eb), so the
 // scaling costs nothing per state entry.  A tensor that is all zero (or holds inf/nan) gets exponent 0.
-// Every thread of the workgroup calls this (it synchronises); sMax is LDS scratch of 3 floats per wave.
+// With st_mu, st_I (the sn4 groups of four consecutive entries of the tile-start state that the workgroup uses, as
+// (mu, I)) the exponents also make room for the state, which the caller adds to the operands of the tile's first
+// token: ev and eb are raised until |M_0| 2^-(ek+ev) and I_0 2^-(2ek+eb) stay below 2^14 (the rows then sit lower in
+// the f16 range; what they lose is small against the state they are added to).
+// Every thread of the workgroup calls this (it synchronises); sMax is LDS scratch of 5 floats per wave.
 struct TileExponents { int ek, ev, eb; };
 
 __device__ __forceinline__ int block_exponent_of(float m, int target) {
@@ -94,8 +98,18 @@ __device__ __forceinline__ int block_exponent_of(float m, int target) {
 template <typename TIn>
 __device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, const TIn* vt, const TIn* bt, int Hq, int H,
                                                               int dk, int dv, int clen, int tid, int nthreads,
-                                                              float* sMax, int v0 = 0, int vn = 0) {
-  float km = 0.f, vm = 0.f, bm = 0.f;
+                                                              float* sMax, int v0 = 0, int vn = 0,
+                                                              const float* st_mu = nullptr, const float* st_I = nullptr,
+                                                              int sn4 = 0) {
+  float km = 0.f, vm = 0.f, bm = 0.f, mm = 0.f, im = 0.f;
+  if (st_mu) {
+#pragma unroll 4
+    for (int idx = tid; idx < sn4; idx += nthreads) {
+      const f32x4 m = *(const f32x4*)(st_mu + 4 * (int64_t)idx), y = *(const f32x4*)(st_I + 4 * (int64_t)idx);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { mm = fmaxf(mm, fabsf(m[e] * y[e])); im = fmaxf(im, fabsf(y[e])); }
+    }
+  }
   const int gk = dk >> 3, gv = (vn > 0 ? vn : dv) >> 3;
   vt += v0;
   bt += v0;
@@ -124,16 +138,24 @@ __device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, con
   km = wave_max(km);
   vm = wave_max(vm);
   bm = wave_max(bm);
+  if (st_mu) { mm = wave_max(mm); im = wave_max(im); }
   const int w = tid >> 6, nw = (nthreads + 63) >> 6;
-  if ((tid & 63) == 0) { sMax[3 * w] = km; sMax[3 * w + 1] = vm; sMax[3 * w + 2] = bm; }
+  if ((tid & 63) == 0) {
+    sMax[5 * w] = km; sMax[5 * w + 1] = vm; sMax[5 * w + 2] = bm; sMax[5 * w + 3] = mm; sMax[5 * w + 4] = im;
+  }
   __syncthreads();
-  km = 0.f; vm = 0.f; bm = 0.f;
-  for (int x = 0; x < nw; ++x) { km = fmaxf(km, sMax[3 * x]); vm = fmaxf(vm, sMax[3 * x + 1]); bm = fmaxf(bm, sMax[3 * x + 2]); }
+  km = 0.f; vm = 0.f; bm = 0.f; mm = 0.f; im = 0.f;
+  for (int x = 0; x < nw; ++x) {
+    km = fmaxf(km, sMax[5 * x]); vm = fmaxf(vm, sMax[5 * x + 1]); bm = fmaxf(bm, sMax[5 * x + 2]);
+    mm = fmaxf(mm, sMax[5 * x + 3]); im = fmaxf(im, sMax[5 * x + 4]);
+  }
   __syncthreads();
   TileExponents e;
   e.ek = block_exponent_of(km, 0);
   e.ev = block_exponent_of(vm, 11);
   e.eb = block_exponent_of(bm, 11);
+  if (mm > 0.f && mm < __builtin_inff()) e.ev = max(e.ev, ilogbf(mm) - 13 - e.ek);
+  if (im > 0.f && im < __builtin_inff()) e.eb = max(e.eb, ilogbf(im) - 13 - 2 * e.ek);
   return e;
 }
 

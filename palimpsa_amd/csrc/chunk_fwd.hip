@@ -323,6 +323,16 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(ChunkArgs a) {
 constexpr int kVH = 72;  // row stride (f16) of the transposed, block-scaled v/b staging tiles of chunk_out_kernel
 constexpr int kDG = 16;  // value rows per staging group
 
+// Adds the tile-start state (already under the block exponents; zero in the lanes that do not hold token 0) to the
+// first element of the operands of tokens 0..7: the first pair becomes a packed multiply-add instead of a multiply.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void fold_state(f16x8& XM, f16x8& XJ, f16x8 kA, f16x8 vv, f16x8 kk, f16x8 bb, float m0, float i0) {
+  const f16x2 am = {(f16_t)m0, (f16_t)0.f}, aj = {(f16_t)i0, (f16_t)0.f};
+  const f16x2 xm = __builtin_elementwise_fma(kA.xy, vv.xy, am), xj = __builtin_elementwise_fma(kk.xy, bb.xy, aj);
+  XM[0] = xm[0]; XM[1] = xm[1];
+  XJ[0] = xj[0]; XJ[1] = xj[1];
+}
+
 // index of the L operand for (tb, ks): tb0,tb1 -> one K step; tb2,tb3 -> two
 __device__ __forceinline__ constexpr int lidx(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
 
@@ -415,9 +425,16 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   }
   stage_load(0);
   // block exponents of the f16 operands (see tile_block_exponents); sO doubles as its scratch
+  // FOLD (f16 operands): the tile-start state rides in the operands of the tile's first token, X'_0 = X_0 + f_0 (M_0, I_0)
+  // under the block exponents (F_t = L[t,0] f_0, and I_t = (1 - F_t) Ip + F_t I_0 + J-sum has no negative term), so the
+  // prefix products yield M_t and I_t without two multiply-adds per state entry; the exponents make room for the state.
+  constexpr bool FOLD = !PREC;
+  const float* st_mu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk;
+  const float* st_I = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk;
   TileExponents bexp = {0, 0, 0};
   if constexpr (!PREC)
-    bexp = tile_block_exponents((const TIn*)a.k + qk_row(a, t0, h), vp, bp, a.Hq, H, dk, dv, clen, tid, NT, sO);
+    bexp = tile_block_exponents((const TIn*)a.k + qk_row(a, t0, h), vp, bp, a.Hq, H, dk, dv, clen, tid, NT, sO, 0, 0,
+                                st_mu, st_I, dv * dk / 4);
   const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
   const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
   const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
@@ -490,11 +507,25 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   // mu = M / I comes out times 2^(ek+eb-ev) and 1 / I times 2^(2ek+eb): put right once per output
   const float scale = ((a.scale * __builtin_amdgcn_exp2f((float)bexp.ev)) * down_k) * down_b;
   const float scale_var = ((a.scale * down_k) * down_k) * down_b;
-  const float* cmu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
-  const float* cI = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk + 16 * nb + 4 * g;
+  const float* cmu = st_mu + 16 * nb + 4 * g;
+  const float* cI = st_I + 16 * nb + 4 * g;
+  // FOLD: the entry of the wave's own key column i instead (operand layout); the lanes that hold token 0 of the
+  // operands (g = 0) carry the factor f_0 2^-(ek+ev) resp. f_0 2^-(2ek+eb), the others zero
+  const float* cmu1 = st_mu + 16 * nb + i;
+  const float* cI1 = st_I + 16 * nb + i;
+  const float f0 = (FOLD && g == 0) ? fast_exp2(sC[0]) : 0.f;
+  const float c0m = (f0 * down_k) * down_v, c0j = ((f0 * down_k) * down_k) * down_b;
 
   // tile-start state of the next value row is fetched one iteration ahead
-  f32x4 mu0_n = *(const f32x4*)(cmu + (int64_t)rs * dk), I0_n = *(const f32x4*)(cI + (int64_t)rs * dk);
+  f32x4 mu0_n = {0.f, 0.f, 0.f, 0.f}, I0_n = {0.f, 0.f, 0.f, 0.f};
+  float mu1_n = 0.f, I1_n = 0.f;
+  if constexpr (FOLD) {
+    mu1_n = cmu1[(int64_t)rs * dk];
+    I1_n = cI1[(int64_t)rs * dk];
+  } else {
+    mu0_n = *(const f32x4*)(cmu + (int64_t)rs * dk);
+    I0_n = *(const f32x4*)(cI + (int64_t)rs * dk);
+  }
   const int n_groups = dv / kDG;
   for (int dg = 0; dg < n_groups; ++dg) {
     const int buf = dg & 1;
@@ -506,10 +537,16 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
         stage_store(buf ^ 1);
       }
       const f32x4 mu0 = mu0_n, I0 = I0_n;
+      const float mu1 = mu1_n, I1 = I1_n;
       {
         const int64_t dn = (int64_t)min(d + RS, dv - 1) * dk;
-        mu0_n = *(const f32x4*)(cmu + dn);
-        I0_n = *(const f32x4*)(cI + dn);
+        if constexpr (FOLD) {
+          mu1_n = cmu1[dn];
+          I1_n = cI1[dn];
+        } else {
+          mu0_n = *(const f32x4*)(cmu + dn);
+          I0_n = *(const f32x4*)(cI + dn);
+        }
       }
       float M0[4];
 #pragma unroll
@@ -528,8 +565,11 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
           split_bf16(xb, XJh[ks], XJl[ks]);
         } else {
           // 8 consecutive tokens of the row: one 16-byte LDS read each; packed f16 products are the operands
-          XM[ks] = kA[ks] * *(const f16x8*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
-          XJ[ks] = kk[ks] * *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+          const f16x8 vv = *(const f16x8*)&sV[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+          const f16x8 bb = *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
+          XM[ks] = kA[ks] * vv;
+          XJ[ks] = kk[ks] * bb;
+          if (FOLD && ks == 0) fold_state(XM[0], XJ[0], kA[0], vv, kk[0], bb, (c0m * mu1) * I1, c0j * I1);
         }
       }
       float p[4], pv[4];
@@ -555,8 +595,8 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
         float acc = 0.f, accv = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float Mf = fmaf(Fm[tb], M0[r], accM[r]);
-          const float If = fmaf(Fj[tb], I0[r], accI[r]);
+          const float Mf = FOLD ? accM[r] : fmaf(Fm[tb], M0[r], accM[r]);
+          const float If = FOLD ? accI[r] : fmaf(Fj[tb], I0[r], accI[r]);
           const float rI = fast_rcp(If);
           acc = fmaf(Mf * rI, qD[tb][r], acc);
           if (HAS_VAR) accv = fmaf(qD[tb][r] * qD[tb][r], rI, accv);
@@ -645,7 +685,11 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
     q_next = *(const bf16x4*)(qbase + 16 * nb + kq_off);
   };
   request(0);
-  const TileExponents bexp = tile_block_exponents(kbase, vp - r0, bp - r0, a.Hq, H, dk, dv, clen, tid, 256, sO, r0, rn);
+  constexpr bool FOLD = true;   // the tile-start state rides in the operands of the first token, see chunk_out_kernel
+  const float* st_mu = a.chunk_mu + (((int64_t)cidx * H + h) * dv + r0) * dk;
+  const float* st_I = a.chunk_I + (((int64_t)cidx * H + h) * dv + r0) * dk;
+  const TileExponents bexp = tile_block_exponents(kbase, vp - r0, bp - r0, a.Hq, H, dk, dv, clen, tid, 256, sO, r0, rn,
+                                                  st_mu, st_I, rn * dk / 4);
   const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
   const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
   const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
@@ -707,9 +751,11 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
   const float scale_var = ((a.scale * down_k) * down_k) * down_b;
 
   const int n_blocks = dk >> 4;
-  const float* cmu0 = a.chunk_mu + (((int64_t)cidx * H + h) * dv + r0) * dk + 4 * g;
-  const float* cI0 = a.chunk_I + (((int64_t)cidx * H + h) * dv + r0) * dk + 4 * g;
-  f32x4 mu0_n = *(const f32x4*)(cmu0 + (int64_t)w * dk), I0_n = *(const f32x4*)(cI0 + (int64_t)w * dk);
+  const float* cmu0 = st_mu + i;   // the entry of the lane's key column i of a block (operand layout)
+  const float* cI0 = st_I + i;
+  const float f0 = (g == 0) ? fast_exp2(sC[0]) : 0.f;   // lanes that hold token 0 of the operands
+  const float c0m = (f0 * down_k) * down_v, c0j = ((f0 * down_k) * down_k) * down_b;
+  float mu1_n = cmu0[(int64_t)w * dk], I1_n = cI0[(int64_t)w * dk];
 #pragma unroll 1
   for (int nb = 0; nb < n_blocks; ++nb) {
     const int buf = nb & 1;
@@ -732,13 +778,13 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
     const float* cI = cI0 + 16 * nb;
 #pragma unroll 1
     for (int d = w; d < rn; d += 4) {
-      const f32x4 mu0 = mu0_n, I0 = I0_n;
+      const float mu1 = mu1_n, I1 = I1_n;
       {
         // the state row of the next iteration: the wave's next row, or its first row of the next column block
         const bool last = d + 4 >= rn;
         const int64_t dn = last ? (int64_t)w * dk + (more ? 16 : 0) : (int64_t)(d + 4) * dk;
-        mu0_n = *(const f32x4*)(cmu + dn);
-        I0_n = *(const f32x4*)(cI + dn);
+        mu1_n = cmu[dn];
+        I1_n = cI[dn];
       }
       float* so = sO + d * kC + 16 * g + i;
       float* sov = sOv + d * kC + 16 * g + i;
@@ -747,14 +793,15 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
         prev = *so;
         if (HAS_VAR) prevv = *sov;
       }
-      float M0[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) M0[r] = mu0[r] * I0[r];
+      const float M0[4] = {0.f, 0.f, 0.f, 0.f}, I0[4] = {0.f, 0.f, 0.f, 0.f};   // (the state is in the operands)
       f16x8 XM[2], XJ[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        XM[ks] = kA[ks] * *(const f16x8*)&sV[d * kVH + 8 * g + 32 * ks];
-        XJ[ks] = kk[ks] * *(const f16x8*)&sB[d * kVH + 8 * g + 32 * ks];
+        const f16x8 vv = *(const f16x8*)&sV[d * kVH + 8 * g + 32 * ks];
+        const f16x8 bb = *(const f16x8*)&sB[d * kVH + 8 * g + 32 * ks];
+        XM[ks] = kA[ks] * vv;
+        XJ[ks] = kk[ks] * bb;
+        if (ks == 0) fold_state(XM[0], XJ[0], kA[0], vv, kk[0], bb, (c0m * mu1) * I1, c0j * I1);
       }
       float p[4], pv[4];
 #pragma unroll
@@ -770,8 +817,8 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
         float acc = 0.f, accv = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float Mf = fmaf(Fm[tb], M0[r], accM[r]);
-          const float If = fmaf(Fj[tb], I0[r], accI[r]);
+          const float Mf = FOLD ? accM[r] : fmaf(Fm[tb], M0[r], accM[r]);
+          const float If = FOLD ? accI[r] : fmaf(Fj[tb], I0[r], accI[r]);
           const float rI = fast_rcp(If);
           acc = fmaf(Mf * rI, qD[tb][r], acc);
           if (HAS_VAR) accv = fmaf(qD[tb][r] * qD[tb][r], rI, accv);

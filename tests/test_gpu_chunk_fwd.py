@@ -167,6 +167,45 @@ def test_block_exponent_of_the_f16_operands(gpu_device, v_scale, k_scale):
     assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
 
 
+@pytest.mark.parametrize("d", [64, 96])
+@pytest.mark.parametrize("case", ["rows_shrink", "large_initial_state", "precision_below_prior", "rows_grow"])
+def test_tile_start_state_in_the_first_token_operands(gpu_device, d, case):
+    """The output kernels add the tile-start state to the f16 operands of a tile's first token and make room for it in
+    the block exponents.  Cases where the state and the rows of a tile are far apart, for both kernel layouts
+    (d = 64: by key columns, d = 96: by value rows): rows that shrink by 1e5 half way (the state then dwarfs them),
+    an initial state 1e4 above the rows, an initial precision far below the prior (I_t = (1 - F_t) Ip + F_t I_0 + ...
+    has no cancelling term), rows that grow by 1e4 (the state is then small against them)."""
+    ck, _ = _ops()
+    B, T, H = 1, 320, 2
+    inp = po.make_inputs(B, T, H, d, d, seed=123)
+    inp["g"] = torch.tensor([0.01, 0.2])     # slow decay: the state outlives the tiles
+    gen = torch.Generator().manual_seed(124)
+    kw = {}
+    if case == "rows_shrink":
+        inp["v"][:, T // 2:] *= 1.0e-5
+        inp["b"][:, T // 2:] *= 1.0e-5
+    elif case == "rows_grow":
+        inp["v"][:, T // 2:] *= 1.0e4
+        inp["b"][:, T // 2:] *= 1.0e4
+    elif case == "large_initial_state":
+        kw = dict(mu0=torch.randn(B, H, d, d, generator=gen) * 30.0, I0=1.0 + 300.0 * torch.rand(B, H, d, d, generator=gen))
+    else:
+        kw = dict(mu0=torch.randn(B, H, d, d, generator=gen), I0=0.01 + 0.04 * torch.rand(B, H, d, d, generator=gen))
+    inp = hp.rounded(inp, torch.bfloat16)
+    dev_kw = {}
+    if kw:
+        dev_kw = dict(initial_mu_state=kw["mu0"].to(gpu_device), initial_I_state=kw["I0"].to(gpu_device))
+    (o, ov), mu, I = _call(ck, hp.to_device(inp, gpu_device), output_final_state=True, output_uncertainty=True,
+                           chunk_size=64, **dev_kw)
+    o_ref, ov_ref, mu_ref, I_ref = hp.oracle_forward(inp, want_var=True, **kw)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(ov.float()).all()
+    # per half of the sequence: the halves differ by orders of magnitude in two of the cases
+    for sl in (slice(0, T // 2), slice(T // 2, T)):
+        assert hp.max_rel(o[:, sl], o_ref[:, sl]) <= 1e-2
+        assert hp.max_rel(ov[:, sl], ov_ref[:, sl]) <= 1e-2
+    assert hp.max_rel(mu, mu_ref) <= STATE_REL_TOL and hp.max_rel(I, I_ref) <= STATE_REL_TOL
+
+
 def test_windowed_no_grad_forward_equals_single_call(gpu_device, monkeypatch):
     """A single long sequence without autograd is run in windows of tiles through the state
     (no tile-start states for the whole sequence); same kernels, same tiles, so the results agree
