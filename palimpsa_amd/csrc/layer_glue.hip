@@ -593,26 +593,53 @@ __global__ __launch_bounds__(256) void epilogue_heads_bwd_kernel(EpilogueArgs A)
   }
 }
 
-// dweight[e] (blocks 0 .. H dv / 64 - 1: one lane per column, the waves' rows added in order) and dD[h] (one wave per head)
-__global__ __launch_bounds__(64) void epilogue_heads_reduce_kernel(EpilogueArgs A, int n_waves /* partial rows */) {
-  const int lane = threadIdx.x;
+// dweight[e] (blocks 0 .. H dv / 64 - 1: 64 columns per block) and dD[h] (one block per head) from the partial rows of
+// the backward kernel.  16 waves per block: wave w adds the rows j = w (mod 16) in order, four loads in flight, and
+// the waves' sums are added in order, so the result does not depend on timing (one wave per block walked the rows
+// alone before: 0.24 ms at 1024 partial rows).
+constexpr int kRedWaves = 16;
+__global__ __launch_bounds__(64 * kRedWaves) void epilogue_heads_reduce_kernel(EpilogueArgs A, int n_waves /* partial rows */) {
+  __shared__ float sPart[kRedWaves][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int dv = A.dv, HD = A.H * dv, n_wblocks = (HD + 63) / 64;
+  float s = 0.f;
   if ((int)blockIdx.x < n_wblocks) {
     const int e = blockIdx.x * 64 + lane;
     if (e < HD) {
-      float s = 0.f;
-      for (int j = 0; j < n_waves; ++j) s += A.part_w[(int64_t)j * HD + e];
-      A.g.dweight[e] = s;
+      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+      int j = w;
+      for (; j + 3 * kRedWaves < n_waves; j += 4 * kRedWaves) {
+        s0 += A.part_w[(int64_t)j * HD + e];
+        s1 += A.part_w[(int64_t)(j + kRedWaves) * HD + e];
+        s2 += A.part_w[(int64_t)(j + 2 * kRedWaves) * HD + e];
+        s3 += A.part_w[(int64_t)(j + 3 * kRedWaves) * HD + e];
+      }
+      for (; j < n_waves; j += kRedWaves) s0 += A.part_w[(int64_t)j * HD + e];
+      s = (s0 + s1) + (s2 + s3);
+    }
+    sPart[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && e < HD) {
+      float t = 0.f;
+#pragma unroll
+      for (int x = 0; x < kRedWaves; ++x) t += sPart[x][lane];
+      A.g.dweight[e] = t;
     }
   } else if (A.t.x) {
     const int h = blockIdx.x - n_wblocks, per = dv >> 3;
-    float s = 0.f;
-    for (int64_t j = lane; j < (int64_t)n_waves * per; j += 64) {
+    for (int64_t j = threadIdx.x; j < (int64_t)n_waves * per; j += 64 * kRedWaves) {
       const int64_t wv = j / per, slot = j - wv * per;
       s += A.part_D[wv * (HD >> 3) + (int64_t)h * per + slot];
     }
     s = wave_sum(s);
-    if (lane == 0) A.g.dD[h] = s;
+    if (lane == 0) sPart[w][0] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float t = 0.f;
+#pragma unroll
+      for (int x = 0; x < kRedWaves; ++x) t += sPart[x][0];
+      A.g.dD[h] = t;
+    }
   }
 }
 
@@ -794,7 +821,7 @@ extern "C" int pal_epilogue_bwd(const PalGlueDims* d, const PalEpilogueTensors* 
       PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, epilogue_heads_bwd_kernel<float>, dim3(nblk), dim3(256), lds, hs, A);
     }
     PAL_HIP_LAUNCH_CHECK();
-    hipLaunchKernelGGL(epilogue_heads_reduce_kernel, dim3((unsigned)((HD + 63) / 64 + d->n_heads)), dim3(64), 0, hs, A, nblk);
+    hipLaunchKernelGGL(epilogue_heads_reduce_kernel, dim3((unsigned)((HD + 63) / 64 + d->n_heads)), dim3(64 * kRedWaves), 0, hs, A, nblk);
     PAL_HIP_LAUNCH_CHECK();
     return PAL_OK;
   }
