@@ -47,11 +47,11 @@ CHUNK = 64
 # per launch at the headline shape, times 64 lanes, divided by tokens*H*dk*dv
 # (profiles/bench_c1.sq_counters_pmc.txt).  Like the traffic figures below they cannot be read from inside this
 # process and are stale once those kernels change.
-VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 31.7, "chunk_out_kernel": 8.0}
+VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 23.5, "chunk_out_kernel": 6.2}
 # HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
 # from inside this process, so the figures are carried here and are stale once those kernels change.
-MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 456.2e6, "recurrent_fwd_kernel": 1111.8e6,
+MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 424.6e6, "recurrent_fwd_kernel": 1111.8e6,
                           # profiles/bench_simple_gla__layer_slice.hbm_traffic_pmc.txt
                           "gla_out_kernel": 141.2e6, "gla_recurrent_fwd_kernel": 543.4e6, "prologue_bwd_kernel": 305.9e6}
 
