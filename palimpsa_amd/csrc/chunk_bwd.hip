@@ -74,8 +74,11 @@ __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2
 //     columns, form dMloc/dJloc and dq, and leave packed bf16 operands in an LDS slot:
 //     role 0 writes P^M_0, P^J_0, X^M_0, X^J_0 (tokens 0..31), role 1 the halves for tokens 32..63;
 //   roles 2/3 ("consumers", token blocks 0-1 / 2-3 of the column token s): pick the slot up one iteration
-//     later and do the reverse contraction, the strictly-lower product and the dv/db/dk/gate epilogue.
+//     later (two with the lagged second producer, see LAG below) and do the reverse contraction, the
+//     strictly-lower product and the dv/db/dk/gate epilogue.
 // Every role has its own loop (its own register allocation) with the same sequence of barriers.
+// The tile-start state (M_0, J_0) of a value row reaches the products through the operands: see FOLD at the
+// producers and the virtual token at the consumers.
 // NB <= 4 column blocks are in flight at a time (16 waves); a wider head dim takes several passes over
 // the tile, the later ones adding their dv/db/gate contributions to those of the earlier ones.
 // PREC (fp32 rows): every operand is carried as two bf16 halves and every product takes three matrix instructions
