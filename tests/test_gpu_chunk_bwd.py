@@ -138,6 +138,21 @@ def test_bf16_gates_and_slow_decay(gpu_device):
     _compare(grads, ref, NAMES, inp=inp, dg_l1=True)
 
 
+@pytest.mark.parametrize("dk,dv", [(64, 64), (48, 96)])
+def test_state_far_above_the_increments_in_the_backward(gpu_device, dk, dv):
+    """The tile kernel of the backward takes the tile-start state through the bf16 operand of a tile's first token.
+    Nearly non-forgetting heads over 24 tiles: the state (J grows with every token) is then two orders of magnitude
+    above a token's own increment, and every gradient still meets the bf16 bar."""
+    B, T, H = 1, 1500, 2
+    inp = hp.rounded(po.make_inputs(B, T, H, dk, dv, seed=41), torch.bfloat16)
+    inp["g"] = torch.tensor([0.002, 0.05])
+    gen = torch.Generator().manual_seed(42)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    ref = hp.oracle_grads(inp, do)
+    grads = _run_bwd(inp, gpu_device, do)
+    _compare(grads, ref, NAMES, inp=inp, dg_l1=True)
+
+
 def test_c1_shape_backward_subset(gpu_device):
     """Config 1 at full size on the GPU (B=8,T=2048,H=12,d=64,bf16); the float64 oracle with autograd
     checks one (batch, head) pair at full T (entries are independent)."""
