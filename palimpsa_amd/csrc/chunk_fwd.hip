@@ -685,7 +685,7 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
     q_next = *(const bf16x4*)(qbase + 16 * nb + kq_off);
   };
   request(0);
-  constexpr bool FOLD = true;   // the tile-start state rides in the operands of the first token, see chunk_out_kernel
+  // the tile-start state rides in the operands of the first token, see FOLD in chunk_out_kernel
   const float* st_mu = a.chunk_mu + (((int64_t)cidx * H + h) * dv + r0) * dk;
   const float* st_I = a.chunk_I + (((int64_t)cidx * H + h) * dv + r0) * dk;
   const TileExponents bexp = tile_block_exponents(kbase, vp - r0, bp - r0, a.Hq, H, dk, dv, clen, tid, 256, sO, r0, rn,
@@ -722,13 +722,11 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
   __syncthreads();
 
   // per-wave constants of the tile (see chunk_out_kernel)
-  float Fm[4], Fj[4], Gi[4], ct[4];
+  float Gi[4], ct[4];
 #pragma unroll
   for (int tb = 0; tb < 4; ++tb) {
     ct[tb] = sC[16 * tb + i];
     const float F = fast_exp2(ct[tb]);
-    Fm[tb] = (F * down_k) * down_v;
-    Fj[tb] = ((F * down_k) * down_k) * down_b;
     Gi[tb] = ((((1.f - F) * Ip) * down_k) * down_k) * down_b;
   }
   f16x8 Lr[6];
@@ -793,7 +791,6 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
         prev = *so;
         if (HAS_VAR) prevv = *sov;
       }
-      const float M0[4] = {0.f, 0.f, 0.f, 0.f}, I0[4] = {0.f, 0.f, 0.f, 0.f};   // (the state is in the operands)
       f16x8 XM[2], XJ[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
@@ -817,10 +814,8 @@ __global__ __launch_bounds__(256, 3) void chunk_out_rows_kernel(ChunkArgs a, int
         float acc = 0.f, accv = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float Mf = FOLD ? accM[r] : fmaf(Fm[tb], M0[r], accM[r]);
-          const float If = FOLD ? accI[r] : fmaf(Fj[tb], I0[r], accI[r]);
-          const float rI = fast_rcp(If);
-          acc = fmaf(Mf * rI, qD[tb][r], acc);
+          const float rI = fast_rcp(accI[r]);
+          acc = fmaf(accM[r] * rI, qD[tb][r], acc);
           if (HAS_VAR) accv = fmaf(qD[tb][r] * qD[tb][r], rI, accv);
         }
         p[tb] = acc;
