@@ -286,9 +286,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     float mu_n = cmu[i], I_n = cI[i];
     const float f0m = (FOLD && g == 0) ? fast_exp2(sC[0]) : 0.f;   // lanes that hold token 0 of the operands
 
-    // The producer of token blocks 2-3 has the longest iteration (both operand halves, twice the matrix instructions):
+    // The producer of token blocks 2-3 has the longest iteration (twice the matrix instructions of the other one):
     // the other three waves of its SIMD finish a row earlier and would leave it to issue alone at half rate, so it
-    // gets the issue slots first (measured: 1 % of the kernel; raising both producers or the consumers costs 3-10 %).
+    // gets the issue slots first (measured: 3.5 % of the kernel; the same or an intermediate priority for the other
+    // producer, or none at all, are all slower).
     if (HF) __builtin_amdgcn_s_setprio(3);
     constexpr int LAGP = (LAG && HF) ? 1 : 0;   // rows this producer runs behind the first one
     int b3 = 0;                                 // LAG: d mod 3, the first producer's slot of the row
