@@ -100,8 +100,9 @@ __device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, con
                                                               int dk, int dv, int clen, int tid, int nthreads,
                                                               float* sMax, int v0 = 0, int vn = 0,
                                                               const float* st_mu = nullptr, const float* st_I = nullptr,
-                                                              int sn4 = 0) {
-  float km = 0.f, vm = 0.f, bm = 0.f, mm = 0.f, im = 0.f;
+                                                              int sn4 = 0, float mm0 = 0.f, float im0 = 0.f) {
+  // (mm0, im0: the thread's maxima of |M_0| and I_0 where the caller has read its share of the state already)
+  float km = 0.f, vm = 0.f, bm = 0.f, mm = mm0, im = im0;
   if (st_mu) {
 #pragma unroll 4
     for (int idx = tid; idx < sn4; idx += nthreads) {
@@ -138,7 +139,8 @@ __device__ __forceinline__ TileExponents tile_block_exponents(const TIn* kt, con
   km = wave_max(km);
   vm = wave_max(vm);
   bm = wave_max(bm);
-  if (st_mu) { mm = wave_max(mm); im = wave_max(im); }
+  mm = wave_max(mm);
+  im = wave_max(im);
   const int w = tid >> 6, nw = (nthreads + 63) >> 6;
   if ((tid & 63) == 0) {
     sMax[5 * w] = km; sMax[5 * w + 1] = vm; sMax[5 * w + 2] = bm; sMax[5 * w + 3] = mm; sMax[5 * w + 4] = im;

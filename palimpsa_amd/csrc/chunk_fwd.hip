@@ -326,11 +326,21 @@ constexpr int kDG = 16;  // value rows per staging group
 // Adds the tile-start state (already under the block exponents; zero in the lanes that do not hold token 0) to the
 // first element of the operands of tokens 0..7: the first pair becomes a packed multiply-add instead of a multiply.
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void fold_state(f16x8& XM, f16x8& XJ, f16x8 kA, f16x8 vv, f16x8 kk, f16x8 bb, float m0, float i0) {
-  const f16x2 am = {(f16_t)m0, (f16_t)0.f}, aj = {(f16_t)i0, (f16_t)0.f};
+__device__ __forceinline__ void fold_state_pairs(f16x8& XM, f16x8& XJ, f16x8 kA, f16x8 vv, f16x8 kk, f16x8 bb, f16x2 am,
+                                                 f16x2 aj) {
   const f16x2 xm = __builtin_elementwise_fma(kA.xy, vv.xy, am), xj = __builtin_elementwise_fma(kk.xy, bb.xy, aj);
   XM[0] = xm[0]; XM[1] = xm[1];
   XJ[0] = xj[0]; XJ[1] = xj[1];
+}
+__device__ __forceinline__ void fold_state(f16x8& XM, f16x8& XJ, f16x8 kA, f16x8 vv, f16x8 kk, f16x8 bb, float m0, float i0) {
+  const f16x2 am = {(f16_t)m0, (f16_t)0.f}, aj = {(f16_t)i0, (f16_t)0.f};
+  fold_state_pairs(XM, XJ, kA, vv, kk, bb, am, aj);
+}
+// chunk_out_kernel keeps the workgroup's tile-start state in LDS (f16) where it is small: at most four column blocks
+// (and, at run time, at most 64 value rows); floats of LDS that takes per (tile, head)
+__host__ __device__ constexpr bool out_state_cache(int NB, bool prec) { return !prec && NB <= 4; }
+__host__ __device__ constexpr int out_state_cache_floats(int NB, bool prec) {
+  return out_state_cache(NB, prec) ? (2 * 64 * 16 * NB * 2) / 4 + 4 : 0;
 }
 
 // index of the L operand for (tb, ks): tb0,tb1 -> one K step; tb2,tb3 -> two
@@ -351,7 +361,12 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   extern __shared__ float smem[];
   using TSt = std::conditional_t<PREC, float, f16_t>;   // element type of the staged v, b rows
   constexpr int NT = NB * RS * 64;        // threads per (tile, head)
-  constexpr int kTileFloats = kC + (HAS_VAR ? 2 : 1) * NB * kDG * kC + (4 * kDG * kVH * (int)sizeof(TSt)) / 4;
+  // CACHE (f16 operands, at most four column blocks, at most 64 value rows): the workgroup's tile-start state is read
+  // once, for the maxima that the block exponents need, and then kept in LDS as the f16 numbers that the first
+  // token's operands take (M_0 f_0 2^-(ek+ev), I_0 f_0 2^-(2ek+eb)), followed by a zero word for the lanes that add nothing
+  constexpr bool CACHE = out_state_cache(NB, PREC);
+  constexpr int kCacheFloats = out_state_cache_floats(NB, PREC);
+  constexpr int kTileFloats = kC + (HAS_VAR ? 2 : 1) * NB * kDG * kC + (4 * kDG * kVH * (int)sizeof(TSt)) / 4 + kCacheFloats;
   const int sub = TS == 1 ? 0 : (int)threadIdx.x / NT;
   const int tid = (int)threadIdx.x - sub * NT;
   const int64_t n_items = (int64_t)a.total_chunks * a.H;
@@ -363,6 +378,9 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   TSt* sB = sV + 2 * kDG * kVH;           // [2][16][kVH] b^T 2^-E
   float* sO = (float*)(sB + 2 * kDG * kVH);   // [NB][16][64] per-wave partial outputs
   float* sOv = sO + NB * kDG * kC;        // same for o_var
+  f16_t* sStM = (f16_t*)(sC + (kTileFloats - kCacheFloats));   // [dv <= 64][dk] CACHE: see above
+  f16_t* sStI = sStM + 64 * 16 * NB;
+  f16_t* sZero = sStI + 64 * 16 * NB;
   const int lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int nb = RS == 1 ? (tid >> 6) : (tid >> 6) % NB, rs = RS == 1 ? 0 : (tid >> 6) / NB;
   const int H = a.H, dk = a.dk, dv = a.dv;
@@ -431,10 +449,33 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   constexpr bool FOLD = !PREC;
   const float* st_mu = a.chunk_mu + (((int64_t)cidx * H + h) * dv) * dk;
   const float* st_I = a.chunk_I + (((int64_t)cidx * H + h) * dv) * dk;
+  const bool cache = CACHE && dv <= 64;
+  float stm[CACHE ? 16 : 1], sti[CACHE ? 16 : 1];   // CACHE: the thread's share of the state, M_0 = mu_0 I_0 and I_0
+  float mm0 = 0.f, im0 = 0.f;
+  if constexpr (CACHE) {
+    if (cache) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int idx = tid + p * NT;
+        f32x4 m = {0.f, 0.f, 0.f, 0.f}, y = {0.f, 0.f, 0.f, 0.f};
+        if (idx < dv * dk / 4) {
+          m = *(const f32x4*)(st_mu + 4 * (int64_t)idx);
+          y = *(const f32x4*)(st_I + 4 * (int64_t)idx);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          stm[4 * p + e] = m[e] * y[e];
+          sti[4 * p + e] = y[e];
+          mm0 = fmaxf(mm0, fabsf(stm[4 * p + e]));
+          im0 = fmaxf(im0, fabsf(y[e]));
+        }
+      }
+    }
+  }
   TileExponents bexp = {0, 0, 0};
   if constexpr (!PREC)
     bexp = tile_block_exponents((const TIn*)a.k + qk_row(a, t0, h), vp, bp, a.Hq, H, dk, dv, clen, tid, NT, sO, 0, 0,
-                                st_mu, st_I, dv * dk / 4);
+                                cache ? nullptr : st_mu, st_I, dv * dk / 4, mm0, im0);
   const float down_k = __builtin_amdgcn_exp2f(-(float)bexp.ek);
   const float down_v = __builtin_amdgcn_exp2f(-(float)bexp.ev);
   const float down_b = __builtin_amdgcn_exp2f(-(float)bexp.eb);
@@ -453,6 +494,24 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
     }
   };
   stage_store(0);
+  if constexpr (CACHE) {
+    if (cache) {
+      const float f0u = fast_exp2(sC[0]);   // written before the barriers of the exponent pass
+      const float cm = (f0u * down_k) * down_v, cj = ((f0u * down_k) * down_k) * down_b;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int idx = tid + p * NT;
+        if (idx < dv * dk / 4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sStM[4 * idx + e] = (f16_t)(cm * stm[4 * p + e]);
+            sStI[4 * idx + e] = (f16_t)(cj * sti[4 * p + e]);
+          }
+        }
+      }
+      if (tid == 0) { sZero[0] = (f16_t)0.f; sZero[1] = (f16_t)0.f; }
+    }
+  }
   __syncthreads();
 
   // ---- per-wave constants of this tile
@@ -519,9 +578,15 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
   // tile-start state of the next value row is fetched one iteration ahead
   f32x4 mu0_n = {0.f, 0.f, 0.f, 0.f}, I0_n = {0.f, 0.f, 0.f, 0.f};
   float mu1_n = 0.f, I1_n = 0.f;
+  // CACHE: the lanes of token 0 walk the cached state by rows, the others stay on the zero word
+  const f16_t* chM = (g == 0) ? sStM + 16 * nb + i : sZero;
+  const f16_t* chI = (g == 0) ? sStI + 16 * nb + i : sZero;
+  const int ch_stride = (g == 0) ? dk : 0;
   if constexpr (FOLD) {
-    mu1_n = cmu1[(int64_t)rs * dk];
-    I1_n = cI1[(int64_t)rs * dk];
+    if (!cache) {
+      mu1_n = cmu1[(int64_t)rs * dk];
+      I1_n = cI1[(int64_t)rs * dk];
+    }
   } else {
     mu0_n = *(const f32x4*)(cmu + (int64_t)rs * dk);
     I0_n = *(const f32x4*)(cI + (int64_t)rs * dk);
@@ -541,8 +606,10 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
       {
         const int64_t dn = (int64_t)min(d + RS, dv - 1) * dk;
         if constexpr (FOLD) {
-          mu1_n = cmu1[dn];
-          I1_n = cI1[dn];
+          if (!cache) {
+            mu1_n = cmu1[dn];
+            I1_n = cI1[dn];
+          }
         } else {
           mu0_n = *(const f32x4*)(cmu + dn);
           I0_n = *(const f32x4*)(cI + dn);
@@ -569,7 +636,16 @@ __global__ __launch_bounds__(NB * RS * TS * 64, 2) void chunk_out_kernel(ChunkAr
           const f16x8 bb = *(const f16x8*)&sB[(buf * kDG + dd) * kVH + 8 * g + 32 * ks];
           XM[ks] = kA[ks] * vv;
           XJ[ks] = kk[ks] * bb;
-          if (FOLD && ks == 0) fold_state(XM[0], XJ[0], kA[0], vv, kk[0], bb, (c0m * mu1) * I1, c0j * I1);
+          if (FOLD && ks == 0) {
+            if (cache) {
+              // a 16-bit read leaves {value, 0} in the register: the addend pair as it is
+              const f16x2 am = __builtin_bit_cast(f16x2, (uint32_t)*(const unsigned short*)(chM + d * ch_stride));
+              const f16x2 aj = __builtin_bit_cast(f16x2, (uint32_t)*(const unsigned short*)(chI + d * ch_stride));
+              fold_state_pairs(XM[0], XJ[0], kA[0], vv, kk[0], bb, am, aj);
+            } else {
+              fold_state(XM[0], XJ[0], kA[0], vv, kk[0], bb, (c0m * mu1) * I1, c0j * I1);
+            }
+          }
         }
       }
       float p[4], pv[4];
@@ -879,7 +955,8 @@ static int launch_out_rows(const ChunkArgs& a, hipStream_t s) {
 template <typename TIn, int NB, bool PREC>
 static int launch_out_nb_p(const ChunkArgs& a, hipStream_t s) {
   const bool var = a.flags & PAL_FLAG_HAS_VAR;
-  const size_t lds = sizeof(float) * (kC + (var ? 2 : 1) * NB * kDG * kC) + 4 * (PREC ? sizeof(float) : sizeof(f16_t)) * kDG * kVH;
+  const size_t lds = sizeof(float) * (kC + (var ? 2 : 1) * NB * kDG * kC + out_state_cache_floats(NB, PREC)) +
+                     4 * (PREC ? sizeof(float) : sizeof(f16_t)) * kDG * kVH;
   const int64_t blocks = (int64_t)a.total_chunks * a.H;
   if (blocks > 0x7fffffff) return PAL_E_DIM;
   if (lds > kMaxLds) return PAL_E_HEADDIM;
