@@ -36,6 +36,7 @@ struct StatePassArgs {
   const float *init_a, *init_b;
   float *fin_a, *fin_b;
   int32_t ds, nsplit, reverse, per_xcd, total;
+  int32_t dks, ksplit;    // key columns per workgroup and slices of the key columns (dk = dks * ksplit)
   float fin_scale;
 };
 
@@ -52,12 +53,14 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
   extern __shared__ float smem[];
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int H = a.H, dk = a.dk, dv = a.dv, ds = A.ds;
+  const int H = a.H, dk = a.dk, dv = a.dv, ds = A.ds, dks = A.dks;
   // consecutive workgroup ids go to different XCDs: give the slices of one (sequence, head) to the same one,
   // they read the same key rows
   const int m = ((int)blockIdx.x & 7) * A.per_xcd + ((int)blockIdx.x >> 3);
   if (m >= A.total) return;
-  const int nh = m / A.nsplit, d0 = (m % A.nsplit) * ds;
+  // a workgroup owns the state entries (value rows [d0, d0 + ds)) x (key columns [k0, k0 + dks))
+  const int n_sl = A.nsplit * A.ksplit, sl = m % n_sl;
+  const int nh = m / n_sl, d0 = (sl / A.ksplit) * ds, k0 = (sl % A.ksplit) * dks;
   const int h = nh % H, n = nh / H;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
@@ -65,10 +68,10 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
 
   float* sA = smem;                                   // [3][64] weight of token s in its tile (ring over tiles)
   float* sF = sA + 3 * kC;                            // [3] decay over the whole tile (+1 pad)
-  uint32_t* sKT = (uint32_t*)(sF + 4);                // [2][dk][36] words = [dk][72] bf16
-  uint32_t* sVT = sKT + 2 * dk * (kStTS / 2);         // [2][ds][36]
+  uint32_t* sKT = (uint32_t*)(sF + 4);                // [2][dks][36] words = [dks][72] bf16
+  uint32_t* sVT = sKT + 2 * dks * (kStTS / 2);        // [2][ds][36]
   uint32_t* sBT = sVT + 2 * ds * (kStTS / 2);         // [2][ds][36] (HAS_J)
-  const int kbuf = dk * (kStTS / 2), vbuf = ds * (kStTS / 2);
+  const int kbuf = dks * (kStTS / 2), vbuf = ds * (kStTS / 2);
 
 
   // Waves 0-3 own the state (a 16x16 block per wave and slot), waves 4-11 feed them: a single wave issues an
@@ -86,7 +89,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
     const int grp = (w - 4) >> 2;           // parity of the tiles this group stages
     const int wg = (w - 4) & 3;             // wave in the group
     const int st = tid - 256 - 256 * grp;
-    const int gk = dk >> 3, gv = ds >> 3;
+    const int gk = dks >> 3, gv = ds >> 3;
     int ksp[NIK];
     uint32_t koff[NIK][2], kdst[NIK];
     bool kval[NIK];
@@ -96,8 +99,8 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
       kval[j] = idx < 32 * gk;
       ksp[j] = idx / gk;
       const int c8 = idx - ksp[j] * gk;
-      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * a.Hq * dk + 8 * c8) * 2) : 0x80000000u;
-      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * a.Hq * dk + 8 * c8) * 2) : 0x80000000u;
+      koff[j][0] = kval[j] ? (uint32_t)(((2 * ksp[j]) * a.Hq * dk + k0 + 8 * c8) * 2) : 0x80000000u;
+      koff[j][1] = kval[j] ? (uint32_t)(((2 * ksp[j] + 1) * a.Hq * dk + k0 + 8 * c8) * 2) : 0x80000000u;
       kdst[j] = (uint32_t)(8 * c8 * (kStTS / 2) + ksp[j]);
     }
     const int vtid = st, btid = (st + 256 - 32 * gv) & 255;
@@ -224,7 +227,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
 
   // ------------------------------------------------------------------ state role
   // state blocks of this wave: block sb = w + 4 jj -> (value rows 16 db.., key columns 16 nb..)
-  const int NB = dk >> 4, NSB = (ds >> 4) * NB;
+  const int NB = dks >> 4, NSB = (ds >> 4) * NB;
   int ldk[kStMaxBlocks], ldv[kStMaxBlocks], goff[kStMaxBlocks];   // operand rows in the staging tiles, entry in a state
   bool sval[kStMaxBlocks];
   f32x4 accM[kStMaxBlocks], accJ[kStMaxBlocks];
@@ -238,7 +241,7 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
     // rows n = 16 nb + 4 g + r (four consecutive key columns), column d = d0 + 16 db + i
     ldk[jj] = (16 * nb + i) * kStTS + 8 * g;
     ldv[jj] = (16 * db + i) * kStTS + 8 * g;
-    goff[jj] = (d0 + 16 * db + i) * dk + 16 * nb + 4 * g;
+    goff[jj] = (d0 + 16 * db + i) * dk + k0 + 16 * nb + 4 * g;
     accM[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
     accJ[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (sval[jj] && A.init_a) {
@@ -329,13 +332,19 @@ static int launch_state_pass_t(const StatePassArgs& A, int kern_id, unsigned gri
 
 template <bool HAS_J>
 static int launch_state_pass_j(const StatePassArgs& A, int kern_id, unsigned grid, size_t lds, hipStream_t s) {
-  switch ((A.c.dk + 63) / 64) {
+  switch ((A.dks + 63) / 64) {
     case 1: return launch_state_pass_t<HAS_J, 1>(A, kern_id, grid, lds, s);
     case 2: return launch_state_pass_t<HAS_J, 2>(A, kern_id, grid, lds, s);
     case 3: return launch_state_pass_t<HAS_J, 3>(A, kern_id, grid, lds, s);
     case 4: return launch_state_pass_t<HAS_J, 4>(A, kern_id, grid, lds, s);
     default: return PAL_E_HEADDIM;
   }
+}
+
+// key columns per workgroup of the one-pass form, see launch_state_pass
+static int state_pass_key_slice(const ChunkArgs& a, int ds) {
+  if (ds == 16 && a.dk % 128 == 0 && (int64_t)a.n_seqs * a.H * (a.dv / 16) < 192) return 64;
+  return a.dk;
 }
 
 // Whether the one-pass form serves this call: bf16 rows, and enough (sequence, head, slice) workgroups that
@@ -348,7 +357,7 @@ bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j) {
   if (a.flags & PAL_FLAG_STATES_ONE_PASS) return true;
   // The walk over the tiles is serial per workgroup (0.4-0.7 us per tile): with fewer workgroups than this the
   // two-kernel form, which spreads the tiles over the whole GPU, is faster.
-  return (int64_t)a.n_seqs * a.H * (a.dv / 16) >= 192;
+  return (int64_t)a.n_seqs * a.H * (a.dv / 16) * (a.dk / state_pass_key_slice(a, 16)) >= 192;
 }
 
 // tiles_a / tiles_b, init_*, fin_*: see StatePassArgs.  reverse walks every sequence from its last tile.
@@ -370,16 +379,25 @@ int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tile
     if (a.dv % c || c * a.dk > 256 * 4 * kStMaxBlocks) continue;
     if ((int64_t)a.n_seqs * a.H * (a.dv / c) >= 192) { ds = c; break; }
   }
+  // key columns per workgroup: all of them, unless even slices of 16 value rows leave the GPU short of workgroups and
+  // the key columns can be halved into slices of 64 (measured at one sequence of 16 heads, 128x128: 128 workgroups
+  // 102 us per 64 tiles, 256 workgroups of 16 x 64 entries 72 us, the two-kernel form 96 us; slices of 32 columns or
+  // 32 x 32 entries are slower again, and with enough workgroups splitting the columns gains nothing)
+  const int dks = state_pass_key_slice(a, ds);
+  if (ds * dks > 256 * 4 * kStMaxBlocks) return PAL_E_HEADDIM;
   A.ds = ds;
   A.nsplit = a.dv / ds;
-  const int64_t total = (int64_t)a.n_seqs * a.H * A.nsplit;
+  A.dks = dks;
+  A.ksplit = a.dk / dks;
+  const int n_sl = A.nsplit * A.ksplit;
+  const int64_t total = (int64_t)a.n_seqs * a.H * n_sl;
   if (total <= 0) return PAL_OK;
   int64_t per_xcd = (total + 7) / 8;
-  per_xcd = (per_xcd + A.nsplit - 1) / A.nsplit * A.nsplit;
+  per_xcd = (per_xcd + n_sl - 1) / n_sl * n_sl;
   if (per_xcd * 8 > 0x7fffffff) return PAL_E_DIM;
   A.total = (int32_t)total;
   A.per_xcd = (int32_t)per_xcd;
-  const size_t lds = sizeof(float) * (3 * kC + 4) + (size_t)2 * 2 * kStTS * (a.dk + ds * (has_j ? 2 : 1));
+  const size_t lds = sizeof(float) * (3 * kC + 4) + (size_t)2 * 2 * kStTS * (dks + ds * (has_j ? 2 : 1));
   if (lds > kMaxLds) return PAL_E_HEADDIM;
   const unsigned grid = (unsigned)(per_xcd * 8);
   return has_j ? launch_state_pass_j<true>(A, kern_id, grid, lds, s) : launch_state_pass_j<false>(A, kern_id, grid, lds, s);

@@ -45,7 +45,7 @@ def _run_palimpsa(inp, mu0, I0, cu, grads):
     return out
 
 
-@pytest.mark.parametrize("case", ["batched", "varlen_ragged", "wide_heads", "init_state_grads"])
+@pytest.mark.parametrize("case", ["batched", "varlen_ragged", "wide_heads", "init_state_grads", "key_slices"])
 def test_palimpsa_forms_agree(gpu_device, state_pass_mode, case):
     dev = gpu_device
     cu = mu0 = I0 = None
@@ -55,8 +55,13 @@ def test_palimpsa_forms_agree(gpu_device, state_pass_mode, case):
     elif case == "varlen_ragged":       # full and partial tiles, a one-token document
         inp = _pal_inputs(1, 64 + 1 + 130 + 257, 2, 32, 48, 2, dev)
         cu = torch.tensor([0, 64, 65, 195, 452], dtype=torch.int32, device=dev)
-    elif case == "wide_heads":
+    elif case == "wide_heads":            # few (sequence, head) pairs: the one-pass form also slices the key columns
         inp = _pal_inputs(2, 129, 2, 256, 144, 3, dev)
+    elif case == "key_slices":            # the same with an initial state, at the shape class of a long single prefill
+        inp = _pal_inputs(1, 300, 12, 128, 128, 6, dev)
+        gen = torch.Generator().manual_seed(10)
+        mu0 = (torch.randn(1, 12, 128, 128, generator=gen) * 0.3).to(dev)
+        I0 = (torch.rand(1, 12, 128, 128, generator=gen) + inp["Ip"].cpu()[None, :, None, None]).to(dev)
     else:
         inp = _pal_inputs(2, 200, 3, 48, 96, 4, dev)
         gen = torch.Generator().manual_seed(9)
