@@ -34,9 +34,11 @@ def _count_chunks(T: int, B: int) -> int:
     return (T + L.PAL_CHUNK - 1) // L.PAL_CHUNK * B
 
 
-# the windowed forward keeps at most this many bytes of tile-start states alive (they then stay in the
-# 256 MB last-level cache between the kernel that writes them and the two that read them)
-_WINDOW_STATE_BYTES = 128 << 20
+# the windowed forward keeps at most this many bytes of tile-start states alive (measured on one sequence of 65536
+# tokens, H = 16, 128 x 128: 64 MB 6.3 ms, 128 MB 5.8, 512 MB 5.65, 1 GB 5.73, all 2.1 GB at once 5.8: the output
+# kernel is bound by vector issue whether the states come from the last-level cache or from HBM, and every window
+# pays the fill of the state pass's pipeline)
+_WINDOW_STATE_BYTES = 512 << 20
 
 
 def _window_tiles(H: int, dv: int, dk: int) -> int:
