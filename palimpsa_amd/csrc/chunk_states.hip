@@ -37,6 +37,7 @@ struct StatePassArgs {
   float *fin_a, *fin_b;
   int32_t ds, nsplit, reverse, per_xcd, total;
   int32_t dks, ksplit;    // key columns per workgroup and slices of the key columns (dk = dks * ksplit)
+  int32_t by_length;      // packed sequences are handed out longest first (see the kernel)
   float fin_scale;
 };
 
@@ -55,13 +56,36 @@ __global__ __launch_bounds__(768) void chunk_states_kernel(StatePassArgs A) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int H = a.H, dk = a.dk, dv = a.dv, ds = A.ds, dks = A.dks;
   // consecutive workgroup ids go to different XCDs: give the slices of one (sequence, head) to the same one,
-  // they read the same key rows
-  const int m = ((int)blockIdx.x & 7) * A.per_xcd + ((int)blockIdx.x >> 3);
-  if (m >= A.total) return;
-  // a workgroup owns the state entries (value rows [d0, d0 + ds)) x (key columns [k0, k0 + dks))
-  const int n_sl = A.nsplit * A.ksplit, sl = m % n_sl;
-  const int nh = m / n_sl, d0 = (sl / A.ksplit) * ds, k0 = (sl % A.ksplit) * dks;
-  const int h = nh % H, n = nh / H;
+  // they read the same key rows.  A workgroup owns the state entries (value rows [d0, d0 + ds)) x (key columns
+  // [k0, k0 + dks)) of a (sequence, head).
+  const int n_sl = A.nsplit * A.ksplit;
+  const int xcd = (int)blockIdx.x & 7, pos = (int)blockIdx.x >> 3;
+  int m, n;
+  if (A.by_length) {
+    // Packed sequences of unequal length (at most 64): the walk over a sequence's tiles is serial, so a long sequence
+    // that starts late ends the kernel late.  The sequence of rank r in descending length goes to XCD r mod 8, in
+    // rank order there; every wave finds the sequence of its rank with one lane per sequence.
+    const int rank = (pos / (H * n_sl)) * 8 + xcd;
+    if (rank >= a.n_seqs) return;
+    int b_l = 0, len_l = -1;
+    if (lane < a.n_seqs) packed_seq_bounds(a.cu_seqlens, lane, a.T, b_l, len_l);
+    int before = 0;   // sequences ahead of lane's own in the order (longer, or as long with a smaller index)
+    for (int j = 0; j < a.n_seqs; ++j) {
+      const int len_j = __builtin_amdgcn_readlane(len_l, j);
+      before += (len_j > len_l || (len_j == len_l && j < lane)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(lane < a.n_seqs && before == rank);
+    n = hit ? (int)__builtin_ctzll(hit) : 0;
+    m = n * H * n_sl + pos % (H * n_sl);
+  } else {
+    m = xcd * A.per_xcd + pos;
+    if (m >= A.total) return;
+    n = (m / n_sl) / H;
+  }
+  const int sl = m % n_sl;
+  const int d0 = (sl / A.ksplit) * ds, k0 = (sl % A.ksplit) * dks;
+  const int h = (m / n_sl) % H;
+  const int nh = n * H + h;
   int bos, len, cbase;
   seq_lookup(a, n, bos, len, cbase);
   const int nchunks = (len + kC - 1) / kC;
@@ -394,6 +418,8 @@ int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tile
   if (total <= 0) return PAL_OK;
   int64_t per_xcd = (total + 7) / 8;
   per_xcd = (per_xcd + n_sl - 1) / n_sl * n_sl;
+  A.by_length = (a.cu_seqlens && a.n_seqs > 1 && a.n_seqs <= 64) ? 1 : 0;
+  if (A.by_length) per_xcd = (int64_t)((a.n_seqs + 7) / 8) * a.H * n_sl;   // whole sequences per XCD
   if (per_xcd * 8 > 0x7fffffff) return PAL_E_DIM;
   A.total = (int32_t)total;
   A.per_xcd = (int32_t)per_xcd;
