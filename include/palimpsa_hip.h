@@ -179,7 +179,10 @@ int pal_recurrent_bwd(const PalDims *dims, const PalFwdTensors *t, const PalBwdT
  * :187-188) for the backward.  The prefix products of the output kernel use f16
  * operands normalised per 64-token tile by three block exponents (of k, v and b),
  * so results do not depend on the magnitude of the rows; within a tile, entries
- * more than 2^26 below the largest of their tensor lose precision.
+ * more than 2^26 below the largest of their tensor lose precision.  The state at
+ * the start of a tile enters those products through the operands of the tile's
+ * first token (as an f16 number: 11 bits, against the 8 of bf16 rows), and the
+ * exponents of v and b are raised where that state is large against the rows.
  * cu_seqlens (varlen) must ascend from 0 to the token count; the kernels clamp
  * every sequence and tile to the token range, so a malformed array cannot make
  * them address memory beyond the tensors (results are then unspecified). */
