@@ -24,7 +24,8 @@ One JSON line is printed; it also carries
   extra.recurrent  token-serial forward and backward (pal_recurrent_fwd / pal_recurrent_bwd) at B=8 T=2048 H=12
                 d=64 fp32, against the HBM peak as the metric asks (the kernels are bound by serial latency)
 Every chunked leg carries two bounds: the bf16 matrix peak priced with the fixed formula of the metric and the
-fp32 vector peak priced with the vector instructions the kernel issues (counter figures, see VALU_LANE_OPS).
+fp32 vector peak priced with the vector instructions the kernel issues (counter figures from profiles/counter_table.txt).
+The decode leg of the metric is also carried as flat decode_* scalars inside the headline line's roofline object.
 """
 from __future__ import annotations
 
@@ -42,18 +43,40 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E peak
 PEAK_FP32_VALU_TFLOPS = 157.3    # MI355X fp32 vector peak (an FMA counted as 2 flops on every lane)
 CHUNK = 64
-# Vector-ALU instructions (matrix instructions excluded) that the two dominant chunked kernels issue per state
-# entry (token x value row x key column), as lane operations: rocprofv3 SQ_INSTS_VALU minus SQ_INSTS_VALU_MFMA_*
-# per launch at the headline shape, times 64 lanes, divided by tokens*H*dk*dv
-# (profiles/bench_c1.sq_counters_pmc.txt).  Like the traffic figures below they cannot be read from inside this
-# process and are stale once those kernels change.
-VALU_LANE_OPS_PER_ENTRY = {"chunk_bwd_local_kernel": 23.5, "chunk_out_kernel": 6.2}
-# HBM bytes per launch of the two priced kernels on the workloads below, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE scaled by a 1 GiB copy (profiles/bench_c1_c3.hbm_traffic_pmc.txt); counters cannot be read
-# from inside this process, so the figures are carried here and are stale once those kernels change.
-MEASURED_TRAFFIC_BYTES = {"chunk_bwd_local_kernel": 424.6e6, "recurrent_fwd_kernel": 1111.8e6,
-                          # profiles/bench_simple_gla__layer_slice.hbm_traffic_pmc.txt
-                          "gla_out_kernel": 141.2e6, "gla_recurrent_fwd_kernel": 543.4e6, "prologue_bwd_kernel": 305.9e6}
+COUNTER_TABLE = os.path.join(ROOT, "profiles", "counter_table.txt")
+
+
+def load_counter_table(path=COUNTER_TABLE):
+    """Per-kernel figures that only the profiler can read (rocprofv3 --pmc, one run per counter): HBM bytes per launch
+    (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size) and vector-ALU instructions per state entry
+    (SQ_INSTS_VALU minus the matrix instructions, times 64 lanes, per token x value row x key column).  They are kept in a
+    small table under profiles/ next to the summaries they come from, one line per (workload, kernel) with the commit the
+    kernels were at when they were collected, so that a stale figure shows in the line this script prints."""
+    table = {}
+    with open(path) as fh:
+        for ln in fh:
+            ln = ln.strip()
+            if not ln or ln.startswith("#"):
+                continue
+            workload, kernel, traffic, valu, commit = ln.split()[:5]
+            table[(workload, kernel)] = {"traffic": None if traffic == "-" else float(traffic),
+                                         "valu_ops_per_entry": None if valu == "-" else float(valu),
+                                         "measured_at": commit}
+    return table
+
+
+COUNTERS = load_counter_table()
+
+
+def counter(workload, kernel, field):
+    return COUNTERS.get((workload, kernel), {}).get(field)
+
+
+def add_traffic(roof, workload, kernel):
+    """Attach the profiler's HBM bytes per launch, and the commit they were measured at, to a roofline entry."""
+    roof["traffic"] = counter(workload, kernel, "traffic")
+    roof["traffic_measured_at"] = counter(workload, kernel, "measured_at")
+    return roof
 
 
 def make_inputs(torch, B, T, H, dk, dv, seed, dtype):
@@ -121,7 +144,7 @@ def timed_loop(torch, step, steps, warmup):
     return ms_mean, ms_median, kernels
 
 
-def mfma_roofline(kernel, kernels, flops_per_launch, entries, note):
+def mfma_roofline(workload, kernel, kernels, flops_per_launch, entries, note):
     """Roofline entry of a chunked kernel: the bf16 matrix peak priced with the metric's fixed flop formula, and the
     fp32 vector peak priced with the vector instructions the kernel issues per state entry."""
     avg_ms = kernels.get(kernel, {"avg_ms": float("nan")})["avg_ms"]
@@ -129,7 +152,8 @@ def mfma_roofline(kernel, kernels, flops_per_launch, entries, note):
     out = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
            "frac": achieved / PEAK_BF16_MFMA_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": flops_per_launch,
            "avg_launch_ms": avg_ms, "note": note}
-    ops = VALU_LANE_OPS_PER_ENTRY.get(kernel)
+    add_traffic(out, workload, kernel)
+    ops = counter(workload, kernel, "valu_ops_per_entry")
     if ops is not None:
         valu = ops * entries * 2 / (avg_ms * 1e-3) / 1e12
         out["valu"] = {"ops_per_entry": ops, "achieved": valu, "peak": PEAK_FP32_VALU_TFLOPS, "unit": "TFLOP/s",
@@ -169,14 +193,16 @@ def bench_chunk(torch, dev, steps, warmup, gates="bf16"):
     # share of the dominant kernel: recompute L@X (M and J) + reverse L^T@dMloc (M and J)
     flops_local = 4 * (CHUNK + 1) * E * token_heads
     roofline = mfma_roofline(
-        "chunk_bwd_local_kernel", kernels, flops_local, token_heads * E,
+        "c1", "chunk_bwd_local_kernel", kernels, flops_local, token_heads * E,
         "flops = 4(C+1)*dk*dv per token-head (recompute + reverse triangular contractions, C=64); step_frac uses "
         "(6C+14)*dk*dv over the whole fwd+bwd step.  The kernel is bound by fp32 vector issue in the tile epilogues "
         "(one division per state entry), not by the matrix cores: see roofline.valu and "
         "profiles/bench_c1.sq_counters_pmc.txt")
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES["chunk_bwd_local_kernel"]
+    if "valu" in roofline:      # flat copies: nested objects do not survive every consumer of this line
+        roofline["valu_frac"] = roofline["valu"]["frac"]
+        roofline["valu_ops_per_entry"] = roofline["valu"]["ops_per_entry"]
     roofline["step_frac"] = flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
-    out_roof = mfma_roofline("chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * token_heads, token_heads * E,
+    out_roof = mfma_roofline("c1", "chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * token_heads, token_heads * E,
                              "flops = 2(C+1)*dk*dv per token-head (prefix products of M and J)")
     return dict(value=tokens / (ms_per_step * 1e-3), ms_per_step=ms_per_step, ms_per_step_median=ms_median,
                 roofline=roofline, roofline_forward=out_roof, kernels=kernels,
@@ -257,7 +283,8 @@ def bench_decode(torch, dev, steps):
         "hbm_gbs_wall": bytes_step * steps / elapsed / 1e9,
         "roofline": {"bound": "hbm", "kernel": "recurrent_fwd_kernel", "achieved": gbs_kernel, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": gbs_kernel / PEAK_HBM_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES["recurrent_fwd_kernel"],
+                     "traffic": counter("c3", "recurrent_fwd_kernel", "traffic"),
+                     "traffic_measured_at": counter("c3", "recurrent_fwd_kernel", "measured_at"),
                      "algorithmic_bytes_per_launch": bytes_step, "avg_launch_ms": avg_ms},
     }
 
@@ -352,7 +379,8 @@ def bench_simple_gla(torch, dev, steps, warmup):
               "tokens_per_s": Bd * dsteps / d_elapsed, "ms_per_step": d_elapsed * 1e3 / dsteps,
               "roofline": {"bound": "hbm", "kernel": "gla_recurrent_fwd_kernel", "achieved": dec_gbs, "peak": PEAK_HBM_GBS,
                            "unit": "GB/s", "frac": dec_gbs / PEAK_HBM_GBS,
-                           "traffic": MEASURED_TRAFFIC_BYTES["gla_recurrent_fwd_kernel"],
+                           "traffic": counter("gla_decode", "gla_recurrent_fwd_kernel", "traffic"),
+                           "traffic_measured_at": counter("gla_decode", "gla_recurrent_fwd_kernel", "measured_at"),
                            "algorithmic_bytes_per_launch": bytes_dec, "avg_launch_ms": dk_ms / max(dk_n, 1)}}
     return {"workload": "chunk_simple_gla fwd+bwd B=8 T=2048 H=12 dk=dv=64 bf16 rows fp32 gates", "decode": decode,
             "tokens_per_s": B * T / (ms * 1e-3), "ms_per_step": ms, "kernel_ms_per_step": sum(v[0] for v in kern.values()) / steps,
@@ -360,7 +388,9 @@ def bench_simple_gla(torch, dev, steps, warmup):
                              "note": "the eager step above recorded once into a HIP graph (torch.cuda.graph) and replayed"},
             "kernels": kernels,
             "roofline": {"bound": "hbm", "kernel": "gla_out_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
-                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES["gla_out_kernel"],
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                         "traffic": counter("gla_c1", "gla_out_kernel", "traffic"),
+                         "traffic_measured_at": counter("gla_c1", "gla_out_kernel", "measured_at"),
                          "algorithmic_bytes_per_launch": bytes_out, "avg_launch_ms": avg_out_ms}}
 
 
@@ -423,7 +453,8 @@ def bench_layer_slice(torch, dev, steps, warmup):
             "kernels": {k: {"avg_ms": v[0] / v[1], "launches": v[1]} for k, v in kern.items()},
             "roofline": {"bound": "hbm", "kernel": "prologue_bwd_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
                          "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
-                         "traffic": MEASURED_TRAFFIC_BYTES["prologue_bwd_kernel"],
+                         "traffic": counter("layer_slice", "prologue_bwd_kernel", "traffic"),
+                         "traffic_measured_at": counter("layer_slice", "prologue_bwd_kernel", "measured_at"),
                          "algorithmic_bytes_per_launch": bytes_pb, "avg_launch_ms": avg_pb}}
 
 
@@ -538,7 +569,7 @@ def bench_c2(torch, dev, steps, warmup):
 
     ms, med, kernels = timed_loop(torch, step, steps, warmup)
     E, th = d * d, T * H
-    roof = mfma_roofline("chunk_bwd_local_kernel", kernels, 4 * (CHUNK + 1) * E * th, th * E,
+    roof = mfma_roofline("c2", "chunk_bwd_local_kernel", kernels, 4 * (CHUNK + 1) * E * th, th * E,
                          "flops = 4(C+1)*dk*dv per token-head; step_frac uses (6C+14)*dk*dv; dk = 96 runs the tile kernel "
                          "in three passes of two column blocks (two workgroups per compute unit)")
     roof["step_frac"] = (6 * CHUNK + 14) * E * th / (ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
@@ -567,7 +598,7 @@ def bench_c4(torch, dev, steps, warmup):
     E, th = d * d, T * H
     # the forward runs in windows of tiles: the per-kernel averages are per window, the flops likewise
     n_launch = max(1, kernels.get("chunk_out_kernel", {"launches": steps})["launches"] // steps)
-    roof = mfma_roofline("chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * th / n_launch, th * E / n_launch,
+    roof = mfma_roofline("c4", "chunk_out_kernel", kernels, 2 * (CHUNK + 1) * E * th / n_launch, th * E / n_launch,
                          f"flops = 2(C+1)*dk*dv per token-head (prefix products of M and J); the sequence is run in "
                          f"{n_launch} windows of tiles handed through the state, one launch each; step_frac uses "
                          "(2C+6)*dk*dv over the whole forward")
@@ -685,7 +716,16 @@ def main():
     extra = {"kernels": res["kernels"], "ms_per_step_median": res["ms_per_step_median"],
              "roofline_forward": res["roofline_forward"]}
     if not args.no_decode:
-        extra["decode"] = bench_decode(torch, dev, args.decode_steps)
+        extra["decode"] = dec = bench_decode(torch, dev, args.decode_steps)
+        # the second half of the metric (decode tokens/s, fraction of the HBM peak) as flat scalars of the headline
+        # line's roofline object
+        dr = dec["roofline"]
+        res["roofline"].update({
+            "decode_workload": dec["workload"], "decode_tokens_per_s": dec["tokens_per_s"],
+            "decode_ms_per_step": dec["ms_per_step"], "decode_kernel_avg_ms": dr["avg_launch_ms"],
+            "decode_algorithmic_bytes": dr["algorithmic_bytes_per_launch"], "decode_gbs": dr["achieved"],
+            "decode_peak_gbs": dr["peak"], "decode_frac": dr["frac"], "decode_traffic": dr["traffic"],
+            "decode_traffic_measured_at": dr["traffic_measured_at"]})
     if not args.no_simple_gla:
         extra["simple_gla"] = bench_simple_gla(torch, dev, args.steps, args.warmup)
     if not args.no_layer_slice:

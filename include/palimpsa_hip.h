@@ -18,6 +18,9 @@
  *     void*); nothing synchronises, allocates or frees.
  *   - return value: 0 = ok; < 0 = argument error found before any HIP call
  *     (PAL_E_*); > 0 = a hipError_t from a launch.
+ *   - row tensors and states are 16-byte aligned, the gate tensor gt 4-byte
+ *     aligned whatever its element type (a bf16 gate is fetched as the aligned
+ *     32-bit word that holds it); PAL_E_ALIGN otherwise.
  *   - dk and dv must be multiples of 16 in [16, 256]; callers with other sizes
  *     zero-pad (padding k,q,v,b with zeros leaves the valid outputs unchanged).
  */
@@ -74,7 +77,7 @@ extern "C" {
 #define PAL_E_CHUNK -8       /* unsupported chunk size                        */
 #define PAL_E_STATE -9       /* init/final state flags and pointers disagree  */
 #define PAL_E_CAPACITY -10   /* output table too small                        */
-#define PAL_E_ALIGN -11      /* pointer not aligned to 16 bytes               */
+#define PAL_E_ALIGN -11      /* pointer not aligned (rows, states: 16 bytes; gt: 4 bytes) */
 #define PAL_E_SCRATCH -12    /* the call needs more than the library's static scratch */
 
 /* Bytes of device memory the library itself holds per GPU for pal_chunk_fwd_static. */
@@ -106,7 +109,7 @@ typedef struct PalDims {
 /* Forward-side tensors.  Unused optional pointers are NULL. */
 typedef struct PalFwdTensors {
   const void *q, *k, *v, *b;      /* dtype                                    */
-  const void *gt;                 /* gate_dtype [B,T,H]                       */
+  const void *gt;                 /* gate_dtype [B,T,H], 4-byte aligned       */
   const float *g, *Ip;            /* fp32 [H]                                 */
   void *o;                        /* dtype [B,T,H,dv]                         */
   void *o_var;                    /* var_dtype [B,T,H,dv] or NULL             */

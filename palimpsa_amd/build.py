@@ -79,25 +79,6 @@ def build(force: bool = False, jobs: int = 8) -> str:
     return LIB_PATH
 
 
-ISSUE_RATES_SRC = os.path.join(CSRC, "bench", "issue_rates.hip")
-ISSUE_RATES_EXE = os.path.join(LIB_DIR, "issue_rates")
-
-
-def build_issue_rates(force: bool = False) -> str:
-    """The stand-alone micro-benchmark of instruction issue rates (csrc/bench/issue_rates.hip): an executable next to
-    the library, run by hand on a GPU box (``palimpsa_amd/lib/issue_rates``); not part of the library."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    if (not force and os.path.exists(ISSUE_RATES_EXE)
-            and os.path.getmtime(ISSUE_RATES_EXE) >= os.path.getmtime(ISSUE_RATES_SRC)):
-        return ISSUE_RATES_EXE
-    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-O3", ISSUE_RATES_SRC, "-o", ISSUE_RATES_EXE]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on {ISSUE_RATES_SRC}:\n{r.stdout}\n{r.stderr}")
-    return ISSUE_RATES_EXE
-
-
 if __name__ == "__main__":
     p = build(force="--force" in sys.argv)
     print(p)
-    print(build_issue_rates(force="--force" in sys.argv))

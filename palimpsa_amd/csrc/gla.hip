@@ -672,6 +672,7 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   const void* ptrs[] = {t->q, t->k, t->v, t->o, t->init_mu, t->final_mu, t->chunk_mu, t->chunk_I};
   for (const void* p : ptrs)
     if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  if (!is_aligned4(t->gt)) return PAL_E_ALIGN;   // gates are fetched as the aligned 32-bit word that holds them
   return PAL_OK;
 }
 

@@ -137,6 +137,7 @@ extern "C" int pal_gla_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, v
   const void* ptrs[] = {t->q, t->k, t->v, t->o, t->init_mu, t->final_mu};
   for (const void* p : ptrs)
     if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  if (!is_aligned4(t->gt)) return PAL_E_ALIGN;   // one alignment rule for the gate tensor at every entry point
   GlaRecArgs a;
   a.q = t->q; a.k = t->k; a.v = t->v; a.gt = t->gt; a.g = t->g; a.o = t->o;
   a.init = t->init_mu; a.final_ = t->final_mu; a.cu_seqlens = t->cu_seqlens;

@@ -25,7 +25,7 @@ const char* pal_strerror(int code) {
     case PAL_E_CHUNK: return "total_chunks does not match the sequence lengths";
     case PAL_E_STATE: return "state flags and state pointers disagree";
     case PAL_E_CAPACITY: return "output table too small";
-    case PAL_E_ALIGN: return "pointer not aligned to 16 bytes";
+    case PAL_E_ALIGN: return "pointer not aligned (row tensors and states: 16 bytes; gate tensor: 4 bytes)";
     case PAL_E_SCRATCH:
       return "the call needs more tile-start states than the library's static scratch holds "
              "(total_chunks * n_heads * dv * dk * 8 bytes > PAL_STATIC_SCRATCH_BYTES); split the sequence";
@@ -106,6 +106,7 @@ int check_fwd_common(const PalDims* d, const PalFwdTensors* t) {
                         t->final_mu, t->final_I, t->chunk_mu, t->chunk_I};
   for (const void* p : ptrs)
     if (p && !is_aligned16(p)) return PAL_E_ALIGN;
+  if (!is_aligned4(t->gt)) return PAL_E_ALIGN;   // gates are fetched as the aligned 32-bit word that holds them
   return PAL_OK;
 }
 

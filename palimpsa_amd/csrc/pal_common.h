@@ -283,5 +283,6 @@ inline int allow_lds(const void* kernel, size_t bytes) {
 }
 
 inline bool is_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+inline bool is_aligned4(const void* p) { return (((uintptr_t)p) & 3u) == 0; }
 
 }  // namespace pal

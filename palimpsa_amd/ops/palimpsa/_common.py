@@ -99,6 +99,8 @@ def prepare_inputs(q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, cu_
     if gt.dtype not in (torch.float32, torch.bfloat16):
         gt = gt.float()
     gt = gt.contiguous()
+    if gt.data_ptr() % 4:       # a bf16 view that starts on an odd element: the kernels fetch gates as aligned words
+        gt = gt.clone()
     g = g.reshape(H).float().contiguous()
     Ip = Ip.reshape(H).float().contiguous()
     n_seqs = B
@@ -145,12 +147,16 @@ def chunk_meta(cu_seqlens: torch.Tensor, total_tokens: int, device: torch.device
     token, length, index in sequence).  Raises ValueError unless cu_seqlens starts at 0, never decreases and
     ends at ``total_tokens`` (the kernels take sequence bounds from it).  Results are kept per tensor object
     (weakly referenced, invalidated by in-place writes through torch), not per address: a new tensor that
-    reuses the memory of a dead one is looked at again."""
+    reuses the memory of a dead one is looked at again.  A host tensor is also compared element by element with
+    the copy taken when its entry was made (its memory may be shared with an array that a loader rewrites without
+    torch noticing).  For a device tensor the entry relies on torch's version counter: a kernel or extension that
+    writes through ``data_ptr()`` must call ``invalidate_chunk_meta()`` (or hand over a new tensor)."""
     key = id(cu_seqlens)
     hit = _chunk_meta_cache.get(key)
     if hit is not None:
-        ref, version, tokens, dev, packed, total = hit
-        if ref() is cu_seqlens and version == cu_seqlens._version and tokens == total_tokens and dev == device:
+        ref, version, tokens, dev, packed, total, host_copy = hit
+        if (ref() is cu_seqlens and version == cu_seqlens._version and tokens == total_tokens and dev == device
+                and (host_copy is None or torch.equal(cu_seqlens.detach().to(torch.int64), host_copy))):
             return packed, total
     if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
         raise ValueError(f"cu_seqlens must be a 1-D tensor of at least two entries, got shape {tuple(cu_seqlens.shape)}")
@@ -169,20 +175,31 @@ def chunk_meta(cu_seqlens: torch.Tensor, total_tokens: int, device: torch.device
         ref = weakref.ref(cu_seqlens, lambda _r, k=key: _chunk_meta_cache.pop(k, None))
     except TypeError:
         return packed, total
-    _chunk_meta_cache[key] = (ref, cu_seqlens._version, int(total_tokens), device, packed, total)
+    host_copy = torch.from_numpy(cu_host).clone() if cu_seqlens.device.type == "cpu" else None
+    _chunk_meta_cache[key] = (ref, cu_seqlens._version, int(total_tokens), device, packed, total, host_copy)
     return packed, total
+
+
+def invalidate_chunk_meta() -> None:
+    """Forget the chunk bookkeeping kept per cu_seqlens tensor (for callers that rewrite a device cu_seqlens
+    tensor behind torch's back)."""
+    _chunk_meta_cache.clear()
 
 
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
 
-def make_dims(p: Prepared, scale: float, flags: int, total_chunks: int = 0, var_dtype: torch.dtype = torch.float32) -> L.PalDims:
+def make_dims(p: Prepared, scale: float, flags: int, total_chunks: int = 0, var_dtype: torch.dtype = torch.float32,
+              mode_flags: Optional[int] = None) -> L.PalDims:
+    """``mode_flags``: the knob bits (state-pass form, fp32 treatment) to use instead of the current settings, for a
+    backward that has to run in the mode its forward ran in."""
     B, T, H, _ = p.v.shape
     return L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=p.dk_p, dv=p.dv_p,
                      total_chunks=total_chunks, dtype=_pal_dtype(p.compute_dtype),
                      gate_dtype=_pal_dtype(p.gt.dtype), var_dtype=_pal_dtype(var_dtype),
-                     flags=flags | L.state_pass_flags(), scale=float(scale), n_qk_heads=p.q.shape[2])
+                     flags=flags | (L.state_pass_flags() if mode_flags is None else int(mode_flags)), scale=float(scale),
+                     n_qk_heads=p.q.shape[2])
 
 
 def make_fwd_tensors(p: Prepared, o, o_var, final_mu, final_I, chunk_table=None, chunk_offsets=None,

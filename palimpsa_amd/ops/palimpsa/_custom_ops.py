@@ -43,9 +43,13 @@ if _HAS_CUSTOM_OP:
     @torch.library.custom_op("palimpsa_amd::chunk_fwd", mutates_args=())
     def chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b: torch.Tensor, gt: torch.Tensor, g: torch.Tensor,
                   Ip: torch.Tensor, init_mu: Optional[torch.Tensor], init_I: Optional[torch.Tensor], scale: float,
-                  output_uncertainty: bool, cu_seqlens: Optional[torch.Tensor]
+                  output_uncertainty: bool, cu_seqlens: Optional[torch.Tensor], mode_flags: int
                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-        """-> (o, o_var | empty, final_mu, final_I, tile_mu, tile_I)"""
+        """-> (o, o_var | empty, final_mu, final_I, tile_mu, tile_I).  ``mode_flags``: the knob bits of PalDims.flags
+        (L.state_pass_flags() when the call was traced); the backward op gets the same value, so a knob changed
+        between the two cannot mix operand modes.  The tile-start states of every tile are always kept (this op does
+        not know whether a backward follows): a long prefill without gradients under a tracer needs
+        total_chunks * H * dv * dk * 8 bytes where the eager entry point runs in windows of 512 MB."""
         p = cm.prepare_inputs(q, k, v, b, gt, g, Ip, init_mu, init_I, cu_seqlens, recurrent=False)
         dev = p.q.device
         B, T, H, _ = p.v.shape
@@ -68,7 +72,7 @@ if _HAS_CUSTOM_OP:
         final_I = torch.empty_like(final_mu)
         tile_mu = torch.empty(_max_tiles(B, T, p.n_seqs, varlen), H, p.dv_p, p.dk_p, dtype=torch.float32, device=dev)
         tile_I = torch.empty_like(tile_mu)
-        dims = cm.make_dims(p, scale, flags, total_chunks, var_dtype=p.compute_dtype)
+        dims = cm.make_dims(p, scale, flags, total_chunks, var_dtype=p.compute_dtype, mode_flags=mode_flags)
         tens = cm.make_fwd_tensors(p, o, o_var, final_mu, final_I, table, offsets, tile_mu, tile_I)
         with torch.cuda.device(dev):
             rc = L.load().pal_chunk_fwd(dims, tens, cm.current_stream_ptr(dev))
@@ -78,7 +82,7 @@ if _HAS_CUSTOM_OP:
         return o, o_var, cm.unpad_state(final_mu, p), cm.unpad_state(final_I, p), tile_mu, tile_I
 
     @chunk_fwd.register_fake
-    def _(q, k, v, b, gt, g, Ip, init_mu, init_I, scale, output_uncertainty, cu_seqlens):
+    def _(q, k, v, b, gt, g, Ip, init_mu, init_I, scale, output_uncertainty, cu_seqlens, mode_flags):
         B, T, H, dv = v.shape
         dk = q.shape[-1]
         n_seqs = B if cu_seqlens is None else cu_seqlens.shape[0] - 1
@@ -93,7 +97,7 @@ if _HAS_CUSTOM_OP:
     def chunk_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b: torch.Tensor, gt: torch.Tensor, g: torch.Tensor,
                   Ip: torch.Tensor, init_mu: Optional[torch.Tensor], init_I: Optional[torch.Tensor], scale: float,
                   cu_seqlens: Optional[torch.Tensor], tile_mu: torch.Tensor, tile_I: torch.Tensor, d_o: torch.Tensor,
-                  d_o_var: Optional[torch.Tensor]
+                  d_o_var: Optional[torch.Tensor], mode_flags: int
                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                              torch.Tensor, torch.Tensor, torch.Tensor]:
         """-> (dq, dk, dv, db, dgt, dg, dIp, d_init_mu | empty, d_init_I | empty)"""
@@ -128,7 +132,7 @@ if _HAS_CUSTOM_OP:
         dIp = torch.empty(H, dtype=torch.float32, device=dev)
         d_mu = torch.empty_like(p.init_mu) if p.init_mu is not None else None
         d_I = torch.empty_like(p.init_I) if p.init_I is not None else None
-        dims = cm.make_dims(p, scale, flags, total_chunks, var_dtype=cd)
+        dims = cm.make_dims(p, scale, flags, total_chunks, var_dtype=cd, mode_flags=mode_flags)
         tens = cm.make_fwd_tensors(p, do_p, None, None, None, table, offsets, tile_mu, tile_I)
         pt = cm._ptr
         grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk_), dv=pt(dv_), db=pt(db),
@@ -146,16 +150,17 @@ if _HAS_CUSTOM_OP:
                 cm.unpad_state(d_I, p).to(init_I.dtype) if d_I is not None else _empty(dg))
 
     @chunk_bwd.register_fake
-    def _(q, k, v, b, gt, g, Ip, init_mu, init_I, scale, cu_seqlens, tile_mu, tile_I, d_o, d_o_var):
+    def _(q, k, v, b, gt, g, Ip, init_mu, init_I, scale, cu_seqlens, tile_mu, tile_I, d_o, d_o_var, mode_flags):
         return (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(b), torch.empty_like(gt),
                 torch.empty_like(g), torch.empty_like(Ip),
                 torch.empty_like(init_mu) if init_mu is not None else g.new_empty(0),
                 torch.empty_like(init_I) if init_I is not None else g.new_empty(0))
 
     def _chunk_setup(ctx, inputs, output):
-        q, k, v, b, gt, g, Ip, init_mu, init_I, scale, output_uncertainty, cu_seqlens = inputs
+        q, k, v, b, gt, g, Ip, init_mu, init_I, scale, output_uncertainty, cu_seqlens, mode_flags = inputs
         ctx.save_for_backward(q, k, v, b, gt, g, Ip, init_mu, init_I, cu_seqlens, output[4], output[5])
         ctx.scale = scale
+        ctx.mode_flags = mode_flags
         ctx.output_uncertainty = output_uncertainty
         ctx.set_materialize_grads(False)
 
@@ -166,10 +171,11 @@ if _HAS_CUSTOM_OP:
         if not ctx.output_uncertainty:
             d_o_var = None
         # gradients arriving at the final states are ignored, as in the reference (chunk...py:522)
-        gr = chunk_bwd(q, k, v, b, gt, g, Ip, init_mu, init_I, ctx.scale, cu, tile_mu, tile_I, d_o, d_o_var)
+        gr = chunk_bwd(q, k, v, b, gt, g, Ip, init_mu, init_I, ctx.scale, cu, tile_mu, tile_I, d_o, d_o_var,
+                       ctx.mode_flags)
         d_mu = gr[7] if init_mu is not None else None
         d_I = gr[8] if init_I is not None else None
-        return gr[0], gr[1], gr[2], gr[3], gr[4], gr[5], gr[6], d_mu, d_I, None, None, None
+        return gr[0], gr[1], gr[2], gr[3], gr[4], gr[5], gr[6], d_mu, d_I, None, None, None, None
 
     chunk_fwd.register_autograd(_chunk_backward, setup_context=_chunk_setup)
 

@@ -238,8 +238,17 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
         # under a tracer the work is handed over as opaque library ops (see _custom_ops.py)
         if cu_seqlens is not None and q.shape[0] != 1:
             raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
+        mode_flags = L.state_pass_flags()
+        if torch.is_grad_enabled() and any(isinstance(x, torch.Tensor) and x.requires_grad
+                                           for x in (q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state)):
+            # refuse here what the backward could not serve, as the eager route does
+            rows_bf16 = all(x.dtype == torch.bfloat16 for x in (q, k, v, b))
+            L.check(L.load().pal_chunk_bwd_supported(
+                cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1]),
+                L.PAL_DTYPE_BF16 if rows_bf16 else L.PAL_DTYPE_F32, mode_flags), "chunk_palimpsa (backward head dims)")
         o, o_var, final_mu_state, final_I_state, _, _ = _ops.chunk_fwd(
-            q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, float(scale), bool(output_uncertainty), cu_seqlens)
+            q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, float(scale), bool(output_uncertainty), cu_seqlens,
+            mode_flags)
         out = (o, o_var) if output_uncertainty else o
         if output_final_state:
             return out, final_mu_state, final_I_state

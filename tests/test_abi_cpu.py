@@ -97,6 +97,10 @@ def test_entry_points_reject_bad_arguments_without_touching_a_gpu(L):
     assert lib.pal_recurrent_fwd(_dims(L, dk=24), _fwd_tensors(L), None) == L.PAL_E_HEADDIM
     assert lib.pal_recurrent_fwd(_dims(L, dk=80), _fwd_tensors(L), None) == L.PAL_E_HEADDIM   # chunk-only size
     assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, q=_fake(0x1004)), None) == L.PAL_E_ALIGN
+    # a gate is fetched as the aligned 32-bit word that holds it: a bf16 gate tensor on a 2-byte boundary is refused
+    assert lib.pal_recurrent_fwd(_dims(L, gate_dtype=L.PAL_DTYPE_BF16), _fwd_tensors(L, gt=_fake(0x5002)),
+                                 None) == L.PAL_E_ALIGN
+    assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, gt=_fake(0x5002)), None) == L.PAL_E_ALIGN
     # state flags and pointers must agree
     assert lib.pal_recurrent_fwd(_dims(L, flags=L.PAL_FLAG_HAS_INIT), _fwd_tensors(L), None) == L.PAL_E_STATE
     assert lib.pal_recurrent_fwd(_dims(L), _fwd_tensors(L, init_mu=_fake(), init_I=_fake()), None) == L.PAL_E_STATE
@@ -186,6 +190,7 @@ def test_simple_gla_entry_points_reject_bad_arguments(L):
         assert fn(_dims(L), _fwd_tensors(L, final_mu=_fake(), **ok), None) == L.PAL_E_STATE
         assert fn(_dims(L), _fwd_tensors(L, cu_seqlens=_fake(), **ok), None) == L.PAL_E_CU_SEQLENS
         assert fn(_dims(L), _fwd_tensors(L, v=_fake(0x3008), **ok), None) == L.PAL_E_ALIGN
+        assert fn(_dims(L, gate_dtype=L.PAL_DTYPE_BF16), _fwd_tensors(L, gt=_fake(0x5002), **ok), None) == L.PAL_E_ALIGN
     # the chunked form needs both tile buffers and a consistent tile count
     assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_mu=_fake(0x9000)), None) == L.PAL_E_NULL
     assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_I=_fake(0xa000)), None) == L.PAL_E_NULL

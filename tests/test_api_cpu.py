@@ -179,3 +179,17 @@ def test_chunk_table_is_kept_per_cu_seqlens_tensor():
     assert m4 is not m3 and torch.equal(m4, m3)
     with pytest.raises(ValueError):
         cm.chunk_meta(cu, 131, torch.device("cpu"))
+    # a host tensor that shares its memory with an array rewritten behind torch's back (no version bump): the entry
+    # is compared with the copy taken when it was made
+    import numpy as np
+    arr = np.array([0, 70, 130], dtype=np.int64)
+    shared = torch.from_numpy(arr)
+    m5, _ = cm.chunk_meta(shared, 130, torch.device("cpu"))
+    arr[1] = 64
+    m6, _ = cm.chunk_meta(shared, 130, torch.device("cpu"))
+    assert m6 is not m5 and torch.equal(m6, m3)
+    arr[2] = 100
+    with pytest.raises(ValueError):
+        cm.chunk_meta(shared, 130, torch.device("cpu"))
+    cm.invalidate_chunk_meta()
+    assert cm.chunk_meta(cu, 130, torch.device("cpu"))[0] is not m3

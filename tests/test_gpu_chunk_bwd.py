@@ -153,14 +153,20 @@ def test_state_far_above_the_increments_in_the_backward(gpu_device, dk, dv):
     _compare(grads, ref, NAMES, inp=inp, dg_l1=True)
 
 
-def test_c1_shape_backward_subset(gpu_device):
+@pytest.mark.parametrize("gate_dtype", [None, torch.bfloat16], ids=["fp32_gates", "bf16_gates"])
+def test_c1_shape_backward_subset(gpu_device, gate_dtype):
     """Config 1 at full size on the GPU (B=8,T=2048,H=12,d=64,bf16); the float64 oracle with autograd
-    checks one (batch, head) pair at full T (entries are independent)."""
+    checks one (batch, head) pair at full T (entries are independent).  With bf16 gates this is the workload
+    bench.py times (config 1 stores the per-token gates in bf16 like the rows); the oracle is fed the same
+    bf16-rounded gates.  fp32 gates are what the reference layer passes."""
     B, T, H, d = 8, 2048, 12, 64
     inp = hp.rounded(po.make_inputs(B, T, H, d, d, seed=0), torch.bfloat16)
+    if gate_dtype is not None:
+        inp["gt"] = inp["gt"].to(gate_dtype).float()
     gen = torch.Generator().manual_seed(1)
     do = torch.randn(B, T, H, d, generator=gen)
-    grads = _run_bwd(inp, gpu_device, do)
+    grads = _run_bwd(inp, gpu_device, do, gate_dtype=gate_dtype)
+    assert grads["gt"].dtype == (gate_dtype or torch.float32)
     bs, hs = [3], [7]
     sub = {n: inp[n][bs][:, :, hs] for n in ("q", "k", "v", "b", "gt")}
     sub["g"], sub["Ip"] = inp["g"][hs], inp["Ip"][hs]

@@ -122,12 +122,18 @@ def test_varlen_equals_per_document_oracle(gpu_device):
     assert hp.max_abs(o2, o_ref2) <= hp.BF16_OUT_ABS_TOL
 
 
-def test_c1_shape_subset_against_oracle_and_full_against_recurrent(gpu_device):
+@pytest.mark.parametrize("gate_dtype", [None, torch.bfloat16], ids=["fp32_gates", "bf16_gates"])
+def test_c1_shape_subset_against_oracle_and_full_against_recurrent(gpu_device, gate_dtype):
     """Config 1 (B=8,T=2048,H=12,d=64,bf16): the oracle checks a (batch, head) subset at full T
-    (entries are independent); the whole tensor is checked against the fp32-state recurrent kernel."""
+    (entries are independent); the whole tensor is checked against the fp32-state recurrent kernel.
+    With bf16 gates (the gate tensor handed over in bf16, as config 1 says and bench.py times) the oracle is fed
+    the same rounded gates."""
     ck, fr = _ops()
     inp = hp.rounded(po.make_inputs(8, 2048, 12, 64, 64, seed=0), torch.bfloat16)
     d = hp.to_device(inp, gpu_device)
+    if gate_dtype is not None:
+        inp["gt"] = inp["gt"].to(gate_dtype).float()
+        d["gt"] = d["gt"].to(gate_dtype)
     o, mu, I = _call(ck, d, output_final_state=True, chunk_size=64)
     o_r, mu_r, I_r = _call(fr, d, output_final_state=True)
     assert hp.max_abs(o.float(), o_r.float()) <= hp.BF16_OUT_ABS_TOL
@@ -136,8 +142,10 @@ def test_c1_shape_subset_against_oracle_and_full_against_recurrent(gpu_device):
     bs, hs = [0, 5], [1, 7, 11]
     sub = {n: inp[n][bs][:, :, hs] for n in ("q", "k", "v", "b", "gt")}
     sub["g"], sub["Ip"] = inp["g"][hs], inp["Ip"][hs]
-    o_ref, _, _, _ = hp.oracle_forward(sub)
+    o_ref, _, mu_ref, I_ref = hp.oracle_forward(sub)
     assert hp.max_abs(o[bs][:, :, hs], o_ref) <= hp.BF16_OUT_ABS_TOL
+    assert hp.max_rel(mu[bs][:, hs], mu_ref) <= STATE_REL_TOL
+    assert hp.max_rel(I[bs][:, hs], I_ref) <= STATE_REL_TOL
 
 
 def test_error_paths_match_reference(gpu_device):
@@ -308,10 +316,10 @@ def test_library_ops_pass_opcheck(gpu_device):
     inp = hp.to_device(hp.rounded(po.make_inputs(1, 70, 2, 16, 32, seed=3), torch.bfloat16), dev)
     q, k, v, b, gt, g, Ip = [inp[n] for n in ("q", "k", "v", "b", "gt", "g", "Ip")]
     tests = ("test_schema", "test_faketensor", "test_autograd_registration")
-    torch.library.opcheck(ops.chunk_fwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, True, None), test_utils=tests)
-    out = ops.chunk_fwd(q, k, v, b, gt, g, Ip, None, None, 0.25, False, None)
+    torch.library.opcheck(ops.chunk_fwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, True, None, 0), test_utils=tests)
+    out = ops.chunk_fwd(q, k, v, b, gt, g, Ip, None, None, 0.25, False, None, 0)
     torch.library.opcheck(ops.chunk_bwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, None, out[4], out[5],
-                                          torch.ones_like(v), None), test_utils=tests)
+                                          torch.ones_like(v), None, 0), test_utils=tests)
     torch.library.opcheck(ops.recurrent_fwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, True, True, None), test_utils=tests)
     torch.library.opcheck(ops.recurrent_bwd, (q, k, v, b, gt, g, Ip, None, None, 0.25, None, torch.ones_like(v), None),
                           test_utils=tests)

@@ -69,6 +69,29 @@ def test_c2_packed_documents_forward_backward(gpu_device):
             err = hp.max_rel(grads[n][:, sl][:, :, hs], ref[n])
             assert err <= hp.BF16_GRAD_NORM_TOL, (j, n, err)
 
+    # the per-head reductions dg, dIp over ALL documents (the kernel sums 22 documents' shares per head): the oracle
+    # runs every document of one head with autograd (float64, document by document so that only one document's
+    # per-token states are alive at a time) and its gradients are added up.  dg is normalised by the l1 mass of its
+    # terms (random dO: |dg| is far below the sum of the magnitudes, see tests/test_gpu_chunk_bwd.py), dIp likewise by
+    # the mass of its per-document terms.
+    h = 12
+    dg_ref = dIp_ref = 0.0
+    dg_mass = dIp_mass = 0.0
+    for j in range(len(cu) - 1):
+        sl = slice(cu[j], cu[j + 1])
+        sub = {n: inp[n][:, sl][:, :, [h]] for n in ("q", "k", "v", "b", "gt")}
+        sub["g"], sub["Ip"] = inp["g"][[h]], inp["Ip"][[h]]
+        ref = hp.oracle_grads(sub, do[:, sl][:, :, [h]])
+        dg_ref += ref["g"].item()
+        dIp_ref += ref["Ip"].item()
+        dg_mass += (sub["gt"].double() * ref["gt"].double()).abs().sum().item() / sub["g"].item()
+        dIp_mass += abs(ref["Ip"].item())
+    e_g = abs(grads["g"][h].item() - dg_ref) / dg_mass
+    e_Ip = abs(grads["Ip"][h].item() - dIp_ref) / dIp_mass
+    print(f"c2 head {h}: dg {grads['g'][h].item():.5e} ref {dg_ref:.5e} |d|/mass {e_g:.2e}; "
+          f"dIp {grads['Ip'][h].item():.5e} ref {dIp_ref:.5e} |d|/mass {e_Ip:.2e}")
+    assert e_g <= hp.BF16_GRAD_NORM_TOL and e_Ip <= hp.BF16_GRAD_NORM_TOL
+
 
 def test_c3_decode_steps_with_state_fed_back(gpu_device):
     _, fr = _ops()
