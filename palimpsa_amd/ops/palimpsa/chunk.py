@@ -225,6 +225,18 @@ class ChunkPalimpsa(torch.autograd.Function):
                 None, None, None, None, None, None, None, None)
 
 
+def _assume_constant(fn):
+    mark = getattr(getattr(torch, "_dynamo", None), "assume_constant_result", None)
+    return mark(fn) if mark is not None else fn
+
+
+@_assume_constant
+def _bwd_supported_code(dk_p: int, dv_p: int, dtype: int, flags: int) -> int:
+    """pal_chunk_bwd_supported as a plain int; a tracer evaluates it once on its constant arguments instead of
+    following the ctypes call."""
+    return int(L.load().pal_chunk_bwd_supported(dk_p, dv_p, dtype, flags))
+
+
 def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state=None, scale=None,
                    chunk_size=16, output_final_state=False, output_uncertainty=False, cu_seqlens=None):
     """Chunked Palimpsa attention; calling convention of chunk_palimpsa in the reference
@@ -243,9 +255,10 @@ def chunk_palimpsa(q, k, v, b, gt, g, Ip, initial_mu_state=None, initial_I_state
                                            for x in (q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state)):
             # refuse here what the backward could not serve, as the eager route does
             rows_bf16 = all(x.dtype == torch.bfloat16 for x in (q, k, v, b))
-            L.check(L.load().pal_chunk_bwd_supported(
-                cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1]),
-                L.PAL_DTYPE_BF16 if rows_bf16 else L.PAL_DTYPE_F32, mode_flags), "chunk_palimpsa (backward head dims)")
+            rc = _bwd_supported_code(cm.padded_dk(q.shape[-1], False), cm.padded_dv(v.shape[-1]),
+                                     L.PAL_DTYPE_BF16 if rows_bf16 else L.PAL_DTYPE_F32, mode_flags)
+            if rc != 0:
+                raise ValueError(f"chunk_palimpsa (backward head dims): unsupported by pal_chunk_bwd (code {rc})")
         o, o_var, final_mu_state, final_I_state, _, _ = _ops.chunk_fwd(
             q, k, v, b, gt, g, Ip, initial_mu_state, initial_I_state, float(scale), bool(output_uncertainty), cu_seqlens,
             mode_flags)
