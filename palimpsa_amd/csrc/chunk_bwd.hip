@@ -98,19 +98,22 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   float* sSt = sF + kC;                  // [2][NST][16][kVS2]
   float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
   float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
-  float* sRed = sPb + NB * kDG2 * kC;    // [NB][64] d log f partials, then [2*NB] sums of dJloc (padded to 16 floats)
-  // LAG: the second producer runs one value row behind the first and takes the operands of tokens 0..31 from the
-  // first one's slot instead of forming them again (it is the longest role of a row); the consumers follow two rows
-  // behind.  The first producer's half of a slot is then alive for three rows, the second one's for two:
-  //   sX  [NB][3 x {P^M_0, P^J_0, X^M_0, X^J_0} | 2 x {P^M_1, P^J_1, X^M_1, X^J_1}][64 lanes],  sMJ [NB][4 slots][2][16].
+  // LAG: the second producer runs one value row behind the first (it takes what the first one leaves for it: the
+  // operands of tokens 0..31, or, with the tile cut in two halves (SUB below), the state after token 31); the consumers
+  // follow two rows behind.  The first producer's half of a slot is then alive for three rows, the second one's for two:
+  //   sX  [NB][3 x {P^M_0, P^J_0, X^M_0, X^J_0} | 2 x {P^M_1, P^J_1, X^M_1, X^J_1}][64 lanes],
+  //   sMJ [NB][3 slots][M_0, J_0, M_31, J_31, what flows back over token 31 (M, J)][16]   (see SUB below).
   // Not with two column blocks per workgroup (two such workgroups share a compute unit's LDS) nor with split operands.
   constexpr bool LAG = local_lag(NB, PREC);
   constexpr int LAGC = LAG ? 2 : 1;        // rows the consumers run behind the first producer
-  float* sMJ = sRed + NB * kC + 16;      // [NB][2 (LAG: 4) slots][2][16] tile-start M_0, J_0 of the rows in flight
+  float* sMJ = sPb + NB * kDG2 * kC;     // [NB][2 slots][2][16] (LAG: [NB][3 slots][6][16]) states of the rows in flight
   constexpr int OPN = PREC ? 16 : 8;       // operands per slot (PREC: the lo halves follow the 8 hi halves)
-  bf16x8* sX = (bf16x8*)(sMJ + NB * (LAG ? 128 : 64));   // [NB][2 slots][OPN operands][64 lanes] (LAG: see above)
+  bf16x8* sX = (bf16x8*)(sMJ + NB * (LAG ? 288 : 64));   // [NB][2 slots][OPN operands][64 lanes] (LAG: see above)
   // [NB][16 rows][4][M 0..3, J 0..3] first column of dM^loc, dJ^loc of a group of value rows (the carry to the previous tile)
   float* sCar = (float*)(sX + NB * (LAG ? 20 : 2 * OPN) * 64);
+  // [NB][64] d log f partials of the consumer waves, then [2 NB] sums of dJloc: written after the last row of a pass,
+  // when the operand slots are dead, so they share their memory
+  float* sRed = (float*)sX;
   const int tid = threadIdx.x;
   int lane = tid & 63, i = lane & 15, g = lane >> 4;   // re-derived per pass from an opaque copy, see below
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: role branches are scalar
@@ -636,6 +639,294 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     }
   };
 
+
+  // ------------------------------------------------------------------ SUB: the tile as two halves of 32 tokens
+  // (bf16 operands, no initial state, LAG).  A causal product over 64 tokens costs 6 matrix instructions per 16
+  // columns (token blocks of 16 against K = 16, 32, 48, 64, padded to multiples of 32), over two halves of 32 tokens
+  // 4: the second half starts from the state after token 31, which the first producer has in its accumulators.
+  // That state travels the way the tile-start state does (FOLD above): the second producer adds f_32 (M_31, J_31) to
+  // the operand of token 32; the strictly-lower product of the second half gets it for token 32 itself as a virtual
+  // token in its last contraction slot.  The reverse contraction of the first half needs what flows back over the
+  // border, f_32 dM^loc_32 = sum_{t >= 32} 2^(c_t - c_31) dMloc_t: the second producer sums it from its fp32 local
+  // gradients and the first consumer adds it to the local gradient of token 31 in its operand.  The two producers
+  // are then the same code on tokens 0..31 and 32..63 and each consumer reads only its own half's operands:
+  // 36 -> 24 matrix instructions and 22 -> 16 KB of LDS traffic per value row and column block.
+  //   sMJ slot of a row (d mod 3): [M_0, J_0, M_31, J_31, f_32 dM^loc_32, f_32 dJ^loc_32][16 key columns]
+  auto producer_sub = [&](auto hfc) {
+    constexpr int HF = decltype(hfc)::value;   // tokens 32HF .. 32HF+31
+    bf16x8 Lop[2];            // L[t,s] inside the half: t = 32HF+16tl+i, s = 32HF+8g+j <= t
+    float kk[8], kk2[8];      // k and its square in operand layout (n = i, s = 32HF+8g+j)
+    float qq[8];              // q in result layout (t = 32HF+16tl+4g+r, n = i)
+    float dq[8];
+    bf16x2 wD[HF ? 4 : 1];    // second half: 2^(c_t - c_31), the weight of token t in what flows back to token 31 (pairs)
+    float sigacc = 0.f;
+    {
+      const TIn* kp = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
+      const TIn* qp = (const TIn*)a.q + qk_row(a, t0, h) + 16 * nb;
+      float ct[2], cs[8];
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl) ct[tl] = sC[32 * HF + 16 * tl + i];
+      *(f32x4*)&cs[0] = *(const f32x4*)&sC[32 * HF + 8 * g];
+      *(f32x4*)&cs[4] = *(const f32x4*)&sC[32 * HF + 8 * g + 4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int s = 32 * HF + 8 * g + j;
+        const bool ok = s < clen;
+        const float kv = to_f32((kp + (int64_t)(ok ? s : 0) * rs)[i]);
+        kk[j] = ok ? kv : 0.f;
+        kk2[j] = kk[j] * kk[j];
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+          const int t = 32 * HF + 16 * tl + i;
+          Lop[tl][j] = (bf16_t)((s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f);
+        }
+      }
+      const float c31 = sC[31];
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = 32 * HF + 16 * tl + 4 * g + r;
+          const bool ok = t < clen;
+          const float qv = to_f32((qp + (int64_t)(ok ? t : 0) * rs)[i]);
+          qq[tl * 4 + r] = ok ? qv : 0.f;
+          dq[tl * 4 + r] = 0.f;
+        }
+      if (HF) {
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+          for (int r = 0; r < 4; r += 2) {
+            const int t = 32 + 16 * tl + 4 * g + r;
+            wD[tl * 2 + r / 2] = pack2(fast_exp2(sC[t] - c31), fast_exp2(sC[t + 1] - c31));
+          }
+      }
+    }
+    // first half: tile-start state of the next value row (entry of the own key column n = i), fetched one row ahead
+    const float* cmu = a.chunk_mu + tile_off + 16 * nb;
+    const float* cI = a.chunk_I + tile_off + 16 * nb;
+    float mu_n = 0.f, I_n = 0.f;
+    if (!HF) { mu_n = cmu[i]; I_n = cI[i]; }
+    // decay of the incoming state into the first token of the half, on the lanes that hold that token's operand
+    const float f0m = (g == 0) ? fast_exp2(HF ? sC[32] - sC[31] : sC[0]) : 0.f;
+    int b3 = 0;                                 // d mod 3: the row's slot of sMJ and of the first producer's operands
+    for (int it = 0; it < dv + LAGC; ++it) {
+      if (it >= HF && it - HF < dv) {
+        const int d = it - HF, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
+        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
+        const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
+        const float* sDov = sSt + (buf * NST + NST - 1) * STG + dd * kVS2;
+        float* mj = sMJ + (nbl * 3 + b3) * 96;
+        float Mp, Jp;   // state before the first token of the half
+        if (!HF) {
+          const float mu0 = mu_n, I0 = I_n;
+          const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
+          mu_n = (cmu + dn)[i];
+          I_n = (cI + dn)[i];
+          Mp = mu0 * I0;
+          Jp = I0 - Ip;
+          if (g == 0) { mj[i] = Mp; mj[16 + i] = Jp; }
+        } else {
+          Mp = mj[32 + i];
+          Jp = mj[48 + i];
+        }
+        const float fM = f0m * Mp, fJ = f0m * Jp;
+        bf16x8 XM, XJ;
+        {
+          const f32x4 v0 = *(const f32x4*)&sV[32 * HF + 8 * g], v1 = *(const f32x4*)&sV[32 * HF + 8 * g + 4];
+          const f32x4 b0 = *(const f32x4*)&sB[32 * HF + 8 * g], b1 = *(const f32x4*)&sB[32 * HF + 8 * g + 4];
+#pragma unroll
+          for (int j = 0; j < 8; j += 2) {
+            const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
+            const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
+            const bf16x2 pm = pack2(j == 0 ? fmaf(kk[j], va, fM) : kk[j] * va, kk[j + 1] * vb);
+            const bf16x2 pj = pack2(j == 0 ? fmaf(kk2[j], ba, fJ) : kk2[j] * ba, kk2[j + 1] * bb);
+            XM[j] = pm[0]; XM[j + 1] = pm[1];
+            XJ[j] = pj[0]; XJ[j + 1] = pj[1];
+          }
+        }
+        bf16x8 PM, PJ;
+        float backM = 0.f, backJ = 0.f;
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+          const int tb = 2 * HF + tl;
+          f32x4 accM = {0.f, 0.f, 0.f, 0.f};
+          f32x4 accI = {Ip, Ip, Ip, Ip};
+          accM = mfma16(Lop[tl], XM, accM);
+          accI = mfma16(Lop[tl], XJ, accI);
+          if (!HF && tl == 1 && g == 3) {   // state after token 31 for the second half of the row
+            mj[32 + i] = accM[3];
+            mj[48 + i] = accI[3] - Ip;
+          }
+          const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
+          f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
+          if (HAS_VAR) dvv = *(const f32x4*)&sDov[16 * tb + 4 * g];
+          float dMl[4], dJl[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float rI = fast_rcp(accI[r]);
+            const float mu = accM[r] * rI;
+            const float q = qq[tl * 4 + r];
+            dMl[r] = (dov[r] * q) * rI;
+            dJl[r] = -(dMl[r] * mu);
+            dq[tl * 4 + r] = fmaf(mu, dov[r], dq[tl * 4 + r]);
+            if (HAS_VAR) {
+              const float wq = dvv[r] * q;          // scale*dovar*q
+              const float w = wq * q * rI;          // scale*dovar*q^2/I
+              dJl[r] = fmaf(-w, rI, dJl[r]);
+              dq[tl * 4 + r] = fmaf(2.f * wq, rI, dq[tl * 4 + r]);
+            }
+          }
+          const int o4 = tl * 4;
+          const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
+          const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
+          const bf16x2 one2 = {(bf16_t)1.f, (bf16_t)1.f};
+          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j0, one2, sigacc, false);
+          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j1, one2, sigacc, false);
+          if (HF) {   // what flows back over the border, from the packed pairs
+            backM = __builtin_amdgcn_fdot2_f32_bf16(m0, wD[tl * 2], backM, false);
+            backM = __builtin_amdgcn_fdot2_f32_bf16(m1, wD[tl * 2 + 1], backM, false);
+            backJ = __builtin_amdgcn_fdot2_f32_bf16(j0, wD[tl * 2], backJ, false);
+            backJ = __builtin_amdgcn_fdot2_f32_bf16(j1, wD[tl * 2 + 1], backJ, false);
+          }
+          PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
+          PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
+        }
+        if (HF) {   // sums over the four lane rows: row 0 gets the mean branch's total, row 1 the precision branch's
+          const float tot = rows4_sum_x4(backM, backJ, 0.f, 0.f);
+          if (g < 2) mj[64 + 16 * g + i] = tot;
+        }
+        bf16x8* mine = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;
+        mine[0] = PM; mine[64] = PJ; mine[2 * 64] = XM; mine[3 * 64] = XJ;
+        b3 = (b3 == 2) ? 0 : b3 + 1;
+      }
+      iter_tail(it);
+    }
+    TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb;
+#pragma unroll
+    for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 32 * HF + 16 * tl + 4 * g + r;
+        if (t < clen) (dqp + (int64_t)t * rso)[i] = from_f32<TIn>(dq[tl * 4 + r]);
+      }
+    const float x = wave_sum(sigacc);
+    if (lane == 0) sRed[NB * kC + HF * NB + nbl] = x;
+  };
+
+  auto consumer_sub = [&](auto hfc) {
+    constexpr int HF = decltype(hfc)::value;   // column tokens 32HF .. 32HF+31 (blocks sb = 2HF+sl)
+    bf16x8 Lr[2];     // reverse operand inside the half: contraction (g,j) <-> token t = 32HF + 16(j/4) + 4g + j%4 >= s
+    bf16x8 Ls[2];     // strictly-lower operand: contraction token s' = 32HF + 8g + j < column token s = 16sb+i
+    float kr[8], kr2[8];   // k and its square in result layout (s = 16sb+i, n = 4g+r)
+    float dkM[8], dkJ[8];
+    float gate[2];
+    {
+      const TIn* kp4 = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
+      float ct[2], cs[8], ctt[8];
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) ct[sl] = sC[16 * (2 * HF + sl) + i];
+      *(f32x4*)&cs[0] = *(const f32x4*)&sC[32 * HF + 8 * g];
+      *(f32x4*)&cs[4] = *(const f32x4*)&sC[32 * HF + 8 * g + 4];
+      *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * HF + 4 * g];
+      *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * HF + 16 + 4 * g];
+      // the last contraction slot of the half (token 31 / 63) is never below a column token of the half: it carries
+      // the state before the half's first token, which only that token's column takes (the later ones have it
+      // through the first token's operand)
+      const float fst = HF ? fast_exp2(sC[32] - sC[31]) : fast_exp2(sC[0]);
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const int s = 16 * (2 * HF + sl) + i;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int sp = 32 * HF + 8 * g + j;
+          float lv = (sp < s) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
+          if (g == 3 && j == 7) lv = (s == 32 * HF) ? fst : 0.f;
+          Ls[sl][j] = (bf16_t)lv;
+          const int t = 32 * HF + 16 * (j >> 2) + 4 * g + (j & 3);
+          Lr[sl][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { kr[sl * 4 + r] = 0.f; dkM[sl * 4 + r] = 0.f; dkJ[sl * 4 + r] = 0.f; }
+        if (s < clen) load_vec<4>(kp4 + (int64_t)s * rs + 4 * g, &kr[sl * 4]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) kr2[sl * 4 + r] = kr[sl * 4 + r] * kr[sl * 4 + r];
+        gate[sl] = 0.f;
+      }
+    }
+    float* car = sCar + ((nbl * kDG2) * 4 + g) * 8;
+    // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
+    float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
+    int b3 = 0;   // d mod 3
+    for (int it = 0; it < dv + LAGC; ++it) {
+      if (it >= LAGC) {
+        const int d = it - LAGC, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
+        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
+        const bf16x8* ph = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;   // the own half's operands
+        const float* mj = sMJ + (nbl * 3 + b3) * 96;
+        b3 = (b3 == 2) ? 0 : b3 + 1;
+        bf16x8 PM = ph[0], PJ = ph[64], XM = ph[2 * 64], XJ = ph[3 * 64];
+        {
+          // virtual token of the strictly-lower products: the state before the half's first token (key column n = i)
+          const bf16x2 st2 = pack2(mj[32 * HF + i], mj[32 * HF + 16 + i]);
+          if (g == 3) { XM[7] = st2[0]; XJ[7] = st2[1]; }
+        }
+        if (!HF) {
+          // what flows back over the border joins the local gradient of token 31 (element 7 of the lanes g = 3)
+          const float bm = mj[64 + i], bj = mj[80 + i];
+          if (g == 3) {
+            PM[7] = (bf16_t)((float)PM[7] + bm);
+            PJ[7] = (bf16_t)((float)PJ[7] + bj);
+          }
+        }
+        float dvp[2], dbp[2];
+        const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl) {
+          const int sb = 2 * HF + sl;
+          const f32x4 aM = mfma16(PM, Lr[sl], z4), aJ = mfma16(PJ, Lr[sl], z4);
+          // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
+          const f32x4 sM = mfma16(XM, Ls[sl], z4), sJ = mfma16(XJ, Ls[sl], z4);
+          const float vS = sV[16 * sb + i];
+          const float bS = sB[16 * sb + i];
+          float dvs = 0.f, dbs = 0.f, gm = gate[sl];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            dvs = fmaf(aM[r], kr[sl * 4 + r], dvs);
+            dbs = fmaf(aJ[r], kr2[sl * 4 + r], dbs);
+            dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
+            dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
+            gm = fmaf(aM[r], sM[r], gm);
+            gm = fmaf(aJ[r], sJ[r], gm);
+          }
+          gate[sl] = gm;
+          dvp[sl] = dvs;
+          dbp[sl] = dbs;
+          if (!HF && sl == 0 && i == 0) {
+            *(f32x4*)&car[dd * 32] = aM;
+            *(f32x4*)&car[dd * 32 + 4] = aJ;
+          }
+        }
+        pw[dd * kC] = rows4_sum_x4(dvp[0], dvp[1], dbp[0], dbp[1]);
+      }
+      iter_tail(it);
+    }
+    TIn* dkp = (TIn*)A.dk + ((int64_t)t0 * H + h) * dk + 16 * nb;
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl) {
+      const int s = 16 * (2 * HF + sl) + i;
+      if (s < clen) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          (dkp + (int64_t)s * rso)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
+      }
+      const float x = rows4_sum(gate[sl]);
+      if (g == 0) sRed[nbl * kC + 16 * (2 * HF + sl) + i] = x;
+    }
+  };
+
   // every role runs dv+1 iterations with the same barriers; a wave whose column block lies beyond dk
   // (last pass of a head dim that is not a multiple of 16*NB) only keeps the barriers
   float gm_tot = 0.f, sg_tot = 0.f;   // threads 0..63: gate term of token tid; thread 0: sum of dJloc
@@ -653,7 +944,12 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     if (MULTI && nbl >= n_act) {
       for (int it = 0; it < dv + LAGC; ++it) iter_tail(it);
     } else if (fold) {
-      if constexpr (!PREC) {
+      if constexpr (LAG) {
+        if (role == 0) producer_sub(std::integral_constant<int, 0>{});
+        else if (role == 1) producer_sub(std::integral_constant<int, 1>{});
+        else if (role == 2) consumer_sub(std::integral_constant<int, 0>{});
+        else consumer_sub(std::integral_constant<int, 1>{});
+      } else if constexpr (!PREC) {
         if (role == 0) producer(std::integral_constant<int, 0>{}, std::true_type{});
         else if (role == 1) producer(std::integral_constant<int, 1>{}, std::true_type{});
         else if (role == 2) consumer(std::integral_constant<int, 0>{}, std::true_type{});
@@ -1199,8 +1495,8 @@ struct BwdPlan {
 
 static size_t local_lds_bytes(int NB, bool var, bool prec) {
   const bool lag = local_lag(NB, prec);
-  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC + NB * kC + 16 +
-                          NB * (lag ? 128 : 64) + NB * kDG2 * 32) +
+  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC +
+                          NB * (lag ? 288 : 64) + NB * kDG2 * 32) +
          (size_t)NB * (lag ? 20 : 2 * (prec ? 16 : 8)) * 64 * 16;
 }
 
