@@ -65,6 +65,11 @@ extern "C" {
  * (its states are fp32: fused_recurrent_palimpsa.py:84-96, :145-154). */
 #define PAL_FLAG_STATE_MU_BF16 2048u
 
+/* pal_chunk_fwd only: fill chunk_mu / chunk_I (and the final states when asked for) and leave the outputs alone; o and
+ * o_var may be NULL.  For a backward whose forward did not keep the tile-start states: the token-serial entry point
+ * hands long sequences to pal_chunk_bwd this way.  No counterpart in the reference. */
+#define PAL_FLAG_STATES_ONLY 4096u
+
 /* error codes (negative) */
 #define PAL_OK 0
 #define PAL_E_NULL -1        /* required pointer is NULL                      */

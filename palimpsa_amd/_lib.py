@@ -17,6 +17,7 @@ PAL_DTYPE_F32, PAL_DTYPE_BF16 = 0, 1
 PAL_FLAG_VARLEN, PAL_FLAG_HAS_INIT, PAL_FLAG_STORE_FINAL, PAL_FLAG_HAS_VAR = 1, 2, 4, 8
 PAL_FLAG_STATES_TWO_KERNELS, PAL_FLAG_STATES_ONE_PASS, PAL_FLAG_FP32_FAST = 256, 512, 1024
 PAL_FLAG_STATE_MU_BF16 = 2048   # pal_recurrent_fwd: mu kept in bf16 between calls (DecodeStep(mu_dtype=torch.bfloat16))
+PAL_FLAG_STATES_ONLY = 4096     # pal_chunk_fwd: tile-start states only, outputs untouched
 PAL_CHUNK = 64
 
 PAL_E_NULL, PAL_E_DIM, PAL_E_HEADDIM, PAL_E_DTYPE, PAL_E_VARLEN_BATCH = -1, -2, -3, -4, -5
@@ -167,6 +168,23 @@ _fp32_fast = os.environ.get("PALIMPSA_FP32_FAST", "0") not in ("", "0")
 def set_fp32_fast(on: bool) -> None:
     global _fp32_fast
     _fp32_fast = bool(on)
+
+
+# Backward of the token-serial entry point: sequences of at least this many tokens on average are handed to the
+# chunked backward kernels (tile-start states from a states-only forward, then pal_chunk_bwd; fp32 rows keep the fp32
+# bar there through split operands), shorter ones run the token-serial backward kernel, which walks a sequence
+# token by token.  None = never.  Initial value from the environment variable PALIMPSA_RECURRENT_BWD_CHUNK_MIN.
+_recurrent_bwd_chunk_min = os.environ.get("PALIMPSA_RECURRENT_BWD_CHUNK_MIN", "128")
+_recurrent_bwd_chunk_min = None if _recurrent_bwd_chunk_min in ("", "none", "None") else int(_recurrent_bwd_chunk_min)
+
+
+def set_recurrent_bwd_chunk_min(tokens) -> None:
+    global _recurrent_bwd_chunk_min
+    _recurrent_bwd_chunk_min = None if tokens is None else int(tokens)
+
+
+def recurrent_bwd_chunk_min():
+    return _recurrent_bwd_chunk_min
 
 
 def state_pass_flags() -> int:

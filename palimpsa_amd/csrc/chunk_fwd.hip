@@ -1165,6 +1165,19 @@ extern "C" int pal_chunk_fwd_static(const PalDims* d, const PalFwdTensors* t, vo
 
 extern "C" int pal_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void* stream) {
   using namespace pal;
+  if (d && t && (d->flags & PAL_FLAG_STATES_ONLY)) {
+    // tile-start states only: the outputs are not touched and need not exist
+    PalDims dd = *d;
+    dd.flags &= ~(uint32_t)(PAL_FLAG_STATES_ONLY | PAL_FLAG_HAS_VAR);
+    PalFwdTensors tt = *t;
+    tt.o = (void*)(uintptr_t)256;   // passes the pointer checks, never dereferenced
+    tt.o_var = nullptr;
+    int rc = check_chunk_common(&dd, &tt);
+    if (rc) return rc;
+    ChunkArgs a;
+    fill_chunk_args(a, &dd, &tt);
+    return launch_tile_states(a, dd.dtype, true, (hipStream_t)stream);
+  }
   int rc = check_chunk_common(d, t);
   if (rc) return rc;
   ChunkArgs a;

@@ -7,7 +7,8 @@ ValueErrors.  Differences, all on purpose:
 
 * rows are consumed in their own dtype (bf16 or fp32) by the kernel; the
   reference casts seven tensors to fp32 on the host first (:226-236);
-* a backward exists (the reference raises NotImplementedError, :250-253).
+* a backward exists (the reference raises NotImplementedError, :250-253): the token-serial backward kernel for
+  short sequences, the chunked backward kernels (same gradients, tiles of 64 tokens in parallel) for long ones.
 """
 from __future__ import annotations
 
@@ -116,20 +117,53 @@ def recurrent_backward(p: "cm.Prepared", scale: float, do, do_var, in_dtypes, g_
         flags |= L.PAL_FLAG_HAS_INIT
     if has_var:
         flags |= L.PAL_FLAG_HAS_VAR
-    dims = L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
-                     dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
-                     flags=flags, scale=float(scale), n_qk_heads=q.shape[2])
     pt = cm._ptr
-    tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
-                           init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))
     grads = L.PalBwdTensors(d_o=pt(do_p), d_o_var=pt(dovar_p), dq=pt(dq), dk=pt(dk_), dv=pt(dv_), db=pt(db),
                             dgt=pt(dgt), dg=pt(dg), dIp=pt(dIp), d_init_mu=pt(d_init_mu), d_init_I=pt(d_init_I))
     lib = L.load()
-    ws_bytes = int(lib.pal_recurrent_bwd_workspace_bytes(dims))
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
-        rc = lib.pal_recurrent_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, cm.current_stream_ptr(dev))
-    L.check(rc, "pal_recurrent_bwd")
+    mode_flags = L.state_pass_flags()
+    route_min = L.recurrent_bwd_chunk_min()
+    if (route_min is not None and B * T >= route_min * p.n_seqs
+            and lib.pal_chunk_bwd_supported(dk_p, dv_p, cm._pal_dtype(cd), mode_flags) == 0):
+        # Long sequences: the token-serial backward walks every sequence token by token (a few microseconds per
+        # token and sequence whatever the batch), the chunked backward works on all tiles of 64 tokens at once.  The
+        # tile-start states it needs come from a states-only pass of the chunked forward; fp32 rows keep the fp32 bar
+        # (split operands).  Same gradients, tested against each other and against the oracle.
+        table = offsets = None
+        if cu is not None:
+            meta, total_chunks = cm.chunk_meta(cu, T, dev)
+            offsets, table = meta[: p.n_seqs + 1], meta[p.n_seqs + 1:]
+        else:
+            total_chunks = (T + L.PAL_CHUNK - 1) // L.PAL_CHUNK * B
+        tile_mu = torch.empty(total_chunks, H, dv_p, dk_p, dtype=torch.float32, device=dev)
+        tile_I = torch.empty_like(tile_mu)
+        dims = L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=dk_p, dv=dv_p, total_chunks=total_chunks,
+                         dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
+                         flags=(flags & ~L.PAL_FLAG_HAS_VAR) | mode_flags | L.PAL_FLAG_STATES_ONLY, scale=float(scale),
+                         n_qk_heads=q.shape[2])
+        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=None,
+                               init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu), chunk_table=pt(table),
+                               chunk_offsets=pt(offsets), chunk_mu=pt(tile_mu), chunk_I=pt(tile_I))
+        with torch.cuda.device(dev):
+            stream = cm.current_stream_ptr(dev)
+            L.check(lib.pal_chunk_fwd(dims, tens, stream), "pal_chunk_fwd (tile-start states)")
+            dims.flags = flags | mode_flags
+            tens.o = pt(do_p)
+            ws_bytes = int(lib.pal_chunk_bwd_workspace_bytes(dims))
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+            rc = lib.pal_chunk_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, stream)
+        L.check(rc, "pal_chunk_bwd")
+    else:
+        dims = L.PalDims(batch=B, seq_len=T, n_seqs=p.n_seqs, n_heads=H, dk=dk_p, dv=dv_p, total_chunks=0,
+                         dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype), var_dtype=L.PAL_DTYPE_F32,
+                         flags=flags, scale=float(scale), n_qk_heads=q.shape[2])
+        tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), b=pt(b), gt=pt(gt), g=pt(g), Ip=pt(Ip), o=pt(do_p),
+                               init_mu=pt(init_mu), init_I=pt(init_I), cu_seqlens=pt(cu))
+        ws_bytes = int(lib.pal_recurrent_bwd_workspace_bytes(dims))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.pal_recurrent_bwd(dims, tens, grads, C.c_void_p(ws.data_ptr()), ws_bytes, cm.current_stream_ptr(dev))
+        L.check(rc, "pal_recurrent_bwd")
     dts = in_dtypes
     dq = cm.unpad_last(dq, p.dk).to(dts[0])
     dk_ = cm.unpad_last(dk_, p.dk).to(dts[1])

@@ -176,6 +176,20 @@ def test_chunk_table_rejects_bad_cu_seqlens(L):
     assert lib.pal_build_chunk_table(None, 2, None, 0, None) == L.PAL_E_NULL
 
 
+def test_states_only_forward_checks_its_arguments(L):
+    """PAL_FLAG_STATES_ONLY: pal_chunk_fwd fills the tile-start states and leaves the outputs alone, so o may be NULL;
+    everything else is checked as usual, before any HIP call."""
+    lib = L.load()
+    so = L.PAL_FLAG_STATES_ONLY
+    assert lib.pal_chunk_fwd(_dims(L, flags=so), _fwd_tensors(L, o=None), None) == L.PAL_E_NULL             # no state buffers
+    assert lib.pal_chunk_fwd(_dims(L, flags=so, total_chunks=3),
+                             _fwd_tensors(L, o=None, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)), None) == L.PAL_E_CHUNK
+    assert lib.pal_chunk_fwd(_dims(L, flags=so), _fwd_tensors(L, o=None, q=None, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)),
+                             None) == L.PAL_E_NULL
+    assert lib.pal_chunk_fwd(_dims(L, flags=so | L.PAL_FLAG_HAS_INIT),
+                             _fwd_tensors(L, o=None, chunk_mu=_fake(0x9000), chunk_I=_fake(0xa000)), None) == L.PAL_E_STATE
+
+
 def test_simple_gla_entry_points_reject_bad_arguments(L):
     """Host-side checks of the entry points without the precision state (no HIP call before they pass)."""
     lib = L.load()

@@ -221,6 +221,61 @@ def test_bf16_rows_backward(gpu_device):
         assert hp.max_rel(got[n], ref[n]) <= hp.BF16_GRAD_NORM_TOL, n
 
 
+@pytest.mark.parametrize("rows", ["fp32", "bf16"])
+def test_long_sequences_take_the_chunked_backward(gpu_device, rows):
+    """Sequences of 128 tokens or more on average: the backward of the token-serial entry point runs the chunked
+    backward kernels on tile-start states from a states-only forward pass.  Dense and packed, initial state and
+    uncertainty gradients included: against float64 autograd through the oracle at the bar of the row dtype, and
+    against the token-serial backward kernel (the route switched off) on the same inputs."""
+    from palimpsa_amd import _lib as L
+    H, dk, dv = 2, 64, 32
+    cu = [0, 200, 201, 520, 700]
+    T, N = cu[-1], len(cu) - 1
+    inp = po.make_inputs(1, T, H, dk, dv, seed=71)
+    if rows == "bf16":
+        inp = hp.rounded(inp, torch.bfloat16)
+    inp["g"] = torch.tensor([0.7, 5.0])
+    gen = torch.Generator().manual_seed(72)
+    mu0 = torch.randn(N, H, dv, dk, generator=gen) * 0.1
+    I0 = 1.0 + torch.rand(N, H, dv, dk, generator=gen)
+    do = torch.randn(1, T, H, dv, generator=gen)
+    dovar = torch.randn(1, T, H, dv, generator=gen) * 0.3
+    ref = hp.oracle_grads(inp, do, dovar, mu0=mu0, I0=I0, cu=cu)
+    assert L.recurrent_bwd_chunk_min() is not None and T >= L.recurrent_bwd_chunk_min() * N
+    L.profile_enable(True)
+    got = _rec_grads(inp, gpu_device, do, dovar, mu0=mu0, I0=I0, cu=cu)
+    torch.cuda.synchronize()
+    ran = L.profile_read()
+    L.profile_enable(False)
+    assert "chunk_bwd_local_kernel" in ran and "recurrent_bwd_kernel" not in ran, sorted(ran)
+    try:
+        L.set_recurrent_bwd_chunk_min(None)
+        serial = _rec_grads(inp, gpu_device, do, dovar, mu0=mu0, I0=I0, cu=cu)
+    finally:
+        L.set_recurrent_bwd_chunk_min(128)
+    names = ["q", "k", "v", "b", "gt", "g", "Ip", "mu0", "I0"]
+    if rows == "fp32":
+        for n in names:
+            assert hp.max_rel(got[n], ref[n]) <= GRAD_TOL, (n, hp.max_rel(got[n], ref[n]))
+            assert hp.max_rel(got[n], serial[n]) <= 2 * GRAD_TOL, (n, hp.max_rel(got[n], serial[n]))
+    else:
+        mass = ((inp["gt"].double() * ref["gt"].double()).abs().sum(dim=(0, 1)) / inp["g"].double()).max().item()
+        for n in names:
+            if n == "g":    # random dO: |dg| is far below the l1 mass of its terms (tests/test_gpu_chunk_bwd.py)
+                err = (got[n].double().cpu() - ref[n].double()).abs().max().item() / mass
+            else:
+                err = hp.max_rel(got[n], ref[n])
+            assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)
+    # a dense batch of short sequences stays with the token-serial kernel
+    short = po.make_inputs(2, 60, H, dk, dv, seed=73)
+    L.profile_enable(True)
+    _rec_grads(short, gpu_device, torch.randn(2, 60, H, dv, generator=gen))
+    torch.cuda.synchronize()
+    ran = L.profile_read()
+    L.profile_enable(False)
+    assert "recurrent_bwd_kernel" in ran and "chunk_bwd_local_kernel" not in ran, sorted(ran)
+
+
 def test_bound_decode_step_matches_entry_point_and_replays_in_a_graph(gpu_device):
     """DecodeStep binds tensors once and updates the state in place: same kernel as
     fused_recurrent_palimpsa with T = 1, so results agree exactly; recorded into a HIP graph (the step
