@@ -1459,6 +1459,22 @@ __global__ __launch_bounds__(256) void group_sum_kernel(const T* src_q, const T*
   store_vec<4>(dst_k + row * dk + 4 * c4, ak);
 }
 
+// dq, dk of [tokens, Hq * rep, dk] summed over the rep value heads of each group into [tokens, Hq, dk]
+int launch_group_sum(const void* src_q, const void* src_k, void* dst_q, void* dst_k, int64_t tokens, int Hq, int rep, int dk,
+                     int dtype, hipStream_t s) {
+  const int64_t n4 = tokens * Hq * (dk / 4);
+  if ((n4 + 255) / 256 > 0x7fffffff) return PAL_E_DIM;
+  const unsigned gblocks = (unsigned)((n4 + 255) / 256);
+  if (dtype == PAL_DTYPE_BF16)
+    hipLaunchKernelGGL(group_sum_kernel<bf16_t>, dim3(gblocks), dim3(256), 0, s, (const bf16_t*)src_q, (const bf16_t*)src_k,
+                       (bf16_t*)dst_q, (bf16_t*)dst_k, n4, Hq, rep, dk);
+  else
+    hipLaunchKernelGGL(group_sum_kernel<float>, dim3(gblocks), dim3(256), 0, s, (const float*)src_q, (const float*)src_k,
+                       (float*)dst_q, (float*)dst_k, n4, Hq, rep, dk);
+  PAL_HIP_LAUNCH_CHECK();
+  return PAL_OK;
+}
+
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static BwdLayout bwd_layout(const PalDims* d) {
@@ -1667,14 +1683,7 @@ extern "C" int pal_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const Pal
   PAL_TIMED_LAUNCH(kKernBwdHeadReduce, s, chunk_bwd_head_reduce_kernel, dim3((unsigned)dd.n_heads), dim3(64), 0, s, A);
   PAL_HIP_LAUNCH_CHECK();
   if (grouped) {
-    const int64_t n4 = (int64_t)A.tokens * A.c.Hq * (dd.dk / 4);
-    const unsigned gblocks = (unsigned)((n4 + 255) / 256);
-    const int rep = A.c.H / A.c.Hq;
-    if (bf) hipLaunchKernelGGL(group_sum_kernel<bf16_t>, dim3(gblocks), dim3(256), 0, s, (const bf16_t*)A.dq, (const bf16_t*)A.dk,
-                               (bf16_t*)gr->dq, (bf16_t*)gr->dk, n4, A.c.Hq, rep, dd.dk);
-    else hipLaunchKernelGGL(group_sum_kernel<float>, dim3(gblocks), dim3(256), 0, s, (const float*)A.dq, (const float*)A.dk,
-                            (float*)gr->dq, (float*)gr->dk, n4, A.c.Hq, rep, dd.dk);
-    PAL_HIP_LAUNCH_CHECK();
+    if (int rc2 = launch_group_sum(A.dq, A.dk, gr->dq, gr->dk, A.tokens, A.c.Hq, A.c.H / A.c.Hq, dd.dk, dd.dtype, s)) return rc2;
   }
   return PAL_OK;
 }

@@ -17,6 +17,8 @@ namespace pal {
 void fill_chunk_args(ChunkArgs& a, const PalDims* d, const PalFwdTensors* t);
 int launch_tile_states(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
 int launch_tile_delta(const ChunkArgs& a, int dtype, bool has_j, hipStream_t s);
+int launch_group_sum(const void* src_q, const void* src_k, void* dst_q, void* dst_k, int64_t tokens, int Hq, int rep, int dk,
+                     int dtype, hipStream_t s);
 bool state_pass_applies(const ChunkArgs& a, int dtype, bool has_j);
 int launch_state_pass(const ChunkArgs& a, bool has_j, void* tiles_a, float* tiles_b, const float* init_a,
                       const float* init_b, float* fin_a, float* fin_b, bool reverse, float fin_scale, int kern_id,
@@ -48,6 +50,9 @@ struct GlaTileArgs {
   float* dot;             // [H][tokens] (head-major, so that the gate kernel reads contiguous rows) or null
   int64_t n_tokens;       // tokens in the batch (row length of dot)
   int32_t dc, de;         // contraction width of the scores, width of the output rows
+  // heads in X, Y, Z and W (H, or the number of shared q/k heads where the tensor is q or k: value head h then reads
+  // the rows of head h / (H / heads)); out always has one row per value head
+  int32_t hX, hY, hZ, hW;
 };
 
 // One kernel for the tile-parallel part of the forward and of the three input gradients.  For the 64
@@ -96,6 +101,9 @@ __global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     sC[lane] = wave_inclusive_scan(-gt * gh, lane);
   }
+  // head of this workgroup's rows in each tensor, and the tensors' token strides in heads
+  const int hsX = A.hX, hsY = A.hY, hsZ = A.hZ, hsW = A.hW;
+  const int hx = h / (H / hsX), hy = h / (H / hsY), hz = h / (H / hsZ), hw = h / (H / hsW);
   // X rows of token block xb as a B operand (column x = 16 xb + i, contraction index c = 32 ks + 8 g + j), from LDS
   auto x_operand = [&](int xb, int ks) { return *(const bf16x8*)(sX + (16 * xb + i) * dcp + 8 * g + 32 * ks); };
   // State operands of this wave: blocks of 16 output columns [w EB, (w+1) EB), rows e = 16 eb + i, contraction
@@ -129,14 +137,14 @@ __global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
   fetch_state(0);
   {
     // Y rows, zero beyond the tile's tokens and beyond dc
-    const TIn* yp = (const TIn*)A.Y + ((int64_t)t0 * H + h) * dc;
+    const TIn* yp = (const TIn*)A.Y + ((int64_t)t0 * hsY + hy) * dc;
     const int groups = 4 * KS;
     for (int idx = tid; idx < kC * groups; idx += 256) {
       const int s = idx / groups, c8 = idx - s * groups;
       bf16x8 yx = {0, 0, 0, 0, 0, 0, 0, 0}, xx = {0, 0, 0, 0, 0, 0, 0, 0};
       if (s < clen && 8 * c8 < dc) {
-        yx = load_bf16x8(yp + (int64_t)s * H * dc + 8 * c8);
-        xx = load_bf16x8((const TIn*)A.X + ((int64_t)(t0 + s) * H + h) * dc + 8 * c8);
+        yx = load_bf16x8(yp + (int64_t)s * hsY * dc + 8 * c8);
+        xx = load_bf16x8((const TIn*)A.X + ((int64_t)(t0 + s) * hsX + hx) * dc + 8 * c8);
       }
       *(bf16x8*)&sY[s * dcp + 8 * c8] = yx;
       *(bf16x8*)&sX[s * dcp + 8 * c8] = xx;
@@ -144,13 +152,13 @@ __global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
     // Z transposed (token index fastest), zero beyond the tile's tokens.  A work item is two consecutive
     // tokens by eight columns: neighbouring lanes read neighbouring 16-byte pieces of a row, and a
     // pair of tokens goes to LDS as one 32-bit word per column.
-    const TIn* zp = (const TIn*)A.Z + ((int64_t)t0 * H + h) * de;
+    const TIn* zp = (const TIn*)A.Z + ((int64_t)t0 * hsZ + hz) * de;
     const int zgroups = de >> 3;
     for (int idx = tid; idx < (kC / 2) * zgroups; idx += 256) {
       const int sp = idx / zgroups, c8 = idx - sp * zgroups;
       bf16x8 z0 = {0, 0, 0, 0, 0, 0, 0, 0}, z1 = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (2 * sp < clen) z0 = load_bf16x8(zp + (int64_t)(2 * sp) * H * de + 8 * c8);
-      if (2 * sp + 1 < clen) z1 = load_bf16x8(zp + (int64_t)(2 * sp + 1) * H * de + 8 * c8);
+      if (2 * sp < clen) z0 = load_bf16x8(zp + (int64_t)(2 * sp) * hsZ * de + 8 * c8);
+      if (2 * sp + 1 < clen) z1 = load_bf16x8(zp + (int64_t)(2 * sp + 1) * hsZ * de + 8 * c8);
 #pragma unroll
       for (int e = 0; e < 8; ++e) *(bf16x2*)&sZT[(8 * c8 + e) * kVT + 2 * sp] = bf16x2{z0[e], z1[e]};
     }
@@ -254,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void gla_tile_kernel(GlaTileArgs A) {
       for (int r = 0; r < 4; ++r) acc[el][xb][r] *= scale;
       if (has_dot && valid && x < clen) {
         float wv[4];
-        load_vec<4>((const TIn*)A.W + ((int64_t)(t0 + x) * H + h) * de + 16 * eb + 4 * g, wv);
+        load_vec<4>((const TIn*)A.W + ((int64_t)(t0 + x) * hsW + hw) * de + 16 * eb + 4 * g, wv);
 #pragma unroll
         for (int r = 0; r < 4; ++r) dot[xb] = fmaf(wv[r], acc[el][xb][r], dot[xb]);
       }
@@ -345,7 +353,7 @@ static int launch_gla_tile_dt(const GlaTileArgs& A, int dtype, GlaRole role, hip
 // products (q for q.dq, k for k.dk) come from the same tiles.
 struct GlaBwdTileArgs {
   ChunkArgs c;                  // T, H, tiles, gate (gt, g), scale, dk, dv
-  const void *q, *k, *v, *d_o;  // rows [token][H][dk | dv]
+  const void *q, *k, *v, *d_o;  // rows [token][H][dv] (v, dO), [token][Hq][dk] (q, k: c.Hq heads)
   const bf16_t *S, *G;          // tile-start states and gradients of the tile-end states, [tile][H][dv][dk]
   void *dq, *dk, *dv;
   float *qdq, *kdk;             // [H][tokens]
@@ -439,7 +447,9 @@ __global__ __launch_bounds__(512, 4) void gla_bwd_tile_kernel(GlaBwdTileArgs A) 
     for (int u = 0; u < 2; ++u) {
       const int s = 2 * sp + u;
       const bool on = s < m.clen && 8 * c8 < d;
-      const int64_t row = ((int64_t)(m.t0 + (on ? s : 0)) * H + m.h) * d + (on ? 8 * c8 : 0);
+      // q and k may carry fewer heads than v and dO (a group of value heads shares one)
+      const int hn = upper ? H : a.Hq, hh = upper ? m.h : m.h / (H / a.Hq);
+      const int64_t row = ((int64_t)(m.t0 + (on ? s : 0)) * hn + hh) * d + (on ? 8 * c8 : 0);
       ra[u] = on ? *(const bf16x8*)(pa + row) : zero;
       rb[u] = on ? *(const bf16x8*)(pb + row) : zero;
       const bool ons = s < dv && 8 * c8 < dk;
@@ -656,7 +666,6 @@ static int check_gla(const PalDims* d, const PalFwdTensors* t) {
   if (!t->q || !t->k || !t->v || !t->gt || !t->g || !t->o || !t->chunk_I) return PAL_E_NULL;
   if (d->flags & PAL_FLAG_HAS_VAR) return PAL_E_STATE;   // no precision state, no output variance
   if (d->flags & PAL_FLAG_STATE_MU_BF16) return PAL_E_STATE;
-  if (d->n_qk_heads != 0 && d->n_qk_heads != d->n_heads) return PAL_E_DIM;   // shared q/k heads: Palimpsa entry points only
   if (((d->flags & PAL_FLAG_HAS_INIT) != 0) != (t->init_mu != nullptr)) return PAL_E_STATE;
   if (((d->flags & PAL_FLAG_STORE_FINAL) != 0) != (t->final_mu != nullptr)) return PAL_E_STATE;
   const bool varlen = d->flags & PAL_FLAG_VARLEN;
@@ -821,7 +830,7 @@ __global__ void gla_bwd_head_reduce_kernel(const float* dg_part, float* dg, int 
 // workspace of the backward: per-tile contributions D (fp32), G tiles (bf16), the two dot-product rows,
 // per-sequence shares of dg
 struct GlaBwdWorkspace {
-  size_t d_tiles, g_tiles, qdq, kdk, dg_part, total;
+  size_t d_tiles, g_tiles, qdq, kdk, dg_part, dq_full, dk_full, total;
 };
 static GlaBwdWorkspace gla_bwd_layout(const PalDims* d) {
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
@@ -834,6 +843,12 @@ static GlaBwdWorkspace gla_bwd_layout(const PalDims* d) {
   w.kdk = w.qdq + up(sizeof(float) * tokens * d->n_heads);
   w.dg_part = w.kdk + up(sizeof(float) * tokens * d->n_heads);
   w.total = w.dg_part + up(sizeof(float) * (size_t)d->n_seqs * d->n_heads);
+  w.dq_full = w.dk_full = w.total;
+  if (d->n_qk_heads > 0 && d->n_qk_heads != d->n_heads) {   // one dq, dk row per value head, summed per group at the end
+    const size_t full = up(tokens * d->n_heads * d->dk * (d->dtype == PAL_DTYPE_BF16 ? 2 : 4));
+    w.dk_full = w.dq_full + full;
+    w.total = w.dk_full + full;
+  }
   return w;
 }
 
@@ -867,6 +882,11 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   ChunkArgs a;
   fill_gla_args(a, d, t);
   a.final_mu = nullptr;
+  // shared q/k heads: the kernels leave one dq, dk row per value head in the workspace; they are summed over each
+  // group in a fixed order at the end (the gate terms q.dq, k.dk are per value head anyway)
+  const bool grouped = a.Hq != a.H;
+  void* dq_out = grouped ? (void*)(ws + w.dq_full) : gr->dq;
+  void* dk_out = grouped ? (void*)(ws + w.dk_full) : gr->dk;
   // D_c = sum_t F_t dO_t q_t^T per tile, then the reverse scan over the tiles of each sequence
   {
     ChunkArgs b = a;
@@ -889,7 +909,7 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
     F.c = a;
     F.q = t->q; F.k = t->k; F.v = t->v; F.d_o = gr->d_o;
     F.S = (const bf16_t*)t->chunk_I; F.G = g_tiles;
-    F.dq = gr->dq; F.dk = gr->dk; F.dv = gr->dv; F.qdq = qdq; F.kdk = kdk;
+    F.dq = dq_out; F.dk = dk_out; F.dv = gr->dv; F.qdq = qdq; F.kdk = kdk;
     F.n_tokens = (int64_t)d->batch * d->seq_len;
     if (int rc = launch_gla_bwd_tile(F, s)) return rc;
   } else {
@@ -897,16 +917,19 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
   A.c = a;
   A.n_tokens = (int64_t)d->batch * d->seq_len;
   // dq: X = dO, Y = v, Z = k, tile-start states read transposed; q . dq on the side
-  A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = (const bf16_t*)t->chunk_I; A.out = gr->dq; A.W = t->q; A.dot = qdq;
+  A.X = gr->d_o; A.Y = t->v; A.Z = t->k; A.St = (const bf16_t*)t->chunk_I; A.out = dq_out; A.W = t->q; A.dot = qdq;
   A.dc = d->dv; A.de = d->dk;
+  A.hX = a.H; A.hY = a.H; A.hZ = a.Hq; A.hW = a.Hq;
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDq, s)) return rc;
   // dv: X = k, Y = q, Z = dO, tile-end state gradients
   A.X = t->k; A.Y = t->q; A.Z = gr->d_o; A.St = g_tiles; A.out = gr->dv; A.W = nullptr; A.dot = nullptr;
   A.dc = d->dk; A.de = d->dv;
+  A.hX = a.Hq; A.hY = a.Hq; A.hZ = a.H; A.hW = a.H;
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDv, s)) return rc;
   // dk: X = v, Y = dO, Z = q, tile-end state gradients read transposed; k . dk on the side
-  A.X = t->v; A.Y = gr->d_o; A.Z = t->q; A.St = g_tiles; A.out = gr->dk; A.W = t->k; A.dot = kdk;
+  A.X = t->v; A.Y = gr->d_o; A.Z = t->q; A.St = g_tiles; A.out = dk_out; A.W = t->k; A.dot = kdk;
   A.dc = d->dv; A.de = d->dk;
+  A.hX = a.H; A.hY = a.H; A.hZ = a.Hq; A.hW = a.Hq;
   if (int rc = launch_gla_tile_dt(A, d->dtype, kGlaDk, s)) return rc;
   }
   {
@@ -917,6 +940,11 @@ extern "C" int pal_gla_chunk_bwd(const PalDims* d, const PalFwdTensors* t, const
     hipLaunchKernelGGL(gla_bwd_head_reduce_kernel, dim3((d->n_heads + 63) / 64), dim3(64), 0, s, dg_part, gr->dg,
                        d->n_seqs, d->n_heads);
     PAL_HIP_LAUNCH_CHECK();
+  }
+  if (grouped) {
+    if (int rc = launch_group_sum(dq_out, dk_out, gr->dq, gr->dk, (int64_t)d->batch * d->seq_len, a.Hq, a.H / a.Hq, d->dk,
+                                  d->dtype, s))
+      return rc;
   }
   return PAL_OK;
 }
@@ -934,5 +962,6 @@ extern "C" int pal_gla_chunk_fwd(const PalDims* d, const PalFwdTensors* t, void*
   A.c = a;
   A.X = t->q; A.Y = t->k; A.Z = t->v; A.St = (const bf16_t*)t->chunk_I; A.out = t->o;
   A.dc = d->dk; A.de = d->dv;
+  A.hX = a.Hq; A.hY = a.Hq; A.hZ = a.H; A.hW = a.H;
   return launch_gla_tile_dt(A, d->dtype, kGlaOut, s);
 }

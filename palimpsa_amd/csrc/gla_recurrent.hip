@@ -24,6 +24,7 @@ struct GlaRecArgs {
   float* final_;
   const int32_t* cu_seqlens;
   int32_t T, H, dk, dv, n_seqs, gate_bf16;
+  int32_t Hq;   // heads of q and k (H, or a divisor of it: a group of H / Hq value heads shares one)
   float scale;
 };
 
@@ -61,12 +62,13 @@ __global__ __launch_bounds__(256) void gla_recurrent_fwd_kernel(GlaRecArgs a) {
 #pragma unroll
     for (int e = 0; e < NQ; ++e) S[e] = __builtin_nontemporal_load(a.init + sbase + (int64_t)e * dv);
   }
-  const TIn* qp = (const TIn*)a.q + (bos * H + h) * dk + n0;
-  const TIn* kp = (const TIn*)a.k + (bos * H + h) * dk + n0;
+  const int Hq = a.Hq, hq = h / (H / Hq);
+  const TIn* qp = (const TIn*)a.q + (bos * Hq + hq) * dk + n0;
+  const TIn* kp = (const TIn*)a.k + (bos * Hq + hq) * dk + n0;
   const TIn* vp = (const TIn*)a.v + (bos * H + h) * dv + d;
   TIn* op = (TIn*)a.o + (bos * H + h) * dv + d;
   for (int t = 0; t < T; ++t) {
-    const int64_t off_k = (int64_t)t * H * dk, off_v = (int64_t)t * H * dv;
+    const int64_t off_k = (int64_t)t * Hq * dk, off_v = (int64_t)t * H * dv;
     const float f = fast_exp2(-load_gate(a.gt, (bos + t) * H + h, a.gate_bf16) * gh);
     const float v = on ? to_f32(vp[off_v]) : 0.f;
     float acc = 0.f;
@@ -142,6 +144,7 @@ extern "C" int pal_gla_recurrent_fwd(const PalDims* d, const PalFwdTensors* t, v
   a.q = t->q; a.k = t->k; a.v = t->v; a.gt = t->gt; a.g = t->g; a.o = t->o;
   a.init = t->init_mu; a.final_ = t->final_mu; a.cu_seqlens = t->cu_seqlens;
   a.T = d->seq_len; a.H = d->n_heads; a.dk = d->dk; a.dv = d->dv; a.n_seqs = d->n_seqs;
+  a.Hq = d->n_qk_heads > 0 ? d->n_qk_heads : d->n_heads;
   a.gate_bf16 = d->gate_dtype == PAL_DTYPE_BF16;
   a.scale = d->scale;
   hipStream_t s = (hipStream_t)stream;

@@ -18,6 +18,11 @@ division by ``I`` a tile's output is two plain matrix products, so the per-token
 ``fused_recurrent_simple_gla`` without autograd runs ``pal_gla_recurrent_fwd``, which keeps the state in the
 caller's ``[N, H, dk, dv]`` layout; with autograd it runs the Palimpsa token-serial kernels with ``b = 0``,
 ``Ip = 1`` and ``gt = -g`` under a unit per-head rate (the precision branch then works on zeros).
+
+``q`` and ``k`` may carry fewer heads than ``v`` (``[B, T, Hq, dk]`` with ``Hq`` a divisor of ``H``): a group of
+``H / Hq`` value heads then shares one q/k head, which is what the reference's MetaMamba2 layer obtains by repeating
+its ``B``, ``C`` groups before the call (layers/meta_mamba2.py:281-282); the kernels index the shared rows and
+``dq``, ``dk`` come back summed over each group.  ``g`` is always ``[B, T, H]``.
 """
 from __future__ import annotations
 
@@ -50,9 +55,9 @@ def _minus_one_rate(H: int, dev: torch.device) -> torch.Tensor:
 def _run(op, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, **kw):
     if g is None:
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
-    if g.shape != q.shape[:3]:
-        raise ValueError(f"g must have shape {tuple(q.shape[:3])}, got {tuple(g.shape)}")
-    H = q.shape[2]
+    if g.shape != v.shape[:3]:
+        raise ValueError(f"g must have shape {tuple(v.shape[:3])}, got {tuple(g.shape)}")
+    H = v.shape[2]
     dev = q.device
     b = torch.zeros_like(v)
     rate = torch.ones(H, dtype=torch.float32, device=dev)
@@ -76,7 +81,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens):
-        H = q.shape[2]
+        H = v.shape[2]
         dev = q.device
         rate = _minus_one_rate(H, dev)
         S0 = None
@@ -128,8 +133,8 @@ class ChunkSimpleGLA(torch.autograd.Function):
         q, k, v, gt, rate, init, cu, table, offsets, tile_S = ctx.saved_tensors
         m = ctx.meta
         dev = q.device
-        B, T, H, dk_p = q.shape
-        dv_p = v.shape[-1]
+        B, T, Hq, dk_p = q.shape
+        H, dv_p = v.shape[2], v.shape[-1]
         cd = m["compute_dtype"]
         if do is None:
             do = torch.zeros(B, T, H, m["dv"], dtype=cd, device=dev)
@@ -143,7 +148,7 @@ class ChunkSimpleGLA(torch.autograd.Function):
         d_init = torch.empty_like(init) if init is not None else None
         dims = L.PalDims(batch=B, seq_len=T, n_seqs=m["n_seqs"], n_heads=H, dk=dk_p, dv=dv_p,
                          total_chunks=m["total_chunks"], dtype=cm._pal_dtype(cd), gate_dtype=cm._pal_dtype(gt.dtype),
-                         var_dtype=cm._pal_dtype(cd), flags=m["flags"], scale=m["scale"])
+                         var_dtype=cm._pal_dtype(cd), flags=m["flags"], scale=m["scale"], n_qk_heads=Hq)
         pt = cm._ptr
         tens = L.PalFwdTensors(q=pt(q), k=pt(k), v=pt(v), gt=pt(gt), g=pt(rate), o=pt(do), init_mu=pt(init),
                                cu_seqlens=pt(cu), chunk_table=pt(table), chunk_offsets=pt(offsets), chunk_I=pt(tile_S))
@@ -164,11 +169,11 @@ class ChunkSimpleGLA(torch.autograd.Function):
         return dq, dk, dv, dg_tok.to(dts[3]), None, d_init, None, None
 
 
-def _check_chunk_args(q, g, cu_seqlens):
+def _check_chunk_args(q, v, g, cu_seqlens):
     if g is None:
         raise ValueError("g (log decay per token and head, [B, T, H]) is required")
-    if g.shape != q.shape[:3]:
-        raise ValueError(f"g must have shape {tuple(q.shape[:3])}, got {tuple(g.shape)}")
+    if v.dim() != 4 or g.shape != v.shape[:3]:
+        raise ValueError(f"g must have shape {tuple(v.shape[:3])}, got {tuple(g.shape)}")
     if cu_seqlens is not None:
         if q.shape[0] != 1:
             raise ValueError(f"Batch size must be 1 for Varlen, got {q.shape[0]}")
@@ -181,7 +186,7 @@ def chunk_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: Optio
                      scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                      output_final_state: bool = False, cu_seqlens: Optional[torch.Tensor] = None):
     """Chunked (training / prefill) form; returns ``(o, final_state | None)``."""
-    _check_chunk_args(q, g, cu_seqlens)
+    _check_chunk_args(q, v, g, cu_seqlens)
     if scale is None:
         scale = q.shape[-1] ** -0.5
     return ChunkSimpleGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
@@ -198,10 +203,10 @@ def fused_recurrent_simple_gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
         isinstance(x, torch.Tensor) and x.requires_grad for x in (q, k, v, g, initial_state))
     if needs_grad:
         return _run(fused_recurrent_palimpsa, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens)
-    _check_chunk_args(q, g, cu_seqlens)
+    _check_chunk_args(q, v, g, cu_seqlens)
     if scale is None:
         scale = q.shape[-1] ** -0.5
-    H = q.shape[2]
+    H = v.shape[2]
     dev = q.device
     rate = _minus_one_rate(H, dev)
     p = cm.prepare_inputs(q, k, v, v, g, rate, rate, None, None, cu_seqlens, recurrent=False)

@@ -205,6 +205,8 @@ def test_simple_gla_entry_points_reject_bad_arguments(L):
         assert fn(_dims(L), _fwd_tensors(L, cu_seqlens=_fake(), **ok), None) == L.PAL_E_CU_SEQLENS
         assert fn(_dims(L), _fwd_tensors(L, v=_fake(0x3008), **ok), None) == L.PAL_E_ALIGN
         assert fn(_dims(L, gate_dtype=L.PAL_DTYPE_BF16), _fwd_tensors(L, gt=_fake(0x5002), **ok), None) == L.PAL_E_ALIGN
+    # q, k with fewer heads than v: a divisor of the head count, as for the Palimpsa entry points
+    assert lib.pal_gla_chunk_fwd(_dims(L, n_qk_heads=3), _fwd_tensors(L, **ok), None) == L.PAL_E_DIM
     # the chunked form needs both tile buffers and a consistent tile count
     assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_mu=_fake(0x9000)), None) == L.PAL_E_NULL
     assert lib.pal_gla_chunk_fwd(_dims(L), _fwd_tensors(L, chunk_I=_fake(0xa000)), None) == L.PAL_E_NULL

@@ -655,3 +655,67 @@ def test_forward_and_backward_replay_in_a_graph(gpu_device):
         torch.cuda.synchronize()
         for a_, b_, n in zip((o_g,) + tuple(grads_g), ref, "oqkvg"):
             assert torch.equal(a_, b_), (seed, n)
+
+
+@pytest.mark.parametrize("dk,dv,dtype", [(64, 64, torch.bfloat16), (48, 96, torch.bfloat16), (32, 64, torch.float32)])
+def test_shared_qk_heads_are_indexed_not_repeated(gpu_device, dk, dv, dtype):
+    """The MetaMamba2 layer with its precision state off repeats its B, C groups over the heads of a group before it
+    calls simple-GLA (layers/meta_mamba2.py:281-282, then :319-323).  The entry points also take the un-repeated
+    [B,T,Hq,dk] rows and index the shared ones: outputs, final state and every gradient must equal the dense closed
+    form on the repeated rows, with dq, dk summed over the heads of each group.  64 x 64 bf16 runs the backward
+    kernel that forms the three input gradients together, the other shapes the three launches; packed documents
+    in the first case; the decode kernel on the same rows."""
+    from palimpsa_amd.ops.simple_gla import chunk_simple_gla, fused_recurrent_simple_gla
+    B, T, H, G = 2, 200, 6, 2
+    rep = H // G
+    q, k, v, g, S0 = _inputs(B, T, H, dk, dv, 91)
+    q = q[:, :, ::rep].repeat_interleave(rep, dim=2).contiguous()     # heads of a group carry the same rows
+    k = k[:, :, ::rep].repeat_interleave(rep, dim=2).contiguous()
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    gen = torch.Generator().manual_seed(92)
+    do = torch.randn(B, T, H, dv, generator=gen)
+    ref_leaves = [x.double().clone().requires_grad_(True) for x in (q, k, v, g, S0)]
+    o_ref, S_ref = _closed_form(*ref_leaves[:4], dk ** -0.5, ref_leaves[4])
+    (o_ref * do.double()).sum().backward()
+    ref = {n: x.grad for n, x in zip(("q", "k", "v", "g", "S0"), ref_leaves)}
+    for n in ("q", "k"):
+        ref[n] = ref[n].reshape(B, T, G, rep, dk).sum(3)
+    dev = gpu_device
+    leaves = dict(q=q[:, :, ::rep].contiguous(), k=k[:, :, ::rep].contiguous(), v=v, g=g, S0=S0)
+    leaves = {n: x.to(dev).clone().requires_grad_(True) for n, x in leaves.items()}
+    assert leaves["q"].shape == (B, T, G, dk)
+    o, S = chunk_simple_gla(q=leaves["q"], k=leaves["k"], v=leaves["v"], g=leaves["g"], initial_state=leaves["S0"],
+                            output_final_state=True)
+    (o.float() * do.to(dev)).sum().backward()
+    out_tol = hp.BF16_OUT_ABS_TOL
+    assert hp.max_abs(o.float(), o_ref) <= out_tol
+    assert hp.max_rel(S, S_ref) <= 1e-2
+    for n, x in leaves.items():
+        assert x.grad.shape == x.shape
+        err = hp.max_rel(x.grad, ref[n])
+        assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)
+    with torch.no_grad():
+        o_r, S_r = fused_recurrent_simple_gla(q=leaves["q"], k=leaves["k"], v=leaves["v"], g=leaves["g"],
+                                              initial_state=leaves["S0"], output_final_state=True)
+    assert hp.max_abs(o_r.float(), o_ref) <= out_tol
+    assert hp.max_rel(S_r, S_ref) <= (1e-2 if dtype == torch.bfloat16 else 1e-4)
+    if dk == 64:
+        # the same tokens as one packed row of three documents, no initial state: equal to the dense batch document
+        # by document
+        cu = torch.tensor([0, 130, 131, B * T], device=dev)
+        pk = {n: leaves[n].detach().reshape(1, B * T, *leaves[n].shape[2:]).clone().requires_grad_(True) for n in ("q", "k", "v", "g")}
+        o_p, _ = chunk_simple_gla(q=pk["q"], k=pk["k"], v=pk["v"], g=pk["g"], cu_seqlens=cu)
+        (o_p.float() * do.to(dev).reshape(1, B * T, H, dv)).sum().backward()
+        flat = lambda x: x.reshape(1, B * T, *x.shape[2:])
+        o_parts = []
+        for a, b_ in ((0, 130), (130, 131), (131, B * T)):
+            lv = [flat(x)[:, a:b_].double().clone().requires_grad_(True) for x in (q, k, v, g)]
+            o_d, _ = _closed_form(*lv, dk ** -0.5)
+            (o_d * flat(do)[:, a:b_].double()).sum().backward()
+            o_parts.append(o_d.detach())
+            for n, x in zip(("q", "k", "v", "g"), lv):
+                want = x.grad.reshape(1, b_ - a, G, rep, dk).sum(3) if n in ("q", "k") else x.grad
+                if b_ - a > 1:      # (the gradients of a one-token document are exact zeros or single products)
+                    err = hp.max_rel(pk[n].grad[:, a:b_], want)
+                    assert err <= hp.BF16_GRAD_NORM_TOL, (n, a, err)
+        assert hp.max_abs(o_p.float(), torch.cat(o_parts, dim=1)) <= out_tol
