@@ -108,7 +108,8 @@ typedef struct PalDims {
                            Hq of H = q,k [B,T,Hq,dk], value head h reads q/k head h / (H / Hq) (what the layers
                            obtain by repeating heads, palimpsa/layers/meta_mamba2.py:281-282, palimpsa.py:266-267,
                            without materialising the repeat); dq, dk [B,T,Hq,dk] are summed over each group.
-                           Palimpsa entry points only; the pal_gla_* entry points want 0 or H.                  */
+                           Every chunked and token-serial entry point takes it, pal_gla_* included (the
+                           MetaMamba2 layer with its precision state off: meta_mamba2.py:281-282, :319-323). */
 } PalDims;
 
 /* Forward-side tensors.  Unused optional pointers are NULL. */
