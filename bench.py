@@ -711,6 +711,9 @@ def main():
     ap.add_argument("--no-layer-slice", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the legs for configurations 0, 2 and 4")
     ap.add_argument("--no-recurrent", action="store_true", help="skip the token-serial forward/backward leg")
+    ap.add_argument("--only", choices=("c0", "c2", "c4", "recurrent", "decode"), default=None,
+                    help="profiling aid: run this one leg alone and print its object (not the contract's line), so that "
+                         "per-kernel profiler averages belong to one workload")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -733,6 +736,15 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.only is not None:
+        short = max(5, min(args.steps, 20))
+        leg = {"c0": lambda: bench_c0(torch, dev, args.steps, args.warmup, False),
+               "c2": lambda: bench_c2(torch, dev, short, min(args.warmup, 3)),
+               "c4": lambda: bench_c4(torch, dev, short, min(args.warmup, 3)),
+               "recurrent": lambda: bench_recurrent(torch, dev, max(3, min(args.steps, 10)), 2),
+               "decode": lambda: bench_decode(torch, dev, args.decode_steps)}[args.only]()
+        print(json.dumps({"only": args.only, "leg": leg}))
+        return
     res = bench_chunk(torch, dev, args.steps, args.warmup, args.gates)
     extra = {"kernels": res["kernels"], "ms_per_step_median": res["ms_per_step_median"],
              "roofline_forward": res["roofline_forward"]}
