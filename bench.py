@@ -22,8 +22,8 @@ One JSON line is printed; it also carries
   extra.c2      config 2 (packed 32768 tokens, lognormal documents, H=16 d=96, chunked forward+backward)
   extra.c4      config 4 (one sequence of 65536 tokens, H=16 d=128, chunked forward with initial and final state)
   extra.recurrent  the token-serial entry point (fused_recurrent_palimpsa) forward and forward+backward at B=8 T=2048 H=12
-                d=64 fp32 (long sequences: the backward runs the chunked kernels) and at B=256 T=64 (the token-serial
-                backward kernel, against the HBM peak as the metric asks; it is bound by serial latency)
+                d=64 fp32 (long sequences: the backward runs the chunked kernels) and at B=256 T=64 with that hand-over
+                switched off (the token-serial backward kernel, against the HBM peak as the metric asks; it is bound by serial latency)
 Every chunked leg carries two bounds: the bf16 matrix peak priced with the fixed formula of the metric and the
 fp32 vector peak priced with the vector instructions the kernel issues (counter figures from profiles/counter_table.txt).
 The decode leg of the metric is also carried as flat decode_* scalars inside the headline line's roofline object.
@@ -630,7 +630,7 @@ def bench_recurrent(torch, dev, steps, warmup):
     ms_f, med_f, k_f = timed_loop(torch, fwd, steps, warmup)
     ms_fb, med_fb, k_fb = timed_loop(torch, fwd_bwd, steps, warmup)
     # the same number of tokens as 256 sequences of 64 tokens (the longest the reference layer hands to this entry
-    # point): below 128 tokens per sequence the backward stays with the token-serial kernel
+    # point), with the hand-over to the chunked kernels switched off: the token-serial backward kernel itself
     Bs, Ts = 256, 64
     inp_s = make_inputs(torch, Bs, Ts, H, d, d, 0, torch.float32)
     leaves_s = {n: inp_s[n].to(dev).requires_grad_(True) for n in names}
@@ -641,7 +641,13 @@ def bench_recurrent(torch, dev, steps, warmup):
             x.grad = None
         fused_recurrent_palimpsa(*[leaves_s[n] for n in names]).backward(do_s)
 
-    ms_s, med_s, k_s = timed_loop(torch, fwd_bwd_short, steps, warmup)
+    from palimpsa_amd import _lib as L
+    keep = L.recurrent_bwd_chunk_min()
+    L.set_recurrent_bwd_chunk_min(None)
+    try:
+        ms_s, med_s, k_s = timed_loop(torch, fwd_bwd_short, steps, warmup)
+    finally:
+        L.set_recurrent_bwd_chunk_min(keep)
     rows = B * T * H
     bytes_f = rows * (4 * 4 * d + 4 + 4 * d)                      # q,k,v,b in, gt in, o out (fp32)
     bytes_b = rows * (4 * 5 * d + 4 + 4 * 4 * d + 4)              # q,k,v,b,do + gt in; dq,dk,dv,db + dgt out (fp32)
@@ -660,11 +666,12 @@ def bench_recurrent(torch, dev, steps, warmup):
                                          "bound by fp32 vector work and serial latency, not by HBM")},
             "forward_backward": {"tokens_per_s": B * T / (ms_fb * 1e-3), "ms_per_step": ms_fb, "ms_per_step_median": med_fb,
                                  "kernels": k_fb,
-                                 "note": "sequences of 128 tokens or more: the backward of this entry point runs the "
+                                 "note": "sequences of 64 tokens or more: the backward of this entry point runs the "
                                          "chunked backward kernels (fp32 rows: split operands, the fp32 bar) on "
                                          "tile-start states from a states-only forward pass"},
             "forward_backward_short": {
-                "workload": f"token-serial forward+backward, B={Bs} T={Ts} H={H} dk=dv={d} fp32 rows (same token count)",
+                "workload": f"token-serial forward+backward kernels, B={Bs} T={Ts} H={H} dk=dv={d} fp32 rows (same token count; "
+                            "the hand-over of the backward to the chunked kernels switched off)",
                 "tokens_per_s": Bs * Ts / (ms_s * 1e-3), "ms_per_step": ms_s, "ms_per_step_median": med_s, "kernels": k_s,
                 "roofline": add_traffic(roof("recurrent_bwd_kernel", k_s, bytes_b,
                                              "rows and dO in, gradients out; the kernel also re-reads its state "

@@ -173,8 +173,10 @@ def set_fp32_fast(on: bool) -> None:
 # Backward of the token-serial entry point: sequences of at least this many tokens on average are handed to the
 # chunked backward kernels (tile-start states from a states-only forward, then pal_chunk_bwd; fp32 rows keep the fp32
 # bar there through split operands), shorter ones run the token-serial backward kernel, which walks a sequence
-# token by token.  None = never.  Initial value from the environment variable PALIMPSA_RECURRENT_BWD_CHUNK_MIN.
-_recurrent_bwd_chunk_min = os.environ.get("PALIMPSA_RECURRENT_BWD_CHUNK_MIN", "128")
+# token by token (measured at 196608 token-heads of 64 x 64, fp32 rows: 256 sequences of 64 tokens 4.97 ms token-serial
+# against 2.9 ms chunked, 8 sequences of 2048 tokens 7.05 against 2.93; a tile costs the same however few of its 64
+# tokens are real, so below a tile per sequence the token-serial kernel wins).  None = never.  Initial value from the environment variable PALIMPSA_RECURRENT_BWD_CHUNK_MIN.
+_recurrent_bwd_chunk_min = os.environ.get("PALIMPSA_RECURRENT_BWD_CHUNK_MIN", "64")
 _recurrent_bwd_chunk_min = None if _recurrent_bwd_chunk_min in ("", "none", "None") else int(_recurrent_bwd_chunk_min)
 
 

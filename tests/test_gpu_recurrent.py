@@ -223,7 +223,7 @@ def test_bf16_rows_backward(gpu_device):
 
 @pytest.mark.parametrize("rows", ["fp32", "bf16"])
 def test_long_sequences_take_the_chunked_backward(gpu_device, rows):
-    """Sequences of 128 tokens or more on average: the backward of the token-serial entry point runs the chunked
+    """Sequences of 64 tokens or more on average: the backward of the token-serial entry point runs the chunked
     backward kernels on tile-start states from a states-only forward pass.  Dense and packed, initial state and
     uncertainty gradients included: against float64 autograd through the oracle at the bar of the row dtype, and
     against the token-serial backward kernel (the route switched off) on the same inputs."""
@@ -248,11 +248,12 @@ def test_long_sequences_take_the_chunked_backward(gpu_device, rows):
     ran = L.profile_read()
     L.profile_enable(False)
     assert "chunk_bwd_local_kernel" in ran and "recurrent_bwd_kernel" not in ran, sorted(ran)
+    keep = L.recurrent_bwd_chunk_min()
     try:
         L.set_recurrent_bwd_chunk_min(None)
         serial = _rec_grads(inp, gpu_device, do, dovar, mu0=mu0, I0=I0, cu=cu)
     finally:
-        L.set_recurrent_bwd_chunk_min(128)
+        L.set_recurrent_bwd_chunk_min(keep)
     names = ["q", "k", "v", "b", "gt", "g", "Ip", "mu0", "I0"]
     if rows == "fp32":
         for n in names:
@@ -267,9 +268,9 @@ def test_long_sequences_take_the_chunked_backward(gpu_device, rows):
                 err = hp.max_rel(got[n], ref[n])
             assert err <= hp.BF16_GRAD_NORM_TOL, (n, err)
     # a dense batch of short sequences stays with the token-serial kernel
-    short = po.make_inputs(2, 60, H, dk, dv, seed=73)
+    short = po.make_inputs(2, 50, H, dk, dv, seed=73)
     L.profile_enable(True)
-    _rec_grads(short, gpu_device, torch.randn(2, 60, H, dv, generator=gen))
+    _rec_grads(short, gpu_device, torch.randn(2, 50, H, dv, generator=gen))
     torch.cuda.synchronize()
     ran = L.profile_read()
     L.profile_enable(False)
