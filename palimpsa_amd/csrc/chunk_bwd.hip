@@ -56,9 +56,10 @@ struct BwdArgs {
 };
 
 constexpr int kVS2 = 68;
-constexpr int kDG2 = 16;
 // local pass: second producer one value row behind the first (see the kernel)
-__host__ __device__ constexpr bool local_lag(int NB, bool prec) { return !prec && NB != 2; }
+__host__ __device__ constexpr bool local_lag(int NB, bool prec) { return !prec; }
+// value rows staged at a time: 8 with two column blocks per workgroup, so that two such workgroups fit a compute unit's LDS
+__host__ __device__ constexpr int local_dg(int NB, bool prec) { return (!prec && NB == 2) ? 8 : 16; }
 
 __device__ __forceinline__ constexpr int lidx2(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
 __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2 * sb + p : 4 + (sb - 2); }
@@ -92,12 +93,13 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
   constexpr int NST = HAS_VAR ? 4 : 3;  // staged tensors: v, b, do, (dovar)
-  constexpr int STG = kDG2 * kVS2;
+  constexpr int DG = local_dg(NB, PREC);   // value rows per staging group
+  constexpr int STG = DG * kVS2;
   float* sC = smem;                      // [64] running log2 decay
   float* sF = sC + kC;                   // [64] 2^c
-  float* sSt = sF + kC;                  // [2][NST][16][kVS2]
-  float* sPv = sSt + 2 * NST * STG;      // [NB][16][64] per-wave partial dv
-  float* sPb = sPv + NB * kDG2 * kC;     // [NB][16][64] per-wave partial db
+  float* sSt = sF + kC;                  // [2][NST][DG][kVS2]
+  float* sPv = sSt + 2 * NST * STG;      // [NB][DG][64] per-wave partial dv
+  float* sPb = sPv + NB * DG * kC;       // [NB][DG][64] per-wave partial db
   // LAG: the second producer runs one value row behind the first (it takes what the first one leaves for it: the
   // operands of tokens 0..31, or, with the tile cut in two halves (SUB below), the state after token 31); the consumers
   // follow two rows behind.  The first producer's half of a slot is then alive for three rows, the second one's for two:
@@ -106,10 +108,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   // Not with two column blocks per workgroup (two such workgroups share a compute unit's LDS) nor with split operands.
   constexpr bool LAG = local_lag(NB, PREC);
   constexpr int LAGC = LAG ? 2 : 1;        // rows the consumers run behind the first producer
-  float* sMJ = sPb + NB * kDG2 * kC;     // [NB][2 slots][2][16] (LAG: [NB][3 slots][6][16]) states of the rows in flight
+  float* sMJ = sPb + NB * DG * kC;     // [NB][2 slots][2][16] (LAG: [NB][3 slots][6][16]) states of the rows in flight
   constexpr int OPN = PREC ? 16 : 8;       // operands per slot (PREC: the lo halves follow the 8 hi halves)
   bf16x8* sX = (bf16x8*)(sMJ + NB * (LAG ? 288 : 64));   // [NB][2 slots][OPN operands][64 lanes] (LAG: see above)
-  // [NB][16 rows][4][M 0..3, J 0..3] first column of dM^loc, dJ^loc of a group of value rows (the carry to the previous tile)
+  // [NB][DG rows][4][M 0..3, J 0..3] first column of dM^loc, dJ^loc of a group of value rows (the carry to the previous tile)
   float* sCar = (float*)(sX + NB * (LAG ? 20 : 2 * OPN) * 64);
   // [NB][64] d log f partials of the consumer waves, then [2 NB] sums of dJloc: written after the last row of a pass,
   // when the operand slots are dead, so they share their memory
@@ -138,14 +140,14 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   }
   // Global addresses are kept as a wave-uniform base plus a 32-bit lane offset, so that the
   // loop-invariant parts live in scalar registers.
-  // Staging of 16 value rows x 64 tokens (v, b, do, dovar) and the dv/db flush: threads 0..255,
+  // Staging of DG value rows x 64 tokens (v, b, do, dovar) and the dv/db flush: threads 0..16 DG - 1,
   // thread = (token s, quad of rows q4).
   const int64_t row0 = ((int64_t)t0 * H + h) * dv;
   const TIn* vp = (const TIn*)a.v + row0;
   const TIn* bp = (const TIn*)a.b + row0;
   const TIn* dop = (const TIn*)A.d_o + row0;
-  const int st_s = tid >> 2, st_q = tid & 3;
-  const bool st_on = tid < kC * kDG2 / 4;
+  const int st_s = tid / (DG / 4), st_q = tid % (DG / 4);
+  const bool st_on = tid < kC * DG / 4;
   const unsigned st_off = (unsigned)(st_s * H * dv + 4 * st_q);
   auto stage = [&](int dg) {
     if (!st_on) return;
@@ -154,14 +156,14 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     unsigned off = st_off;
     asm volatile("" : "+v"(off));
     if (st_s < clen) {
-      load_vec<4>(vp + dg * kDG2 + off, st[0]);
-      load_vec<4>(bp + dg * kDG2 + off, st[1]);
-      load_vec<4>(dop + dg * kDG2 + off, st[2]);
+      load_vec<4>(vp + dg * DG + off, st[0]);
+      load_vec<4>(bp + dg * DG + off, st[1]);
+      load_vec<4>(dop + dg * DG + off, st[2]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) st[2][e] *= scale;
       if (HAS_VAR) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) st[NST - 1][e] = scale * load_rt(A.d_o_var, row0 + dg * kDG2 + off + e, a.var_bf16);
+        for (int e = 0; e < 4; ++e) st[NST - 1][e] = scale * load_rt(A.d_o_var, row0 + dg * DG + off + e, a.var_bf16);
       }
     } else {
 #pragma unroll
@@ -173,26 +175,26 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
     for (int x = 0; x < NST; ++x)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * kDG2 + 4 * st_q + e) * kVS2 + st_s] = st[x][e];
+      for (int e = 0; e < 4; ++e) sSt[((buf * NST + x) * DG + 4 * st_q + e) * kVS2 + st_s] = st[x][e];
   };
   const int64_t rs = qk_stride(a);      // token stride of q, k
   const int64_t rso = (int64_t)H * dk;  // token stride of dq, dk (one row per value head)
   const int64_t tile_off = (((int64_t)cidx * H + h) * dv) * dk;
-  const int n_groups = dv / kDG2;
+  const int n_groups = dv / DG;
   int pass = 0, nb = nbl, n_act = NB;   // set per pass: global column block of this wave, active blocks
 
-  // end of one iteration, identical for every role: stage the next group of 16 value rows mid-group
+  // end of one iteration, identical for every role: stage the next group of DG value rows mid-group
   // into the other buffer, synchronise, and flush dv/db once the consumers have finished a group
   auto iter_tail = [&](int it) {
-    if ((it & 15) == 8 && (it >> 4) + 1 < n_groups) stage((it >> 4) + 1);
+    if ((it & (DG - 1)) == DG / 2 && it / DG + 1 < n_groups) stage(it / DG + 1);
     __syncthreads();
-    if (it >= LAGC && ((it - LAGC) & 15) == 15) {
-      const int dg = (it - LAGC) >> 4;
+    if (it >= LAGC && ((it - LAGC) & (DG - 1)) == DG - 1) {
+      const int dg = (it - LAGC) / DG;
       if (st_on && st_s < clen) {
         unsigned off = st_off;
         asm volatile("" : "+v"(off));
-        TIn* dvo = (TIn*)A.dv + row0 + dg * kDG2 + off;
-        TIn* dbo = (TIn*)A.db + row0 + dg * kDG2 + off;
+        TIn* dvo = (TIn*)A.dv + row0 + dg * DG + off;
+        TIn* dbo = (TIn*)A.db + row0 + dg * DG + off;
         float sv[4] = {0.f, 0.f, 0.f, 0.f}, sb_[4] = {0.f, 0.f, 0.f, 0.f};
         if (MULTI && pass > 0) {   // later passes add to what the earlier column groups left
           load_vec<4>(dvo, sv);
@@ -203,8 +205,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
           for (int w = 0; w < NB; ++w) {
             if (!MULTI || w < n_act) {
-              sv[e] += sPv[(w * kDG2 + 4 * st_q + e) * kC + st_s];
-              sb_[e] += sPb[(w * kDG2 + 4 * st_q + e) * kC + st_s];
+              sv[e] += sPv[(w * DG + 4 * st_q + e) * kC + st_s];
+              sb_[e] += sPb[(w * DG + 4 * st_q + e) * kC + st_s];
             }
           }
         }
@@ -212,13 +214,13 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         store_vec<4>(dbo, sb_);
       }
       // carry handed to the previous tile, f_first * dM^loc at the first token: thread = (column block, row, quad of columns)
-      if (tid < n_act * 64) {
-        const int w = tid >> 6, row = (tid >> 2) & 15, q4 = tid & 3;
+      if (tid < n_act * DG * 4) {
+        const int w = tid / (DG * 4), row = (tid >> 2) & (DG - 1), q4 = tid & 3;
         const float f_first = fast_exp2(sC[0]);
         const f32x4 cm = *(const f32x4*)&sCar[tid * 8], cj = *(const f32x4*)&sCar[tid * 8 + 4];
         const float rm[4] = {f_first * cm[0], f_first * cm[1], f_first * cm[2], f_first * cm[3]};
         const float rj[4] = {f_first * cj[0], f_first * cj[1], f_first * cj[2], f_first * cj[3]};
-        const int64_t co = tile_off + (int64_t)(dg * kDG2 + row) * dk + 16 * (pass * NB + w) + 4 * q4;
+        const int64_t co = tile_off + (int64_t)(dg * DG + row) * dk + 16 * (pass * NB + w) + 4 * q4;
         store_vec<4>((TIn*)A.wDM + co, rm);
         store_vec<4>((TIn*)A.wDJ + co, rj);
       }
@@ -298,7 +300,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     int b3 = 0;                                 // LAG: d mod 3, the first producer's slot of the row
     for (int it = 0; it < dv + LAGC; ++it) {
       if (it >= LAGP && it - LAGP < dv) {
-        const int d = it - LAGP, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const int d = it - LAGP, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
@@ -520,14 +522,14 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     // the carries between tiles are kept in the dtype of the rows: bf16 rows feed them to the matrix cores in bf16
     // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers.  The consumer of the
     // first column token parks them per group of value rows; the flush of the group scales and stores them.
-    float* car = sCar + ((nbl * kDG2) * 4 + g) * 8;
+    float* car = sCar + ((nbl * DG) * 4 + g) * 8;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
-    float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
+    float* pw = ((g < 2) ? sPv : sPb) + nbl * DG * kC + 16 * (2 * HF + (g & 1)) + i;
 
     int b3 = 0;   // LAG: d mod 3
     for (int it = 0; it < dv + LAGC; ++it) {
       if (it >= LAGC) {
-        const int d = it - LAGC, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const int d = it - LAGC, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
@@ -712,7 +714,7 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     int b3 = 0;                                 // d mod 3: the row's slot of sMJ and of the first producer's operands
     for (int it = 0; it < dv + LAGC; ++it) {
       if (it >= HF && it - HF < dv) {
-        const int d = it - HF, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const int d = it - HF, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
@@ -855,13 +857,13 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         gate[sl] = 0.f;
       }
     }
-    float* car = sCar + ((nbl * kDG2) * 4 + g) * 8;
+    float* car = sCar + ((nbl * DG) * 4 + g) * 8;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
-    float* pw = ((g < 2) ? sPv : sPb) + nbl * kDG2 * kC + 16 * (2 * HF + (g & 1)) + i;
+    float* pw = ((g < 2) ? sPv : sPb) + nbl * DG * kC + 16 * (2 * HF + (g & 1)) + i;
     int b3 = 0;   // d mod 3
     for (int it = 0; it < dv + LAGC; ++it) {
       if (it >= LAGC) {
-        const int d = it - LAGC, dd = d & (kDG2 - 1), buf = (d / kDG2) & 1;
+        const int d = it - LAGC, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
         const bf16x8* ph = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;   // the own half's operands
@@ -1511,8 +1513,9 @@ struct BwdPlan {
 
 static size_t local_lds_bytes(int NB, bool var, bool prec) {
   const bool lag = local_lag(NB, prec);
-  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * kDG2 * kVS2 + 2 * NB * kDG2 * kC +
-                          NB * (lag ? 288 : 64) + NB * kDG2 * 32) +
+  const int DG = local_dg(NB, prec);
+  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * DG * kVS2 + 2 * NB * DG * kC +
+                          NB * (lag ? 288 : 64) + NB * DG * 32) +
          (size_t)NB * (lag ? 20 : 2 * (prec ? 16 : 8)) * 64 * 16;
 }
 
