@@ -56,13 +56,11 @@ struct BwdArgs {
 };
 
 constexpr int kVS2 = 68;
-// local pass: second producer one value row behind the first (see the kernel)
-__host__ __device__ constexpr bool local_lag(int NB, bool prec) { return !prec; }
+// local pass: rows the consumers run behind the first producer (the second producer runs one row behind it)
+constexpr int kLagC = 2;
 // value rows staged at a time: 8 with two column blocks per workgroup, so that two such workgroups fit a compute unit's LDS
 __host__ __device__ constexpr int local_dg(int NB, bool prec) { return (!prec && NB == 2) ? 8 : 16; }
 
-__device__ __forceinline__ constexpr int lidx2(int tb, int ks) { return tb < 2 ? tb : 2 + 2 * (tb - 2) + ks; }
-__device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2 * sb + p : 4 + (sb - 2); }
 
 // ------------------------------------------------- local pass, four wave roles
 // One workgroup per (tile, head).  For every value row d the tile recomputes M_t, I_t for its 64 tokens
@@ -71,19 +69,18 @@ __device__ __forceinline__ constexpr int ridx(int sb, int p) { return sb < 2 ? 2
 // Organised for four waves per SIMD: one wave issues a VALU instruction every 5-9 cycles at best while
 // the SIMD can start one every 2-3, so the work on a block of 16 key columns is cut into four roles
 // small enough for 128 registers each.  A workgroup has 4*NB waves; wave = role*NB + (column block).
-//   roles 0/1 ("producers", token blocks 0-1 / 2-3): recompute the states of one value row for 16 key
-//     columns, form dMloc/dJloc and dq, and leave packed bf16 operands in an LDS slot:
-//     role 0 writes P^M_0, P^J_0, X^M_0, X^J_0 (tokens 0..31), role 1 the halves for tokens 32..63;
-//   roles 2/3 ("consumers", token blocks 0-1 / 2-3 of the column token s): pick the slot up one iteration
-//     later (two with the lagged second producer, see LAG below) and do the reverse contraction, the
-//     strictly-lower product and the dv/db/dk/gate epilogue.
+//   roles 0/1 ("producers", tokens 0..31 / 32..63): recompute the states of one value row for 16 key
+//     columns, form dMloc/dJloc and dq, and leave packed bf16 operands P^M, P^J (local gradients) and X^M, X^J
+//     (rank-one updates) of their half of the tile in an LDS slot;
+//   roles 2/3 ("consumers", column tokens s in 0..31 / 32..63): pick their half's slot up two iterations after the
+//     first producer wrote its own and do the reverse contraction, the strictly-lower product and the
+//     dv/db/dk/gate epilogue.
 // Every role has its own loop (its own register allocation) with the same sequence of barriers.
-// The tile-start state (M_0, J_0) of a value row reaches the products through the operands: see FOLD at the
-// producers and the virtual token at the consumers.
+// The tile is worked as two halves of 32 tokens coupled through LDS (see the producers).
 // NB <= 4 column blocks are in flight at a time (16 waves); a wider head dim takes several passes over
 // the tile, the later ones adding their dv/db/gate contributions to those of the earlier ones.
 // PREC (fp32 rows): every operand is carried as two bf16 halves and every product takes three matrix instructions
-// (split_bf16 / mfma16_split); the LDS slots hold 16 operands instead of 8 and a wave may use 256 registers
+// (split_bf16 / mfma16_split); the LDS slots hold twice the operands and a wave may use 256 registers
 // (two waves per SIMD), so at most 2 column blocks are in flight.
 // Three column blocks (dk = 48) are 12 waves, three per SIMD and one workgroup per compute unit (its LDS): that
 // instance may use 168 registers.
@@ -96,23 +93,21 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   constexpr int DG = local_dg(NB, PREC);   // value rows per staging group
   constexpr int STG = DG * kVS2;
   float* sC = smem;                      // [64] running log2 decay
-  float* sF = sC + kC;                   // [64] 2^c
+  float* sF = sC + kC;                   // [64] decay from before the half of the tile: 2^c_t (t < 32), 2^(c_t - c_31)
   float* sSt = sF + kC;                  // [2][NST][DG][kVS2]
   float* sPv = sSt + 2 * NST * STG;      // [NB][DG][64] per-wave partial dv
   float* sPb = sPv + NB * DG * kC;       // [NB][DG][64] per-wave partial db
-  // LAG: the second producer runs one value row behind the first (it takes what the first one leaves for it: the
-  // operands of tokens 0..31, or, with the tile cut in two halves (SUB below), the state after token 31); the consumers
-  // follow two rows behind.  The first producer's half of a slot is then alive for three rows, the second one's for two:
-  //   sX  [NB][3 x {P^M_0, P^J_0, X^M_0, X^J_0} | 2 x {P^M_1, P^J_1, X^M_1, X^J_1}][64 lanes],
-  //   sMJ [NB][3 slots][M_0, J_0, M_31, J_31, what flows back over token 31 (M, J)][16]   (see SUB below).
-  // Not with two column blocks per workgroup (two such workgroups share a compute unit's LDS) nor with split operands.
-  constexpr bool LAG = local_lag(NB, PREC);
-  constexpr int LAGC = LAG ? 2 : 1;        // rows the consumers run behind the first producer
-  float* sMJ = sPb + NB * DG * kC;     // [NB][2 slots][2][16] (LAG: [NB][3 slots][6][16]) states of the rows in flight
-  constexpr int OPN = PREC ? 16 : 8;       // operands per slot (PREC: the lo halves follow the 8 hi halves)
-  bf16x8* sX = (bf16x8*)(sMJ + NB * (LAG ? 288 : 64));   // [NB][2 slots][OPN operands][64 lanes] (LAG: see above)
+  // The second producer runs one value row behind the first (it takes the state after token 31 from it), the
+  // consumers follow two rows behind.  The first producer's half of a slot is then alive for three rows, the second
+  // one's for two:
+  //   sX  [NB][3 x {P^M_0, P^J_0, X^M_0, X^J_0} | 2 x {P^M_1, P^J_1, X^M_1, X^J_1}][64 lanes]
+  //       (PREC: each group of four is followed by its four lo halves),
+  //   sMJ [NB][3 slots][M_0, J_0, M_31, J_31, what flows back over token 31 (M, J)][16]   (see the producers).
+  float* sMJ = sPb + NB * DG * kC;
+  constexpr int XS = PREC ? 2 : 1;
+  bf16x8* sX = (bf16x8*)(sMJ + NB * 288);
   // [NB][DG rows][4][M 0..3, J 0..3] first column of dM^loc, dJ^loc of a group of value rows (the carry to the previous tile)
-  float* sCar = (float*)(sX + NB * (LAG ? 20 : 2 * OPN) * 64);
+  float* sCar = (float*)(sX + NB * 20 * XS * 64);
   // [NB][64] d log f partials of the consumer waves, then [2 NB] sums of dJloc: written after the last row of a pass,
   // when the operand slots are dead, so they share their memory
   float* sRed = (float*)sX;
@@ -135,7 +130,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
     const float c = wave_inclusive_scan(-gt * gh, lane);
     sC[lane] = c;
-    sF[lane] = fast_exp2(c);
+    const float c31 = __shfl(c, 31);   // every lane takes part: not inside the conditional
+    sF[lane] = fast_exp2(lane >= 32 ? c - c31 : c);
     if (lane == 63) A.wFtot[(int64_t)cidx * H + h] = c;
   }
   // Global addresses are kept as a wave-uniform base plus a 32-bit lane offset, so that the
@@ -188,8 +184,8 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
   auto iter_tail = [&](int it) {
     if ((it & (DG - 1)) == DG / 2 && it / DG + 1 < n_groups) stage(it / DG + 1);
     __syncthreads();
-    if (it >= LAGC && ((it - LAGC) & (DG - 1)) == DG - 1) {
-      const int dg = (it - LAGC) / DG;
+    if (it >= kLagC && ((it - kLagC) & (DG - 1)) == DG - 1) {
+      const int dg = (it - kLagC) / DG;
       if (st_on && st_s < clen) {
         unsigned off = st_off;
         asm volatile("" : "+v"(off));
@@ -228,439 +224,37 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     }
   };
 
-  // ------------------------------------------------------------------ producers
-  // FOLD (bf16 operands, no initial state): the tile-start state rides in the operand of the tile's first token,
-  // X'_0 = X_0 + f_0 (M_0, J_0), since F_t = L[t,0] f_0: the prefix product then yields M_t, J_t without the
-  // two multiply-adds per state entry.  The state is rounded to bf16 there like every other operand; a J_0 below
-  // zero (an initial state with I_0 < Ip) would cancel against Ip, so launches with an initial state keep the fp32 form.
-  auto producer = [&](auto hfc, auto foldc) {
-    constexpr int HF = decltype(hfc)::value;   // token blocks 2HF, 2HF+1 (index tl)
-    constexpr bool FOLD = decltype(foldc)::value;
-    bf16x8 Lop[HF ? 4 : 2];   // forward operand L[t,s], s <= t: HF=0 [tl], HF=1 [2tl+ks]
-    bf16x8 Lol[PREC ? (HF ? 4 : 2) : 1];   // PREC: its lo halves
-    float kk[HF ? 16 : 8];    // k in operand layout (n = i, s = 8g+j+32ks)
-    // its square, kept where the registers are there for it (measured: 5 % of the kernel at dk = 64; with several
-    // passes over the tile the loop spills and is 1-2 % slower, there the square is formed per value row)
-    constexpr bool KK2 = !MULTI && NB != 3;
-    float kk2[KK2 ? (HF ? 16 : 8) : 1];
-    float qq[8];              // q in result layout (t = 16tb+4g+r, n = i)
-    float dq[8];
-    float sigacc = 0.f;
-    {
-      const TIn* kp = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
-      const TIn* qp = (const TIn*)a.q + qk_row(a, t0, h) + 16 * nb;
-      float ct[2];
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl) ct[tl] = sC[16 * (2 * HF + tl) + i];
-#pragma unroll
-      for (int ks = 0; ks <= HF; ++ks) {
-        float cs[8];
-        *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
-        *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int s = 8 * g + j + 32 * ks;
-          const bool ok = s < clen;
-          const float kv = to_f32((kp + (int64_t)(ok ? s : 0) * rs)[i]);
-          kk[ks * 8 + j] = ok ? kv : 0.f;
-          if constexpr (KK2) kk2[ks * 8 + j] = kk[ks * 8 + j] * kk[ks * 8 + j];
-#pragma unroll
-          for (int tl = 0; tl < 2; ++tl) {
-            const int t = 16 * (2 * HF + tl) + i;
-            const float lv = (s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f;
-            const bf16_t lh = (bf16_t)lv;
-            Lop[HF ? 2 * tl + ks : tl][j] = lh;
-            if constexpr (PREC) Lol[HF ? 2 * tl + ks : tl][j] = (bf16_t)(lv - (float)lh);
-          }
-        }
-      }
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int t = 16 * (2 * HF + tl) + 4 * g + r;
-          const bool ok = t < clen;
-          const float qv = to_f32((qp + (int64_t)(ok ? t : 0) * rs)[i]);
-          qq[tl * 4 + r] = ok ? qv : 0.f;
-          dq[tl * 4 + r] = 0.f;
-        }
-    }
-    // tile-start state of the next value row (entry of the own key column n = i), fetched one iteration ahead
-    const float* cmu = a.chunk_mu + tile_off + 16 * nb;
-    const float* cI = a.chunk_I + tile_off + 16 * nb;
-    float mu_n = cmu[i], I_n = cI[i];
-    const float f0m = (FOLD && g == 0) ? fast_exp2(sC[0]) : 0.f;   // lanes that hold token 0 of the operands
-
-    // The producer of token blocks 2-3 has the longest iteration (twice the matrix instructions of the other one):
-    // the other three waves of its SIMD finish a row earlier and would leave it to issue alone at half rate, so it
-    // gets the issue slots first (measured: 3.5 % of the kernel; the same or an intermediate priority for the other
-    // producer, or none at all, are all slower).
-    if (HF) __builtin_amdgcn_s_setprio(3);
-    constexpr int LAGP = (LAG && HF) ? 1 : 0;   // rows this producer runs behind the first one
-    int b3 = 0;                                 // LAG: d mod 3, the first producer's slot of the row
-    for (int it = 0; it < dv + LAGC; ++it) {
-      if (it >= LAGP && it - LAGP < dv) {
-        const int d = it - LAGP, dd = d & (DG - 1), buf = (d / DG) & 1;
-        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
-        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
-        const float* sDo = sSt + (buf * NST + 2) * STG + dd * kVS2;
-        const float* sDov = sSt + (buf * NST + NST - 1) * STG + dd * kVS2;
-        const float mu0 = mu_n, I0 = I_n;
-        {
-          const int64_t dn = (int64_t)min(d + 1, dv - 1) * dk;
-          mu_n = (cmu + dn)[i];
-          I_n = (cI + dn)[i];
-        }
-        const float M0 = mu0 * I0, J0 = I0 - Ip;
-        const float fM = f0m * M0, fJ = f0m * J0;
-        if (!HF && g == 0) {
-          float* mj = sMJ + (LAG ? nbl * 4 + (d & 3) : nbl * 2 + (d & 1)) * 32;
-          mj[i] = M0;
-          mj[16 + i] = J0;
-        }
-        bf16x8 XM[HF + 1], XJ[HF + 1];
-        bf16x8 XMl[PREC ? HF + 1 : 1], XJl[PREC ? HF + 1 : 1];
-#pragma unroll
-        for (int ks = 0; ks <= HF; ++ks) {
-          if (LAG && HF && ks == 0) {   // tokens 0..31: as the first producer left them a row ago
-            const bf16x8* p0 = sX + (nbl * 20 + 4 * b3) * 64 + lane;
-            XM[0] = p0[2 * 64];
-            XJ[0] = p0[3 * 64];
-            continue;
-          }
-          const f32x4 v0 = *(const f32x4*)&sV[8 * g + 32 * ks];
-          const f32x4 v1 = *(const f32x4*)&sV[8 * g + 32 * ks + 4];
-          const f32x4 b0 = *(const f32x4*)&sB[8 * g + 32 * ks];
-          const f32x4 b1 = *(const f32x4*)&sB[8 * g + 32 * ks + 4];
-          if constexpr (PREC) {
-            float xm[8], xj[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float vv = j < 4 ? v0[j & 3] : v1[j & 3], bb = j < 4 ? b0[j & 3] : b1[j & 3];
-              const float kx = kk[ks * 8 + j];
-              xm[j] = kx * vv;
-              xj[j] = (kx * bb) * kx;
-            }
-            split_bf16(xm, XM[ks], XMl[ks]);
-            split_bf16(xj, XJ[ks], XJl[ks]);
-          } else {
-#pragma unroll
-          for (int j = 0; j < 8; j += 2) {
-            const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
-            const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
-            const float ka = kk[ks * 8 + j], kb = kk[ks * 8 + j + 1];
-            const bool tok0 = FOLD && ks == 0 && j == 0;
-            const bf16x2 pm = pack2(tok0 ? fmaf(ka, va, fM) : ka * va, kb * vb);
-            const float kab = KK2 ? kk2[ks * 8 + j] : ka * ba, kbb = KK2 ? kk2[ks * 8 + j + 1] : kb * bb;
-            const float ja = KK2 ? ba : ka, jb = KK2 ? bb : kb;
-            const bf16x2 pj = pack2(tok0 ? fmaf(kab, ja, fJ) : kab * ja, kbb * jb);
-            XM[ks][j] = pm[0]; XM[ks][j + 1] = pm[1];
-            XJ[ks][j] = pj[0]; XJ[ks][j + 1] = pj[1];
-          }
-          }
-        }
-        bf16x8 PM, PJ;
-        float pmf[PREC ? 8 : 1], pjf[PREC ? 8 : 1];   // PREC: the local gradients in fp32 until they are split
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl) {
-          const int tb = 2 * HF + tl;
-          f32x4 accM = {0.f, 0.f, 0.f, 0.f};
-          f32x4 accI = {Ip, Ip, Ip, Ip};
-          if constexpr (PREC) {
-            accM = mfma16_split(Lop[HF ? 2 * tl : tl], Lol[HF ? 2 * tl : tl], XM[0], XMl[0], accM);
-            accI = mfma16_split(Lop[HF ? 2 * tl : tl], Lol[HF ? 2 * tl : tl], XJ[0], XJl[0], accI);
-            if (HF) {
-              accM = mfma16_split(Lop[2 * tl + HF], Lol[2 * tl + HF], XM[HF], XMl[HF], accM);
-              accI = mfma16_split(Lop[2 * tl + HF], Lol[2 * tl + HF], XJ[HF], XJl[HF], accI);
-            }
-          } else {
-          accM = mfma16(Lop[HF ? 2 * tl : tl], XM[0], accM);
-          accI = mfma16(Lop[HF ? 2 * tl : tl], XJ[0], accI);
-          if (HF) {
-            accM = mfma16(Lop[2 * tl + HF], XM[HF], accM);
-            accI = mfma16(Lop[2 * tl + HF], XJ[HF], accI);
-          }
-          }
-          f32x4 Fv = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (!FOLD) Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
-          const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
-          f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
-          if (HAS_VAR) dvv = *(const f32x4*)&sDov[16 * tb + 4 * g];
-          float dMl[4], dJl[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float Mf = FOLD ? accM[r] : fmaf(Fv[r], M0, accM[r]);
-            const float If = FOLD ? accI[r] : fmaf(Fv[r], J0, accI[r]);
-            const float rI = fast_rcp(If);
-            const float mu = Mf * rI;
-            const float q = qq[tl * 4 + r];
-            dMl[r] = (dov[r] * q) * rI;
-            dJl[r] = -(dMl[r] * mu);
-            dq[tl * 4 + r] = fmaf(mu, dov[r], dq[tl * 4 + r]);
-            if (HAS_VAR) {
-              const float wq = dvv[r] * q;          // scale*dovar*q
-              const float w = wq * q * rI;          // scale*dovar*q^2/I
-              dJl[r] = fmaf(-w, rI, dJl[r]);
-              dq[tl * 4 + r] = fmaf(2.f * wq, rI, dq[tl * 4 + r]);
-            }
-            if constexpr (PREC) sigacc += dJl[r];
-          }
-          const int o4 = tl * 4;
-          if constexpr (PREC) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) { pmf[o4 + r] = dMl[r]; pjf[o4 + r] = dJl[r]; }
-          } else {
-          const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
-          const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
-          // the sum of dJloc (for dIp) from the packed pairs: one instruction per two entries
-          const bf16x2 one2 = {(bf16_t)1.f, (bf16_t)1.f};
-          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j0, one2, sigacc, false);
-          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j1, one2, sigacc, false);
-          PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
-          PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
-          }
-        }
-        if constexpr (LAG) {
-          bf16x8* mine = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;
-          mine[0] = PM; mine[64] = PJ; mine[2 * 64] = XM[HF]; mine[3 * 64] = XJ[HF];
-          b3 = (b3 == 2) ? 0 : b3 + 1;
-        } else {
-        bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
-        if constexpr (PREC) {
-          bf16x8 PMl, PJl;
-          split_bf16(pmf, PM, PMl);
-          split_bf16(pjf, PJ, PJl);
-          slot[(8 + 0 + HF) * 64] = PMl; slot[(8 + 2 + HF) * 64] = PJl;
-          slot[(8 + 4 + HF) * 64] = XMl[HF]; slot[(8 + 6 + HF) * 64] = XJl[HF];
-        }
-        slot[(0 + HF) * 64] = PM; slot[(2 + HF) * 64] = PJ;
-        slot[(4 + HF) * 64] = XM[HF]; slot[(6 + HF) * 64] = XJ[HF];
-        }
-      }
-      iter_tail(it);
-    }
-
-    if (HF) __builtin_amdgcn_s_setprio(0);
-    TIn* dqp = (TIn*)A.dq + ((int64_t)t0 * H + h) * dk + 16 * nb;
-#pragma unroll
-    for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = 16 * (2 * HF + tl) + 4 * g + r;
-        if (t < clen) (dqp + (int64_t)t * rso)[i] = from_f32<TIn>(dq[tl * 4 + r]);
-      }
-    const float x = wave_sum(sigacc);
-    if (lane == 0) sRed[NB * kC + HF * NB + nbl] = x;
-  };
-
-  // ------------------------------------------------------------------ consumers
-  auto consumer = [&](auto hfc, auto foldc) {
-    constexpr int HF = decltype(hfc)::value;   // column-token blocks 2HF, 2HF+1 (index sl)
-    constexpr bool FOLD = decltype(foldc)::value;   // the operands of token 0 carry f_0 (M_0, J_0), see the producers
-    bf16x8 Lop[6];    // reverse operand, HF=0 [2sl+p], HF=1 [sl] (p=1); strictly-lower operand, HF=0 [4+sl], HF=1 [2+2sl+ks]
-    bf16x8 Lol[PREC ? 6 : 1];   // PREC: its lo halves
-    float kr[8];      // k in result layout (s = 16sb+i, n = 4g+r)
-    float dkM[8], dkJ[8];
-    float gate[2], Fs[2];
-    {
-      const TIn* kp4 = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
-      float ct[2];
-#pragma unroll
-      for (int sl = 0; sl < 2; ++sl) ct[sl] = sC[16 * (2 * HF + sl) + i];
-      // strictly-lower operand: column token t = 16sb + i, contraction token s = 8g + j + 32ks < t
-#pragma unroll
-      for (int ks = 0; ks <= HF; ++ks) {
-        float cs[8];
-        *(f32x4*)&cs[0] = *(const f32x4*)&sC[8 * g + 32 * ks];
-        *(f32x4*)&cs[4] = *(const f32x4*)&sC[8 * g + 32 * ks + 4];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int s = 8 * g + j + 32 * ks;
-#pragma unroll
-          for (int sl = 0; sl < 2; ++sl) {
-            const int t = 16 * (2 * HF + sl) + i;
-            float lv = (s < t) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
-            // the last contraction slot of the wave's range (token 31 / 63) is never below a column token of the
-            // wave: it carries the tile-start state instead, with the decay F_t from the start of the tile
-            // (FOLD: the product has the state already, through token 0, for every column token but token 0 itself)
-            if (!PREC && ks == HF && g == 3 && j == 7) lv = (FOLD && t != 0) ? 0.f : fast_exp2(ct[sl]);
-            const bf16_t lh = (bf16_t)lv;
-            Lop[HF ? 2 + 2 * sl + ks : 4 + sl][j] = lh;
-            if constexpr (PREC) Lol[HF ? 2 + 2 * sl + ks : 4 + sl][j] = (bf16_t)(lv - (float)lh);
-          }
-        }
-      }
-      // reverse operand: column s = 16sb + i, contraction index (g,j) <-> token t = 16(2p + j/4) + 4g + j%4 >= s
-#pragma unroll
-      for (int p = HF; p < 2; ++p) {
-        float ctt[8];
-        *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * p + 4 * g];
-        *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * p + 16 + 4 * g];
-#pragma unroll
-        for (int sl = 0; sl < 2; ++sl) {
-          const int s = 16 * (2 * HF + sl) + i;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int t = 16 * (2 * p + (j >> 2)) + 4 * g + (j & 3);
-            const float lv = (t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f;
-            const bf16_t lh = (bf16_t)lv;
-            Lop[HF ? sl : 2 * sl + p][j] = lh;
-            if constexpr (PREC) Lol[HF ? sl : 2 * sl + p][j] = (bf16_t)(lv - (float)lh);
-          }
-        }
-      }
-#pragma unroll
-      for (int sl = 0; sl < 2; ++sl) {
-        const int s = 16 * (2 * HF + sl) + i;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) { kr[sl * 4 + r] = 0.f; dkM[sl * 4 + r] = 0.f; dkJ[sl * 4 + r] = 0.f; }
-        if (s < clen) load_vec<4>(kp4 + (int64_t)s * rs + 4 * g, &kr[sl * 4]);
-        gate[sl] = 0.f;
-        Fs[sl] = sF[16 * (2 * HF + sl) + i];
-      }
-    }
-    // the carries between tiles are kept in the dtype of the rows: bf16 rows feed them to the matrix cores in bf16
-    // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers.  The consumer of the
-    // first column token parks them per group of value rows; the flush of the group scales and stores them.
-    float* car = sCar + ((nbl * DG) * 4 + g) * 8;
-    // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
-    float* pw = ((g < 2) ? sPv : sPb) + nbl * DG * kC + 16 * (2 * HF + (g & 1)) + i;
-
-    int b3 = 0;   // LAG: d mod 3
-    for (int it = 0; it < dv + LAGC; ++it) {
-      if (it >= LAGC) {
-        const int d = it - LAGC, dd = d & (DG - 1), buf = (d / DG) & 1;
-        const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
-        const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
-        const bf16x8* slot = sX + ((nbl * 2 + (d & 1)) * OPN) * 64 + lane;
-        const bf16x8* p0 = sX + (nbl * 20 + 4 * b3) * 64 + lane;              // LAG: the first producer's operands
-        const bf16x8* p1 = sX + (nbl * 20 + 12 + 4 * (d & 1)) * 64 + lane;    //      the second producer's
-        const float* mj = sMJ + (LAG ? nbl * 4 + (d & 3) : nbl * 2 + (d & 1)) * 32;
-        if constexpr (LAG) b3 = (b3 == 2) ? 0 : b3 + 1;
-        // HF=0 (column tokens 0..31): reverse needs both P halves, strictly-lower only X_0;
-        // HF=1 (column tokens 32..63): reverse needs P_1 only, strictly-lower both X halves
-        const bf16x8 PM1 = LAG ? p1[0] : slot[1 * 64], PJ1 = LAG ? p1[64] : slot[3 * 64];
-        bf16x8 XM0 = LAG ? p0[2 * 64] : slot[4 * 64], XJ0 = LAG ? p0[3 * 64] : slot[6 * 64];
-        bf16x8 Ma = LAG ? (HF ? p1[2 * 64] : p0[0]) : slot[(HF ? 5 : 0) * 64];    // HF=0: P^M_0, HF=1: X^M_1
-        bf16x8 Ja = LAG ? (HF ? p1[3 * 64] : p0[64]) : slot[(HF ? 7 : 2) * 64];   // HF=0: P^J_0, HF=1: X^J_1
-        bf16x8 PM1l, PJ1l, XM0l, XJ0l, Mal, Jal;     // PREC: the lo halves of the six
-        if constexpr (PREC) {
-          PM1l = slot[(8 + 1) * 64]; PJ1l = slot[(8 + 3) * 64]; XM0l = slot[(8 + 4) * 64]; XJ0l = slot[(8 + 6) * 64];
-          Mal = slot[(8 + (HF ? 5 : 0)) * 64];
-          Jal = slot[(8 + (HF ? 7 : 2)) * 64];
-        }
-        f32x4 M0T, J0T;
-        if constexpr (PREC) {
-          M0T = *(const f32x4*)&mj[4 * g];
-          J0T = *(const f32x4*)&mj[16 + 4 * g];
-        } else if (!(FOLD && HF)) {
-          // tile-start state of the row as the virtual token of the strictly-lower product: element 7 of the lanes
-          // g = 3 of its last operand (token 31 / 63 of the contraction, which no column token of this wave uses)
-          const bf16x2 mj2 = pack2(mj[i], mj[16 + i]);
-          if (g == 3) {
-            if (HF) { Ma[7] = mj2[0]; Ja[7] = mj2[1]; } else { XM0[7] = mj2[0]; XJ0[7] = mj2[1]; }
-          }
-        }
-        float dvp[2], dbp[2];
-#pragma unroll
-        for (int sl = 0; sl < 2; ++sl) {
-          const int sb = 2 * HF + sl;
-          f32x4 aM = {0.f, 0.f, 0.f, 0.f}, aJ = {0.f, 0.f, 0.f, 0.f};
-          f32x4 sM = {0.f, 0.f, 0.f, 0.f}, sJ = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (PREC) {
-            if (!HF) {
-              aM = mfma16_split(Ma, Mal, Lop[2 * sl], Lol[2 * sl], aM);
-              aJ = mfma16_split(Ja, Jal, Lop[2 * sl], Lol[2 * sl], aJ);
-              aM = mfma16_split(PM1, PM1l, Lop[2 * sl + 1], Lol[2 * sl + 1], aM);
-              aJ = mfma16_split(PJ1, PJ1l, Lop[2 * sl + 1], Lol[2 * sl + 1], aJ);
-              sM = mfma16_split(XM0, XM0l, Lop[4 + sl], Lol[4 + sl], sM);
-              sJ = mfma16_split(XJ0, XJ0l, Lop[4 + sl], Lol[4 + sl], sJ);
-            } else {
-              aM = mfma16_split(PM1, PM1l, Lop[sl], Lol[sl], aM);
-              aJ = mfma16_split(PJ1, PJ1l, Lop[sl], Lol[sl], aJ);
-              sM = mfma16_split(XM0, XM0l, Lop[2 + 2 * sl], Lol[2 + 2 * sl], sM);
-              sJ = mfma16_split(XJ0, XJ0l, Lop[2 + 2 * sl], Lol[2 + 2 * sl], sJ);
-              sM = mfma16_split(Ma, Mal, Lop[2 + 2 * sl + 1], Lol[2 + 2 * sl + 1], sM);
-              sJ = mfma16_split(Ja, Jal, Lop[2 + 2 * sl + 1], Lol[2 + 2 * sl + 1], sJ);
-            }
-          } else if (!HF) {
-            aM = mfma16(Ma, Lop[2 * sl], aM);
-            aJ = mfma16(Ja, Lop[2 * sl], aJ);
-            aM = mfma16(PM1, Lop[2 * sl + 1], aM);
-            aJ = mfma16(PJ1, Lop[2 * sl + 1], aJ);
-            // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
-            sM = mfma16(XM0, Lop[4 + sl], sM);
-            sJ = mfma16(XJ0, Lop[4 + sl], sJ);
-          } else {
-            aM = mfma16(PM1, Lop[sl], aM);
-            aJ = mfma16(PJ1, Lop[sl], aJ);
-            sM = mfma16(XM0, Lop[2 + 2 * sl], sM);
-            sJ = mfma16(XJ0, Lop[2 + 2 * sl], sJ);
-            sM = mfma16(Ma, Lop[2 + 2 * sl + 1], sM);
-            sJ = mfma16(Ja, Lop[2 + 2 * sl + 1], sJ);
-          }
-          const float vS = sV[16 * sb + i];
-          const float bS = sB[16 * sb + i];
-          float dvs = 0.f, dbs = 0.f, gm = gate[sl];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float kv = kr[sl * 4 + r];
-            dvs = fmaf(aM[r], kv, dvs);
-            dbs = fmaf(aJ[r] * kv, kv, dbs);
-            dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
-            dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
-            const float Ss = PREC ? fmaf(Fs[sl], M0T[r], sM[r]) : sM[r];
-            const float SJ = PREC ? fmaf(Fs[sl], J0T[r], sJ[r]) : sJ[r];
-            gm = fmaf(aM[r], Ss, gm);
-            gm = fmaf(aJ[r], SJ, gm);
-          }
-          gate[sl] = gm;
-          dvp[sl] = dvs;
-          dbp[sl] = dbs;
-          if (!HF && sl == 0 && i == 0) {
-            *(f32x4*)&car[dd * 32] = aM;
-            *(f32x4*)&car[dd * 32 + 4] = aJ;
-          }
-        }
-        pw[dd * kC] = rows4_sum_x4(dvp[0], dvp[1], dbp[0], dbp[1]);
-      }
-      iter_tail(it);
-    }
-
-    TIn* dkp = (TIn*)A.dk + ((int64_t)t0 * H + h) * dk + 16 * nb;
-#pragma unroll
-    for (int sl = 0; sl < 2; ++sl) {
-      const int s = 16 * (2 * HF + sl) + i;
-      if (s < clen) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          (dkp + (int64_t)s * rso)[4 * g + r] = from_f32<TIn>(fmaf(2.f * kr[sl * 4 + r], dkJ[sl * 4 + r], dkM[sl * 4 + r]));
-      }
-      const float x = rows4_sum(gate[sl]);
-      if (g == 0) sRed[nbl * kC + 16 * (2 * HF + sl) + i] = x;
-    }
-  };
-
-
-  // ------------------------------------------------------------------ SUB: the tile as two halves of 32 tokens
-  // (bf16 operands, no initial state, LAG).  A causal product over 64 tokens costs 6 matrix instructions per 16
-  // columns (token blocks of 16 against K = 16, 32, 48, 64, padded to multiples of 32), over two halves of 32 tokens
-  // 4: the second half starts from the state after token 31, which the first producer has in its accumulators.
-  // That state travels the way the tile-start state does (FOLD above): the second producer adds f_32 (M_31, J_31) to
-  // the operand of token 32; the strictly-lower product of the second half gets it for token 32 itself as a virtual
-  // token in its last contraction slot.  The reverse contraction of the first half needs what flows back over the
-  // border, f_32 dM^loc_32 = sum_{t >= 32} 2^(c_t - c_31) dMloc_t: the second producer sums it from its fp32 local
-  // gradients and the first consumer adds it to the local gradient of token 31 in its operand.  The two producers
-  // are then the same code on tokens 0..31 and 32..63 and each consumer reads only its own half's operands:
-  // 36 -> 24 matrix instructions and 22 -> 16 KB of LDS traffic per value row and column block.
+  // ------------------------------------------------------------------ the tile as two halves of 32 tokens
+  // A causal product over 64 tokens costs 6 matrix instructions per 16 columns (token blocks of 16 against
+  // K = 16, 32, 48, 64, padded to multiples of 32), over two halves of 32 tokens 4: the second half starts from the
+  // state after token 31, which the first producer has in its accumulators and leaves in sMJ for the second one, a
+  // row behind.  The reverse contraction of the first half needs what flows back over the border,
+  // f_32 dM^loc_32 = sum_{t >= 32} 2^(c_t - c_31) dMloc_t: the second producer sums it from its local gradients and
+  // the first consumer adds it to the local gradient of token 31 in its operand.  The two producers are then the
+  // same code on tokens 0..31 and 32..63 and each consumer reads only its own half's operands: 24 matrix
+  // instructions (PREC: 72) and 16 KB of LDS traffic per value row and column block.
   //   sMJ slot of a row (d mod 3): [M_0, J_0, M_31, J_31, f_32 dM^loc_32, f_32 dJ^loc_32][16 key columns]
-  auto producer_sub = [&](auto hfc) {
+  // How the state before a half (M_p, J_p) enters its products:
+  //   FOLD (bf16 operands, no initial state): it rides in the operand of the half's first token,
+  //     X'_first = X_first + f_first (M_p, J_p), since the decay from before the half to token t is L[t,first] f_first;
+  //     the strictly-lower product gets it for the first token itself as a virtual token in its last contraction slot
+  //     (token 31 / 63, which is never below a column token of the half).  The state is rounded to bf16 there like
+  //     every other operand; a J_0 below zero (an initial state with I_0 < Ip) would cancel against Ip, so launches
+  //     with an initial state take the next form;
+  //   else in fp32: M_t = Fh_t M_p + (product), with Fh_t = sF[t] the decay from before the half; the strictly-lower
+  //     product of bf16 operands takes Fh_s M_p through the virtual token (on every column), that of split
+  //     operands (PREC) adds it in fp32.
+  auto producer = [&](auto hfc, auto foldc) {
     constexpr int HF = decltype(hfc)::value;   // tokens 32HF .. 32HF+31
+    constexpr bool FOLD = decltype(foldc)::value;
     bf16x8 Lop[2];            // L[t,s] inside the half: t = 32HF+16tl+i, s = 32HF+8g+j <= t
+    bf16x8 Lol[PREC ? 2 : 1]; // PREC: its lo halves
     float kk[8], kk2[8];      // k and its square in operand layout (n = i, s = 32HF+8g+j)
     float qq[8];              // q in result layout (t = 32HF+16tl+4g+r, n = i)
     float dq[8];
-    bf16x2 wD[HF ? 4 : 1];    // second half: 2^(c_t - c_31), the weight of token t in what flows back to token 31 (pairs)
+    // second half: 2^(c_t - c_31), the weight of token t in what flows back to token 31 (bf16 pairs / PREC: fp32)
+    bf16x2 wD[(HF && !PREC) ? 4 : 1];
+    float wDf[(HF && PREC) ? 8 : 1];
     float sigacc = 0.f;
     {
       const TIn* kp = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
@@ -680,10 +274,12 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl) {
           const int t = 32 * HF + 16 * tl + i;
-          Lop[tl][j] = (bf16_t)((s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f);
+          const float lv = (s <= t) ? fast_exp2(ct[tl] - cs[j]) : 0.f;
+          const bf16_t lh = (bf16_t)lv;
+          Lop[tl][j] = lh;
+          if constexpr (PREC) Lol[tl][j] = (bf16_t)(lv - (float)lh);
         }
       }
-      const float c31 = sC[31];
 #pragma unroll
       for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
@@ -696,12 +292,16 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         }
       if (HF) {
 #pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
+        for (int tl = 0; tl < 2; ++tl) {
+          const f32x4 w4 = *(const f32x4*)&sF[32 + 16 * tl + 4 * g];
+          if constexpr (PREC) {
 #pragma unroll
-          for (int r = 0; r < 4; r += 2) {
-            const int t = 32 + 16 * tl + 4 * g + r;
-            wD[tl * 2 + r / 2] = pack2(fast_exp2(sC[t] - c31), fast_exp2(sC[t + 1] - c31));
+            for (int r = 0; r < 4; ++r) wDf[tl * 4 + r] = w4[r];
+          } else {
+            wD[tl * 2] = pack2(w4[0], w4[1]);
+            wD[tl * 2 + 1] = pack2(w4[2], w4[3]);
           }
+        }
       }
     }
     // first half: tile-start state of the next value row (entry of the own key column n = i), fetched one row ahead
@@ -709,10 +309,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     const float* cI = a.chunk_I + tile_off + 16 * nb;
     float mu_n = 0.f, I_n = 0.f;
     if (!HF) { mu_n = cmu[i]; I_n = cI[i]; }
-    // decay of the incoming state into the first token of the half, on the lanes that hold that token's operand
-    const float f0m = (g == 0) ? fast_exp2(HF ? sC[32] - sC[31] : sC[0]) : 0.f;
+    // FOLD: decay of the incoming state into the first token of the half, on the lanes that hold that token's operand
+    const float f0m = (FOLD && g == 0) ? sF[32 * HF] : 0.f;
     int b3 = 0;                                 // d mod 3: the row's slot of sMJ and of the first producer's operands
-    for (int it = 0; it < dv + LAGC; ++it) {
+    for (int it = 0; it < dv + kLagC; ++it) {
       if (it >= HF && it - HF < dv) {
         const int d = it - HF, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
@@ -733,42 +333,63 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           Mp = mj[32 + i];
           Jp = mj[48 + i];
         }
-        const float fM = f0m * Mp, fJ = f0m * Jp;
         bf16x8 XM, XJ;
+        bf16x8 XMl, XJl;   // PREC: the lo halves
         {
           const f32x4 v0 = *(const f32x4*)&sV[32 * HF + 8 * g], v1 = *(const f32x4*)&sV[32 * HF + 8 * g + 4];
           const f32x4 b0 = *(const f32x4*)&sB[32 * HF + 8 * g], b1 = *(const f32x4*)&sB[32 * HF + 8 * g + 4];
+          if constexpr (PREC) {
+            float xm[8], xj[8];
 #pragma unroll
-          for (int j = 0; j < 8; j += 2) {
-            const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
-            const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
-            const bf16x2 pm = pack2(j == 0 ? fmaf(kk[j], va, fM) : kk[j] * va, kk[j + 1] * vb);
-            const bf16x2 pj = pack2(j == 0 ? fmaf(kk2[j], ba, fJ) : kk2[j] * ba, kk2[j + 1] * bb);
-            XM[j] = pm[0]; XM[j + 1] = pm[1];
-            XJ[j] = pj[0]; XJ[j + 1] = pj[1];
+            for (int j = 0; j < 8; ++j) {
+              xm[j] = kk[j] * (j < 4 ? v0[j & 3] : v1[j & 3]);
+              xj[j] = kk2[j] * (j < 4 ? b0[j & 3] : b1[j & 3]);
+            }
+            split_bf16(xm, XM, XMl);
+            split_bf16(xj, XJ, XJl);
+          } else {
+            const float fM = f0m * Mp, fJ = f0m * Jp;
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+              const float va = j < 4 ? v0[j & 3] : v1[j & 3], vb = j < 4 ? v0[(j & 3) + 1] : v1[(j & 3) + 1];
+              const float ba = j < 4 ? b0[j & 3] : b1[j & 3], bb = j < 4 ? b0[(j & 3) + 1] : b1[(j & 3) + 1];
+              const bool tok0 = FOLD && j == 0;
+              const bf16x2 pm = pack2(tok0 ? fmaf(kk[j], va, fM) : kk[j] * va, kk[j + 1] * vb);
+              const bf16x2 pj = pack2(tok0 ? fmaf(kk2[j], ba, fJ) : kk2[j] * ba, kk2[j + 1] * bb);
+              XM[j] = pm[0]; XM[j + 1] = pm[1];
+              XJ[j] = pj[0]; XJ[j + 1] = pj[1];
+            }
           }
         }
         bf16x8 PM, PJ;
+        float pmf[PREC ? 8 : 1], pjf[PREC ? 8 : 1];   // PREC: the local gradients in fp32 until they are split
         float backM = 0.f, backJ = 0.f;
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl) {
           const int tb = 2 * HF + tl;
           f32x4 accM = {0.f, 0.f, 0.f, 0.f};
           f32x4 accI = {Ip, Ip, Ip, Ip};
-          accM = mfma16(Lop[tl], XM, accM);
-          accI = mfma16(Lop[tl], XJ, accI);
-          if (!HF && tl == 1 && g == 3) {   // state after token 31 for the second half of the row
-            mj[32 + i] = accM[3];
-            mj[48 + i] = accI[3] - Ip;
+          if constexpr (PREC) {
+            accM = mfma16_split(Lop[tl], Lol[tl], XM, XMl, accM);
+            accI = mfma16_split(Lop[tl], Lol[tl], XJ, XJl, accI);
+          } else {
+            accM = mfma16(Lop[tl], XM, accM);
+            accI = mfma16(Lop[tl], XJ, accI);
           }
+          f32x4 Fv = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (!FOLD) Fv = *(const f32x4*)&sF[16 * tb + 4 * g];
           const f32x4 dov = *(const f32x4*)&sDo[16 * tb + 4 * g];
           f32x4 dvv = {0.f, 0.f, 0.f, 0.f};
           if (HAS_VAR) dvv = *(const f32x4*)&sDov[16 * tb + 4 * g];
           float dMl[4], dJl[4];
+          float M3 = 0.f, I3 = 0.f;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float rI = fast_rcp(accI[r]);
-            const float mu = accM[r] * rI;
+            const float Mf = FOLD ? accM[r] : fmaf(Fv[r], Mp, accM[r]);
+            const float If = FOLD ? accI[r] : fmaf(Fv[r], Jp, accI[r]);
+            if (r == 3) { M3 = Mf; I3 = If; }
+            const float rI = fast_rcp(If);
+            const float mu = Mf * rI;
             const float q = qq[tl * 4 + r];
             dMl[r] = (dov[r] * q) * rI;
             dJl[r] = -(dMl[r] * mu);
@@ -779,27 +400,51 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
               dJl[r] = fmaf(-w, rI, dJl[r]);
               dq[tl * 4 + r] = fmaf(2.f * wq, rI, dq[tl * 4 + r]);
             }
+            if constexpr (PREC) sigacc += dJl[r];
+          }
+          if (!HF && tl == 1 && g == 3) {   // state after token 31 for the second half of the row
+            mj[32 + i] = M3;
+            mj[48 + i] = I3 - Ip;
           }
           const int o4 = tl * 4;
-          const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
-          const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
-          const bf16x2 one2 = {(bf16_t)1.f, (bf16_t)1.f};
-          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j0, one2, sigacc, false);
-          sigacc = __builtin_amdgcn_fdot2_f32_bf16(j1, one2, sigacc, false);
-          if (HF) {   // what flows back over the border, from the packed pairs
-            backM = __builtin_amdgcn_fdot2_f32_bf16(m0, wD[tl * 2], backM, false);
-            backM = __builtin_amdgcn_fdot2_f32_bf16(m1, wD[tl * 2 + 1], backM, false);
-            backJ = __builtin_amdgcn_fdot2_f32_bf16(j0, wD[tl * 2], backJ, false);
-            backJ = __builtin_amdgcn_fdot2_f32_bf16(j1, wD[tl * 2 + 1], backJ, false);
+          if constexpr (PREC) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              pmf[o4 + r] = dMl[r];
+              pjf[o4 + r] = dJl[r];
+              if (HF) {   // what flows back over the border
+                backM = fmaf(wDf[o4 + r], dMl[r], backM);
+                backJ = fmaf(wDf[o4 + r], dJl[r], backJ);
+              }
+            }
+          } else {
+            const bf16x2 m0 = pack2(dMl[0], dMl[1]), m1 = pack2(dMl[2], dMl[3]);
+            const bf16x2 j0 = pack2(dJl[0], dJl[1]), j1 = pack2(dJl[2], dJl[3]);
+            // the sum of dJloc (for dIp) from the packed pairs: one instruction per two entries
+            const bf16x2 one2 = {(bf16_t)1.f, (bf16_t)1.f};
+            sigacc = __builtin_amdgcn_fdot2_f32_bf16(j0, one2, sigacc, false);
+            sigacc = __builtin_amdgcn_fdot2_f32_bf16(j1, one2, sigacc, false);
+            if (HF) {   // what flows back over the border, from the packed pairs
+              backM = __builtin_amdgcn_fdot2_f32_bf16(m0, wD[tl * 2], backM, false);
+              backM = __builtin_amdgcn_fdot2_f32_bf16(m1, wD[tl * 2 + 1], backM, false);
+              backJ = __builtin_amdgcn_fdot2_f32_bf16(j0, wD[tl * 2], backJ, false);
+              backJ = __builtin_amdgcn_fdot2_f32_bf16(j1, wD[tl * 2 + 1], backJ, false);
+            }
+            PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
+            PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
           }
-          PM[o4 + 0] = m0[0]; PM[o4 + 1] = m0[1]; PM[o4 + 2] = m1[0]; PM[o4 + 3] = m1[1];
-          PJ[o4 + 0] = j0[0]; PJ[o4 + 1] = j0[1]; PJ[o4 + 2] = j1[0]; PJ[o4 + 3] = j1[1];
         }
         if (HF) {   // sums over the four lane rows: row 0 gets the mean branch's total, row 1 the precision branch's
           const float tot = rows4_sum_x4(backM, backJ, 0.f, 0.f);
           if (g < 2) mj[64 + 16 * g + i] = tot;
         }
-        bf16x8* mine = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;
+        bf16x8* mine = sX + ((nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * XS) * 64 + lane;
+        if constexpr (PREC) {
+          bf16x8 PMl, PJl;
+          split_bf16(pmf, PM, PMl);
+          split_bf16(pjf, PJ, PJl);
+          mine[4 * 64] = PMl; mine[5 * 64] = PJl; mine[6 * 64] = XMl; mine[7 * 64] = XJl;
+        }
         mine[0] = PM; mine[64] = PJ; mine[2 * 64] = XM; mine[3 * 64] = XJ;
         b3 = (b3 == 2) ? 0 : b3 + 1;
       }
@@ -817,13 +462,16 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     if (lane == 0) sRed[NB * kC + HF * NB + nbl] = x;
   };
 
-  auto consumer_sub = [&](auto hfc) {
+  // ------------------------------------------------------------------ consumers
+  auto consumer = [&](auto hfc, auto foldc) {
     constexpr int HF = decltype(hfc)::value;   // column tokens 32HF .. 32HF+31 (blocks sb = 2HF+sl)
+    constexpr bool FOLD = decltype(foldc)::value;
     bf16x8 Lr[2];     // reverse operand inside the half: contraction (g,j) <-> token t = 32HF + 16(j/4) + 4g + j%4 >= s
     bf16x8 Ls[2];     // strictly-lower operand: contraction token s' = 32HF + 8g + j < column token s = 16sb+i
+    bf16x8 Lrl[PREC ? 2 : 1], Lsl[PREC ? 2 : 1];   // PREC: their lo halves
     float kr[8], kr2[8];   // k and its square in result layout (s = 16sb+i, n = 4g+r)
     float dkM[8], dkJ[8];
-    float gate[2];
+    float gate[2], Fs[2];
     {
       const TIn* kp4 = (const TIn*)a.k + qk_row(a, t0, h) + 16 * nb;
       float ct[2], cs[8], ctt[8];
@@ -833,21 +481,25 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
       *(f32x4*)&cs[4] = *(const f32x4*)&sC[32 * HF + 8 * g + 4];
       *(f32x4*)&ctt[0] = *(const f32x4*)&sC[32 * HF + 4 * g];
       *(f32x4*)&ctt[4] = *(const f32x4*)&sC[32 * HF + 16 + 4 * g];
-      // the last contraction slot of the half (token 31 / 63) is never below a column token of the half: it carries
-      // the state before the half's first token, which only that token's column takes (the later ones have it
-      // through the first token's operand)
-      const float fst = HF ? fast_exp2(sC[32] - sC[31]) : fast_exp2(sC[0]);
 #pragma unroll
       for (int sl = 0; sl < 2; ++sl) {
         const int s = 16 * (2 * HF + sl) + i;
+        Fs[sl] = sF[s];   // decay from before the half to the column token
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int sp = 32 * HF + 8 * g + j;
           float lv = (sp < s) ? fast_exp2(ct[sl] - cs[j]) : 0.f;
-          if (g == 3 && j == 7) lv = (s == 32 * HF) ? fst : 0.f;
-          Ls[sl][j] = (bf16_t)lv;
+          // the virtual token (bf16 operands): the state before the half, for the half's first token only when the
+          // operands carry it already (FOLD), else for every column token
+          if (!PREC && g == 3 && j == 7) lv = (FOLD && s != 32 * HF) ? 0.f : Fs[sl];
+          const bf16_t lh = (bf16_t)lv;
+          Ls[sl][j] = lh;
+          if constexpr (PREC) Lsl[sl][j] = (bf16_t)(lv - (float)lh);
           const int t = 32 * HF + 16 * (j >> 2) + 4 * g + (j & 3);
-          Lr[sl][j] = (bf16_t)((t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f);
+          const float rv = (t >= s) ? fast_exp2(ctt[j] - ct[sl]) : 0.f;
+          const bf16_t rh = (bf16_t)rv;
+          Lr[sl][j] = rh;
+          if constexpr (PREC) Lrl[sl][j] = (bf16_t)(rv - (float)rh);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) { kr[sl * 4 + r] = 0.f; dkM[sl * 4 + r] = 0.f; dkJ[sl * 4 + r] = 0.f; }
@@ -857,20 +509,30 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
         gate[sl] = 0.f;
       }
     }
+    // the carries between tiles are kept in the dtype of the rows: bf16 rows feed them to the matrix cores in bf16
+    // anyway (carry apply), and the scan that sums them over the tiles runs in fp32 registers.  The consumer of the
+    // first column token parks them per group of value rows; the flush of the group scales and stores them.
     float* car = sCar + ((nbl * DG) * 4 + g) * 8;
     // after the 4-way transposing reduction, row g of the wave holds dv (g<2) or db (g>=2) of token block g&1
     float* pw = ((g < 2) ? sPv : sPb) + nbl * DG * kC + 16 * (2 * HF + (g & 1)) + i;
     int b3 = 0;   // d mod 3
-    for (int it = 0; it < dv + LAGC; ++it) {
-      if (it >= LAGC) {
-        const int d = it - LAGC, dd = d & (DG - 1), buf = (d / DG) & 1;
+    for (int it = 0; it < dv + kLagC; ++it) {
+      if (it >= kLagC) {
+        const int d = it - kLagC, dd = d & (DG - 1), buf = (d / DG) & 1;
         const float* sV = sSt + (buf * NST + 0) * STG + dd * kVS2;
         const float* sB = sSt + (buf * NST + 1) * STG + dd * kVS2;
-        const bf16x8* ph = sX + (nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * 64 + lane;   // the own half's operands
+        // the own half's operands
+        const bf16x8* ph = sX + ((nbl * 20 + (HF ? 12 + 4 * (d & 1) : 4 * b3)) * XS) * 64 + lane;
         const float* mj = sMJ + (nbl * 3 + b3) * 96;
         b3 = (b3 == 2) ? 0 : b3 + 1;
         bf16x8 PM = ph[0], PJ = ph[64], XM = ph[2 * 64], XJ = ph[3 * 64];
-        {
+        bf16x8 PMl, PJl, XMl, XJl;   // PREC: the lo halves
+        f32x4 MpT = {0.f, 0.f, 0.f, 0.f}, JpT = {0.f, 0.f, 0.f, 0.f};   // PREC: state before the half, key columns n = 4g+r
+        if constexpr (PREC) {
+          PMl = ph[4 * 64]; PJl = ph[5 * 64]; XMl = ph[6 * 64]; XJl = ph[7 * 64];
+          MpT = *(const f32x4*)&mj[32 * HF + 4 * g];
+          JpT = *(const f32x4*)&mj[32 * HF + 16 + 4 * g];
+        } else {
           // virtual token of the strictly-lower products: the state before the half's first token (key column n = i)
           const bf16x2 st2 = pack2(mj[32 * HF + i], mj[32 * HF + 16 + i]);
           if (g == 3) { XM[7] = st2[0]; XJ[7] = st2[1]; }
@@ -879,8 +541,15 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
           // what flows back over the border joins the local gradient of token 31 (element 7 of the lanes g = 3)
           const float bm = mj[64 + i], bj = mj[80 + i];
           if (g == 3) {
-            PM[7] = (bf16_t)((float)PM[7] + bm);
-            PJ[7] = (bf16_t)((float)PJ[7] + bj);
+            if constexpr (PREC) {
+              const float xm = ((float)PM[7] + (float)PMl[7]) + bm, xj = ((float)PJ[7] + (float)PJl[7]) + bj;
+              const bf16_t mh = (bf16_t)xm, jh = (bf16_t)xj;
+              PM[7] = mh; PMl[7] = (bf16_t)(xm - (float)mh);
+              PJ[7] = jh; PJl[7] = (bf16_t)(xj - (float)jh);
+            } else {
+              PM[7] = (bf16_t)((float)PM[7] + bm);
+              PJ[7] = (bf16_t)((float)PJ[7] + bj);
+            }
           }
         }
         float dvp[2], dbp[2];
@@ -888,9 +557,19 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
 #pragma unroll
         for (int sl = 0; sl < 2; ++sl) {
           const int sb = 2 * HF + sl;
-          const f32x4 aM = mfma16(PM, Lr[sl], z4), aJ = mfma16(PJ, Lr[sl], z4);
-          // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
-          const f32x4 sM = mfma16(XM, Ls[sl], z4), sJ = mfma16(XJ, Ls[sl], z4);
+          f32x4 aM, aJ, sM, sJ;
+          if constexpr (PREC) {
+            aM = mfma16_split(PM, PMl, Lr[sl], Lrl[sl], z4);
+            aJ = mfma16_split(PJ, PJl, Lr[sl], Lrl[sl], z4);
+            sM = mfma16_split(XM, XMl, Ls[sl], Lsl[sl], z4);
+            sJ = mfma16_split(XJ, XJl, Ls[sl], Lsl[sl], z4);
+          } else {
+            aM = mfma16(PM, Lr[sl], z4);
+            aJ = mfma16(PJ, Lr[sl], z4);
+            // S[n, s] = f_s M_{s-1}: strictly-lower product in the same [n, s] layout
+            sM = mfma16(XM, Ls[sl], z4);
+            sJ = mfma16(XJ, Ls[sl], z4);
+          }
           const float vS = sV[16 * sb + i];
           const float bS = sB[16 * sb + i];
           float dvs = 0.f, dbs = 0.f, gm = gate[sl];
@@ -900,8 +579,10 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
             dbs = fmaf(aJ[r], kr2[sl * 4 + r], dbs);
             dkM[sl * 4 + r] = fmaf(aM[r], vS, dkM[sl * 4 + r]);
             dkJ[sl * 4 + r] = fmaf(aJ[r], bS, dkJ[sl * 4 + r]);
-            gm = fmaf(aM[r], sM[r], gm);
-            gm = fmaf(aJ[r], sJ[r], gm);
+            const float Ss = PREC ? fmaf(Fs[sl], MpT[r], sM[r]) : sM[r];
+            const float SJ = PREC ? fmaf(Fs[sl], JpT[r], sJ[r]) : sJ[r];
+            gm = fmaf(aM[r], Ss, gm);
+            gm = fmaf(aJ[r], SJ, gm);
           }
           gate[sl] = gm;
           dvp[sl] = dvs;
@@ -944,14 +625,9 @@ void chunk_bwd_local_roles_kernel(BwdArgs A) {
     stage(0);
     __syncthreads();
     if (MULTI && nbl >= n_act) {
-      for (int it = 0; it < dv + LAGC; ++it) iter_tail(it);
+      for (int it = 0; it < dv + kLagC; ++it) iter_tail(it);
     } else if (fold) {
-      if constexpr (LAG) {
-        if (role == 0) producer_sub(std::integral_constant<int, 0>{});
-        else if (role == 1) producer_sub(std::integral_constant<int, 1>{});
-        else if (role == 2) consumer_sub(std::integral_constant<int, 0>{});
-        else consumer_sub(std::integral_constant<int, 1>{});
-      } else if constexpr (!PREC) {
+      if constexpr (!PREC) {
         if (role == 0) producer(std::integral_constant<int, 0>{}, std::true_type{});
         else if (role == 1) producer(std::integral_constant<int, 1>{}, std::true_type{});
         else if (role == 2) consumer(std::integral_constant<int, 0>{}, std::true_type{});
@@ -1512,11 +1188,9 @@ struct BwdPlan {
 };
 
 static size_t local_lds_bytes(int NB, bool var, bool prec) {
-  const bool lag = local_lag(NB, prec);
   const int DG = local_dg(NB, prec);
-  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * DG * kVS2 + 2 * NB * DG * kC +
-                          NB * (lag ? 288 : 64) + NB * DG * 32) +
-         (size_t)NB * (lag ? 20 : 2 * (prec ? 16 : 8)) * 64 * 16;
+  return sizeof(float) * (2 * kC + 2 * (var ? 4 : 3) * DG * kVS2 + 2 * NB * DG * kC + NB * 288 + NB * DG * 32) +
+         (size_t)NB * 20 * (prec ? 2 : 1) * 64 * 16;
 }
 
 // prec: the fp32-accurate variants (fp32 rows without PAL_FLAG_FP32_FAST)
