@@ -10,6 +10,8 @@
 // by a group of GL lanes (the power of two >= d/8), eight consecutive elements per lane (16-byte
 // accesses for bf16 rows); a workgroup of 256 threads owns one head and a range of tokens, so that the
 // per-head sums of the backward are accumulated in a fixed order (no atomics).
+#include <type_traits>
+
 #include "pal_common.h"
 #include "pal_host.h"
 #include "pal_profile.h"
@@ -17,6 +19,12 @@
 namespace pal {
 
 constexpr int kGlueIter = 8;   // rows per row slot of a workgroup
+// rows of a slot that are fetched before the first of them is used: a thread has one or two 16-byte fetches per row and
+// tensor, and taken one row at a time each fetch waits for the stores of the row before it (the kernels ran at
+// 3.3-3.7 TB/s that way).  Four rows in the forward kernels; two in the backward ones, which hold twice the tensors
+// per row (with four they need 200 registers and lose more to the occupancy than they gain).
+constexpr int kGlueBatch = 4;
+constexpr int kGlueBatchBwd = 2;
 
 template <typename T>
 __device__ __forceinline__ void load8(const T* p, float* x) {
@@ -28,6 +36,11 @@ __device__ __forceinline__ void store8(T* p, const float* x) {
   store_vec<4>(p, x);
   store_vec<4>(p + 4, x + 4);
 }
+// eight fp32 elements as two 16-byte accesses (rows are 16-byte aligned)
+struct F32x8 {
+  f32x4 lo, hi;
+  __device__ __forceinline__ float operator[](int e) const { return e < 4 ? lo[e & 3] : hi[e & 3]; }
+};
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
@@ -95,18 +108,29 @@ __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
     const T* src = (const T*)(task ? A.t.k_raw : A.t.q_raw);
     T* dst = (T*)(task ? A.t.k : A.t.q);
     const bool on = 8 * l < d;
-    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-      float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (on) load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, x);
-      float ss = 0.f;
+    for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatch * rows) {
+      float xb[kGlueBatch][8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
-      ss = group_sum(ss, GL);
-      const float inv = rcpf_(fmaxf(__builtin_amdgcn_sqrtf(ss), A.eps));
+      for (int u = 0; u < kGlueBatch; ++u) {
+        const int tok = tb + u * rows;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] *= inv;
-      if (on)
-        for (int r = 0; r < rep; ++r) store8(dst + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, x);
+        for (int e = 0; e < 8; ++e) xb[u][e] = 0.f;
+        if (on && tok < tok1) load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, xb[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kGlueBatch; ++u) {
+        const int tok = tb + u * rows;
+        float* x = xb[u];
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+        ss = group_sum(ss, GL);
+        const float inv = rcpf_(fmaxf(__builtin_amdgcn_sqrtf(ss), A.eps));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= inv;
+        if (on && tok < tok1)
+          for (int r = 0; r < rep; ++r) store8(dst + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, x);
+      }
     }
   } else {
     const int GL = A.GLv, d = A.dv;
@@ -114,28 +138,47 @@ __global__ __launch_bounds__(256) void prologue_fwd_kernel(PrologueArgs A) {
     const bool on = 8 * l < d;
     const float sp = A.t.b_raw ? softplusf_(A.t.b_scale[h]) : 0.f;
     const float bias = A.t.dt_bias[h];
-    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-      const int64_t th = (int64_t)tok * A.H + h;
-      float gtv = softplusf_(to_f32(((const T*)A.t.dt_raw)[th]) + bias), bs;
-      if (A.mamba) {
-        gtv = fminf(fmaxf(gtv, A.dt_min), A.dt_max);
-        bs = gtv;
-      } else {
-        bs = round_to<T>(sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th])));
+    const bool has_b = A.t.b_raw != nullptr;
+    for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatch * rows) {
+      float xb[kGlueBatch][8], bb[kGlueBatch][8], dtr[kGlueBatch], bsr[kGlueBatch];
+#pragma unroll
+      for (int u = 0; u < kGlueBatch; ++u) {
+        const int tok = tb + u * rows;
+        dtr[u] = bsr[u] = 0.f;
+        if (tok < tok1) {
+          const int64_t th = (int64_t)tok * A.H + h;
+          dtr[u] = to_f32(((const T*)A.t.dt_raw)[th]);
+          if (!A.mamba) bsr[u] = to_f32(((const T*)A.t.bs_raw)[th]);
+          if (on) {
+            load8((const T*)A.t.x + th * d + 8 * l, xb[u]);
+            if (has_b) load8((const T*)A.t.b_raw + th * d + 8 * l, bb[u]);
+          }
+        }
       }
-      if (l == 0) A.t.gt[th] = gtv;
-      if (!on) continue;
-      float x[8];
-      load8((const T*)A.t.x + th * d + 8 * l, x);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] *= bs;
-      store8((T*)A.t.v + th * d + 8 * l, x);
-      if (A.t.b_raw) {
-        float br[8];
-        load8((const T*)A.t.b_raw + th * d + 8 * l, br);
+      for (int u = 0; u < kGlueBatch; ++u) {
+        const int tok = tb + u * rows;
+        if (tok >= tok1) break;
+        const int64_t th = (int64_t)tok * A.H + h;
+        float gtv = softplusf_(dtr[u] + bias), bs;
+        if (A.mamba) {
+          gtv = fminf(fmaxf(gtv, A.dt_min), A.dt_max);
+          bs = gtv;
+        } else {
+          bs = round_to<T>(sigmoidf_(bsr[u]));
+        }
+        if (l == 0) A.t.gt[th] = gtv;
+        if (!on) continue;
+        float* x = xb[u];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) br[e] = sigmoidf_(br[e]) * sp * bs;
-        store8((T*)A.t.b + th * d + 8 * l, br);
+        for (int e = 0; e < 8; ++e) x[e] *= bs;
+        store8((T*)A.t.v + th * d + 8 * l, x);
+        if (has_b) {
+          float* br = bb[u];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) br[e] = sigmoidf_(br[e]) * sp * bs;
+          store8((T*)A.t.b + th * d + 8 * l, br);
+        }
       }
     }
   }
@@ -157,30 +200,41 @@ __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
     const T* gsrc = (const T*)(task ? A.g.dk : A.g.dq);
     T* dst = (T*)(task ? A.g.dk_raw : A.g.dq_raw);
     const bool on = 8 * l < d;
-    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-      float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (on) {
-        load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, x);
-        for (int r = 0; r < rep; ++r) {
-          float gy[8];
-          load8(gsrc + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, gy);
+    for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatchBwd * rows) {
+      float xb[kGlueBatchBwd][8], sb[kGlueBatchBwd][8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) s[e] += gy[e];
+      for (int u = 0; u < kGlueBatchBwd; ++u) {
+        const int tok = tb + u * rows;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xb[u][e] = sb[u][e] = 0.f;
+        if (on && tok < tok1) {
+          load8(src + ((int64_t)tok * A.Hqk + h) * d + 8 * l, xb[u]);
+          for (int r = 0; r < rep; ++r) {
+            float gy[8];
+            load8(gsrc + ((int64_t)tok * A.H + h * rep + r) * d + 8 * l, gy);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sb[u][e] += gy[e];
+          }
         }
       }
-      float ss = 0.f, xs = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { ss = fmaf(x[e], x[e], ss); xs = fmaf(x[e], s[e], xs); }
-      ss = group_sum(ss, GL);
-      xs = group_sum(xs, GL);
-      const float nrm = __builtin_amdgcn_sqrtf(ss);
-      const bool clamped = nrm < A.eps;
-      const float inv = rcpf_(fmaxf(nrm, A.eps));
-      const float c = clamped ? 0.f : xs * inv * inv * inv;   // (y . s) / n^2 * ... folded: dx = s/n - x (x.s)/n^3
-      float out[8];
+      for (int u = 0; u < kGlueBatchBwd; ++u) {
+        const int tok = tb + u * rows;
+        const float *x = xb[u], *s = sb[u];
+        float ss = 0.f, xs = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) out[e] = s[e] * inv - x[e] * c;
-      if (on) store8(dst + ((int64_t)tok * A.Hqk + h) * d + 8 * l, out);
+        for (int e = 0; e < 8; ++e) { ss = fmaf(x[e], x[e], ss); xs = fmaf(x[e], s[e], xs); }
+        ss = group_sum(ss, GL);
+        xs = group_sum(xs, GL);
+        const float nrm = __builtin_amdgcn_sqrtf(ss);
+        const bool clamped = nrm < A.eps;
+        const float inv = rcpf_(fmaxf(nrm, A.eps));
+        const float c = clamped ? 0.f : xs * inv * inv * inv;   // dx = s/n - x (x.s)/n^3
+        float out[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = s[e] * inv - x[e] * c;
+        if (on && tok < tok1) store8(dst + ((int64_t)tok * A.Hqk + h) * d + 8 * l, out);
+      }
     }
   } else {
     const int GL = A.GLv, d = A.dv;
@@ -190,55 +244,78 @@ __global__ __launch_bounds__(256) void prologue_bwd_kernel(PrologueArgs A) {
     const float sp = has_b ? softplusf_(A.t.b_scale[h]) : 0.f;
     const float bias = A.t.dt_bias[h];
     float acc_dt = 0.f, acc_bs = 0.f;   // this thread's share of ddt_bias[h] and of sum db * sigmoid(b_raw) * bs
-    for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-      const int64_t th = (int64_t)tok * A.H + h;
-      const float pre = to_f32(((const T*)A.t.dt_raw)[th]) + bias;
-      float sg = 0.f, bs;
-      bool pass = true;     // mamba: the clamp lets the gradient through (bounds included, as torch.clamp)
-      if (A.mamba) {
-        const float spd = softplusf_(pre);
-        pass = spd >= A.dt_min && spd <= A.dt_max;
-        bs = fminf(fmaxf(spd, A.dt_min), A.dt_max);
-      } else {
-        sg = sigmoidf_(to_f32(((const T*)A.t.bs_raw)[th]));
-        bs = round_to<T>(sg);
-      }
-      float dbs = 0.f, dsp = 0.f;
-      if (on) {
-        float x[8], gv[8];
-        load8((const T*)A.t.x + th * d + 8 * l, x);
-        load8((const T*)A.g.dv + th * d + 8 * l, gv);
-        float dx[8];
+    for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatchBwd * rows) {
+      float xb[kGlueBatchBwd][8], gvb[kGlueBatchBwd][8], brb[kGlueBatchBwd][8], gbb[kGlueBatchBwd][8];
+      float dtr[kGlueBatchBwd], bsr[kGlueBatchBwd], dgr[kGlueBatchBwd];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { dx[e] = gv[e] * bs; dbs = fmaf(gv[e], x[e], dbs); }
-        store8((T*)A.g.dx + th * d + 8 * l, dx);
-        if (has_b) {
-          float br[8], gb[8], out[8];
-          load8((const T*)A.t.b_raw + th * d + 8 * l, br);
-          load8((const T*)A.g.db + th * d + 8 * l, gb);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float s = sigmoidf_(br[e]);
-            out[e] = gb[e] * sp * bs * s * (1.f - s);
-            dsp = fmaf(gb[e], s, dsp);
+      for (int u = 0; u < kGlueBatchBwd; ++u) {
+        const int tok = tb + u * rows;
+        dtr[u] = bsr[u] = dgr[u] = 0.f;
+        if (tok < tok1) {
+          const int64_t th = (int64_t)tok * A.H + h;
+          dtr[u] = to_f32(((const T*)A.t.dt_raw)[th]);
+          if (!A.mamba) bsr[u] = to_f32(((const T*)A.t.bs_raw)[th]);
+          if (l == 0) dgr[u] = A.g.dgt[th];
+          if (on) {
+            load8((const T*)A.t.x + th * d + 8 * l, xb[u]);
+            load8((const T*)A.g.dv + th * d + 8 * l, gvb[u]);
+            if (has_b) {
+              load8((const T*)A.t.b_raw + th * d + 8 * l, brb[u]);
+              load8((const T*)A.g.db + th * d + 8 * l, gbb[u]);
+            }
           }
-          store8((T*)A.g.db_raw + th * d + 8 * l, out);
         }
       }
-      dbs = group_sum(fmaf(dsp, sp, dbs), GL);   // d/d bs of v = x bs and b = s sp bs
-      if (l == 0) {
-        float ddt;
+#pragma unroll
+      for (int u = 0; u < kGlueBatchBwd; ++u) {
+        const int tok = tb + u * rows;
+        if (tok >= tok1) break;   // the lanes of a row leave together
+        const int64_t th = (int64_t)tok * A.H + h;
+        const float pre = dtr[u] + bias;
+        float sg = 0.f, bs;
+        bool pass = true;     // mamba: the clamp lets the gradient through (bounds included, as torch.clamp)
         if (A.mamba) {
-          // gt is an output and the multiplier of x and b
-          ddt = pass ? (A.g.dgt[th] + dbs) * sigmoidf_(pre) : 0.f;
+          const float spd = softplusf_(pre);
+          pass = spd >= A.dt_min && spd <= A.dt_max;
+          bs = fminf(fmaxf(spd, A.dt_min), A.dt_max);
         } else {
-          ((T*)A.g.dbs_raw)[th] = from_f32<T>(dbs * sg * (1.f - sg));
-          ddt = A.g.dgt[th] * sigmoidf_(pre);
+          sg = sigmoidf_(bsr[u]);
+          bs = round_to<T>(sg);
         }
-        ((T*)A.g.ddt_raw)[th] = from_f32<T>(ddt);
-        acc_dt += ddt;
+        float dbs = 0.f, dsp = 0.f;
+        if (on) {
+          const float *x = xb[u], *gv = gvb[u];
+          float dx[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { dx[e] = gv[e] * bs; dbs = fmaf(gv[e], x[e], dbs); }
+          store8((T*)A.g.dx + th * d + 8 * l, dx);
+          if (has_b) {
+            const float *br = brb[u], *gb = gbb[u];
+            float out[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float s = sigmoidf_(br[e]);
+              out[e] = gb[e] * sp * bs * s * (1.f - s);
+              dsp = fmaf(gb[e], s, dsp);
+            }
+            store8((T*)A.g.db_raw + th * d + 8 * l, out);
+          }
+        }
+        dbs = group_sum(fmaf(dsp, sp, dbs), GL);   // d/d bs of v = x bs and b = s sp bs
+        if (l == 0) {
+          float ddt;
+          if (A.mamba) {
+            // gt is an output and the multiplier of x and b
+            ddt = pass ? (dgr[u] + dbs) * sigmoidf_(pre) : 0.f;
+          } else {
+            ((T*)A.g.dbs_raw)[th] = from_f32<T>(dbs * sg * (1.f - sg));
+            ddt = dgr[u] * sigmoidf_(pre);
+          }
+          ((T*)A.g.ddt_raw)[th] = from_f32<T>(ddt);
+          acc_dt += ddt;
+        }
+        acc_bs = fmaf(dsp, bs, acc_bs);
       }
-      acc_bs = fmaf(dsp, bs, acc_bs);
     }
     // workgroup totals in a fixed order: lanes, then waves
     acc_dt = wave_sum(acc_dt);
@@ -291,35 +368,45 @@ __global__ __launch_bounds__(256) void epilogue_fwd_kernel(EpilogueArgs A) {
   float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (on) load8(A.t.weight + 8 * l, w);
   const float inv_d = 1.f / (float)d;
-  for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-    const int64_t th = (int64_t)tok * A.H + h;
-    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (on) {
-      load8((const T*)A.t.o + th * d + 8 * l, r);
-      if (A.t.x) {
-        float x[8];
-        load8((const T*)A.t.x + th * d + 8 * l, x);
+  const bool has_x = A.t.x != nullptr, has_gate = A.t.gate != nullptr;
+  for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatch * rows) {
+    float rb[kGlueBatch][8], xb[kGlueBatch][8], gb[kGlueBatch][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) r[e] = fmaf(x[e], Dh, r[e]);
+    for (int u = 0; u < kGlueBatch; ++u) {
+      const int tok = tb + u * rows;
+      const int64_t th = (int64_t)tok * A.H + h;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rb[u][e] = xb[u][e] = gb[u][e] = 0.f;
+      if (on && tok < tok1) {
+        load8((const T*)A.t.o + th * d + 8 * l, rb[u]);
+        if (has_x) load8((const T*)A.t.x + th * d + 8 * l, xb[u]);
+        if (has_gate) load8((const T*)A.t.gate + th * d + 8 * l, gb[u]);
       }
     }
-    float ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ss = fmaf(r[e], r[e], ss);
-    ss = group_sum(ss, GL);
-    const float rstd = rsqrtf(ss * inv_d + A.eps);
-    if (l == 0) A.t.rstd[th] = rstd;
-    if (!on) continue;
-    float y[8];
+    for (int u = 0; u < kGlueBatch; ++u) {
+      const int tok = tb + u * rows;
+      if (tok >= tok1) break;   // the lanes of a row leave together
+      const int64_t th = (int64_t)tok * A.H + h;
+      float* r = rb[u];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = r[e] * rstd * w[e];
-    if (A.t.gate) {
-      float gt[8];
-      load8((const T*)A.t.gate + th * d + 8 * l, gt);
+      for (int e = 0; e < 8; ++e) r[e] = fmaf(xb[u][e], Dh, r[e]);
+      float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] *= gt[e] * sigmoidf_(gt[e]);
+      for (int e = 0; e < 8; ++e) ss = fmaf(r[e], r[e], ss);
+      ss = group_sum(ss, GL);
+      const float rstd = rsqrtf(ss * inv_d + A.eps);
+      if (l == 0) A.t.rstd[th] = rstd;
+      if (!on) continue;
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = r[e] * rstd * w[e];
+      if (has_gate) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] *= gb[u][e] * sigmoidf_(gb[u][e]);
+      }
+      store8((T*)A.t.y + th * d + 8 * l, y);
     }
-    store8((T*)A.t.y + th * d + 8 * l, y);
   }
 }
 
@@ -339,59 +426,73 @@ __global__ __launch_bounds__(256) void epilogue_bwd_kernel(EpilogueArgs A) {
   const float inv_d = 1.f / (float)d;
   float dw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float accD = 0.f;
-  for (int tok = tok0 + slot; tok < tok1; tok += rows) {
-    const int64_t th = (int64_t)tok * A.H + h;
-    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    float gy[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    float sw[8], dsw[8];   // swish(gate) and its derivative
+  const bool has_x = A.t.x != nullptr, has_gate = A.t.gate != nullptr;
+  for (int tb = tok0 + slot; tb < tok1; tb += kGlueBatchBwd * rows) {
+    float rb[kGlueBatchBwd][8], xb[kGlueBatchBwd][8], gyb[kGlueBatchBwd][8], gtb[kGlueBatchBwd][8], rsb[kGlueBatchBwd];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) { sw[e] = 1.f; dsw[e] = 0.f; }
-    if (on) {
-      load8((const T*)A.t.o + th * d + 8 * l, r);
-      load8((const T*)A.g.dy + th * d + 8 * l, gy);
-      if (A.t.x) {
-        load8((const T*)A.t.x + th * d + 8 * l, x);
+    for (int u = 0; u < kGlueBatchBwd; ++u) {
+      const int tok = tb + u * rows;
+      const int64_t th = (int64_t)tok * A.H + h;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) r[e] = fmaf(x[e], Dh, r[e]);
-      }
-      if (A.t.gate) {
-        float gt[8];
-        load8((const T*)A.t.gate + th * d + 8 * l, gt);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float s = sigmoidf_(gt[e]);
-          sw[e] = gt[e] * s;
-          dsw[e] = s * (1.f + gt[e] * (1.f - s));
+      for (int e = 0; e < 8; ++e) rb[u][e] = xb[u][e] = gyb[u][e] = gtb[u][e] = 0.f;
+      rsb[u] = 0.f;
+      if (tok < tok1) {
+        rsb[u] = A.t.rstd[th];
+        if (on) {
+          load8((const T*)A.t.o + th * d + 8 * l, rb[u]);
+          load8((const T*)A.g.dy + th * d + 8 * l, gyb[u]);
+          if (has_x) load8((const T*)A.t.x + th * d + 8 * l, xb[u]);
+          if (has_gate) load8((const T*)A.t.gate + th * d + 8 * l, gtb[u]);
         }
       }
     }
-    const float rstd = A.t.rstd[th];
-    // n = r rstd;  y = n w sw;  dn = dy w sw;  dr = rstd (dn - n mean(dn n))
-    float n[8], dn[8], dot = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      n[e] = r[e] * rstd;
-      dn[e] = gy[e] * w[e] * sw[e];
-      dot = fmaf(dn[e], n[e], dot);
-      dw[e] = fmaf(gy[e] * n[e], sw[e], dw[e]);
-    }
-    dot = group_sum(dot, GL) * inv_d;
-    if (!on) continue;
-    float dr[8];
+    for (int u = 0; u < kGlueBatchBwd; ++u) {
+      const int tok = tb + u * rows;
+      if (tok >= tok1) break;   // the lanes of a row leave together
+      const int64_t th = (int64_t)tok * A.H + h;
+      float* r = rb[u];
+      const float *x = xb[u], *gy = gyb[u];
+      float sw[8], dsw[8];   // swish(gate) and its derivative
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dr[e] = rstd * (dn[e] - n[e] * dot);
-    store8((T*)A.g.d_o + th * d + 8 * l, dr);
-    if (A.t.x) {
-      float dx[8];
+      for (int e = 0; e < 8; ++e) {
+        r[e] = fmaf(x[e], Dh, r[e]);
+        sw[e] = 1.f;
+        dsw[e] = 0.f;
+        if (has_gate) {
+          const float z = gtb[u][e], s = sigmoidf_(z);
+          sw[e] = z * s;
+          dsw[e] = s * (1.f + z * (1.f - s));
+        }
+      }
+      const float rstd = rsb[u];
+      // n = r rstd;  y = n w sw;  dn = dy w sw;  dr = rstd (dn - n mean(dn n))
+      float n[8], dn[8], dot = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { dx[e] = dr[e] * Dh; accD = fmaf(dr[e], x[e], accD); }
-      store8((T*)A.g.dx + th * d + 8 * l, dx);
-    }
-    if (A.t.gate) {
-      float dg[8];
+      for (int e = 0; e < 8; ++e) {
+        n[e] = r[e] * rstd;
+        dn[e] = gy[e] * w[e] * sw[e];
+        dot = fmaf(dn[e], n[e], dot);
+        dw[e] = fmaf(gy[e] * n[e], sw[e], dw[e]);
+      }
+      dot = group_sum(dot, GL) * inv_d;
+      if (!on) continue;
+      float dr[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) dg[e] = gy[e] * n[e] * w[e] * dsw[e];
-      store8((T*)A.g.dgate + th * d + 8 * l, dg);
+      for (int e = 0; e < 8; ++e) dr[e] = rstd * (dn[e] - n[e] * dot);
+      store8((T*)A.g.d_o + th * d + 8 * l, dr);
+      if (has_x) {
+        float dx[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dx[e] = dr[e] * Dh; accD = fmaf(dr[e], x[e], accD); }
+        store8((T*)A.g.dx + th * d + 8 * l, dx);
+      }
+      if (has_gate) {
+        float dg[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dg[e] = gy[e] * n[e] * w[e] * dsw[e];
+        store8((T*)A.g.dgate + th * d + 8 * l, dg);
+      }
     }
   }
   // dweight: the row slots' shares are added in slot order
@@ -490,98 +591,125 @@ __global__ __launch_bounds__(256) void epilogue_heads_fwd_kernel(EpilogueArgs A)
 
 // r = u s, u = o + x D, s = swish(gate);  n = r rstd;  y = n w;  g = dy w;  dr = rstd (g - n mean(g n));
 // du = dr s (= d_o), dx = du D, dgate = dr u s', dD[h] += du . x, dweight += dy n.
-// Two passes over the token's rows (the second finds them in the cache): the mean first, then the gradients.
+// Two passes over the token's rows: the mean first, then the gradients.  NCH = passes of 512 elements, a template
+// parameter: bf16 rows of up to 2048 elements stay in registers as loaded between the passes, longer or fp32 rows are
+// fetched again (they come from the cache).  The sums over tokens (dweight, dD) are kept in the wave's own part of
+// the LDS, not in registers: with 8 accumulators per pass in registers the kernel ran at two waves per SIMD and
+// 2.8 TB/s.
 // part_w: [workgroups][H dv] partial dweight, part_D: [workgroups][H dv / 8] partial dD (one slot per eight elements).
-template <typename T>
-__global__ __launch_bounds__(256) void epilogue_heads_bwd_kernel(EpilogueArgs A) {
+template <typename T, int NCH /* 0: any number of passes, rows fetched twice */>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NCH <= 1 ? 4 : (NCH == 4 ? 2 : 3))))
+void epilogue_heads_bwd_kernel(EpilogueArgs A) {
   extern __shared__ float sPartial[];   // [4 waves][H dv + H dv / 8]
+  constexpr bool KEEP = NCH > 0;
+  static_assert(!KEEP || (sizeof(T) == 2 && NCH <= 4), "rows kept in registers: bf16, at most 2048 elements");
+  const int nch = KEEP ? NCH : (A.H * A.dv + 511) >> 9;
+  using Raw = typename std::conditional<sizeof(T) == 2, bf16x8, F32x8>::type;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int dv = A.dv, HD = A.H * dv, nch = (HD + 511) >> 9;
+  const int dv = A.dv, HD = A.H * dv;
   const float inv_n = 1.f / (float)HD;
   const int64_t wave_id = (int64_t)blockIdx.x * 4 + w;
-  float dw[kHeadsMaxCh][8], accD[kHeadsMaxCh];
-#pragma unroll
-  for (int c = 0; c < kHeadsMaxCh; ++c) {
-    accD[c] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) dw[c][e] = 0.f;
-  }
-  // u, swish(gate) and its derivative, x of eight elements of a token
-  auto fetch = [&](int64_t row, int e0, float* u, float* sw, float* dsw, float* x, float& Dh) {
-    load8((const T*)A.t.o + row + e0, u);
-    Dh = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { sw[e] = 1.f; dsw[e] = 0.f; x[e] = 0.f; }
-    if (A.t.x) {
-      load8((const T*)A.t.x + row + e0, x);
-      Dh = A.t.D[e0 / dv];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) u[e] = fmaf(x[e], Dh, u[e]);
-    }
-    if (A.t.gate) {
-      float z[8];
-      load8((const T*)A.t.gate + row + e0, z);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float sg = sigmoidf_(z[e]);
-        sw[e] = z[e] * sg;
-        dsw[e] = sg * (1.f + z[e] * (1.f - sg));
-      }
-    }
+  const bool has_x = A.t.x != nullptr, has_gate = A.t.gate != nullptr;
+  const int per_wave = HD + (HD >> 3);
+  float* mine = sPartial + w * per_wave;   // this wave's sums: touched by no other wave before the barrier below
+  for (int e = lane; e < per_wave; e += 64) mine[e] = 0.f;
+  struct Rows { Raw o, x, z, gy; };
+  auto fetch = [&](int64_t off, Rows& R) {
+    R.o = *(const Raw*)((const T*)A.t.o + off);
+    R.gy = *(const Raw*)((const T*)A.g.dy + off);
+    if (has_x) R.x = *(const Raw*)((const T*)A.t.x + off);
+    if (has_gate) R.z = *(const Raw*)((const T*)A.t.gate + off);
   };
   for (int it = 0; it < kHeadsIter; ++it) {
     const int tok = (int)wave_id * kHeadsIter + it;
     if (tok >= A.tokens) break;
     const int64_t row = (int64_t)tok * HD;
     const float rstd = A.t.rstd[tok];
+    Rows keep[KEEP ? NCH : 1];
     float dot = 0.f;
+    if constexpr (KEEP) {   // every fetch of the token in flight before the first use
 #pragma unroll
-    for (int c = 0; c < kHeadsMaxCh; ++c) {
-      const int e0 = 512 * c + 8 * lane;
-      if (c < nch && e0 < HD) {
-        float u[8], sw[8], dsw[8], x[8], gy[8], wv[8], Dh;
-        fetch(row, e0, u, sw, dsw, x, Dh);
-        load8((const T*)A.g.dy + row + e0, gy);
-        load8(A.t.weight + e0, wv);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dot = fmaf(gy[e] * wv[e], u[e] * sw[e] * rstd, dot);
+      for (int c = 0; c < NCH; ++c) {
+        const int e0 = 512 * c + 8 * lane;
+        if (e0 < HD) fetch(row + e0, keep[c]);
       }
     }
-    dot = wave_sum(dot) * inv_n;
-#pragma unroll
-    for (int c = 0; c < kHeadsMaxCh; ++c) {
+    auto pass1 = [&](int c) {
       const int e0 = 512 * c + 8 * lane;
-      if (c < nch && e0 < HD) {
-        float u[8], sw[8], dsw[8], x[8], gy[8], wv[8], Dh;
-        fetch(row, e0, u, sw, dsw, x, Dh);
-        load8((const T*)A.g.dy + row + e0, gy);
+      if (e0 < HD) {
+        Rows tmp;
+        if constexpr (!KEEP) fetch(row + e0, tmp);
+        const Rows& R = KEEP ? keep[c] : tmp;
+        const float Dh = has_x ? A.t.D[e0 / dv] : 0.f;
+        float wv[8];
         load8(A.t.weight + e0, wv);
-        float du[8], dz[8], dx[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float n = u[e] * sw[e] * rstd;
-          const float dr = rstd * (gy[e] * wv[e] - n * dot);
-          du[e] = dr * sw[e];
-          dz[e] = dr * u[e] * dsw[e];
+          float r = (float)R.o[e];
+          if (has_x) r = fmaf((float)R.x[e], Dh, r);
+          if (has_gate) {
+            const float z = (float)R.z[e];
+            r *= z * sigmoidf_(z);
+          }
+          dot = fmaf((float)R.gy[e] * wv[e], r, dot);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);   // one pass of 512 elements at a time: the registers of a pass are reused
+    };
+    if constexpr (KEEP) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) pass1(c);
+    } else {
+#pragma unroll 1
+      for (int c = 0; c < nch; ++c) pass1(c);
+    }
+    dot = wave_sum(dot) * (rstd * inv_n);
+    auto pass2 = [&](int c) {
+      const int e0 = 512 * c + 8 * lane;
+      if (e0 < HD) {
+        Rows tmp;
+        if constexpr (!KEEP) fetch(row + e0, tmp);
+        const Rows& R = KEEP ? keep[c] : tmp;
+        const float Dh = has_x ? A.t.D[e0 / dv] : 0.f;
+        float wv[8], du[8], dz[8], dx[8], gn[8];
+        load8(A.t.weight + e0, wv);
+        float aD = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float x = has_x ? (float)R.x[e] : 0.f, gy = (float)R.gy[e];
+          const float u = fmaf(x, Dh, (float)R.o[e]);
+          float sw = 1.f, dsw = 0.f;
+          if (has_gate) {
+            const float z = (float)R.z[e], sg = sigmoidf_(z);
+            sw = z * sg;
+            dsw = sg * (1.f + z * (1.f - sg));
+          }
+          const float n = u * sw * rstd;
+          const float dr = rstd * (gy * wv[e] - n * dot);
+          du[e] = dr * sw;
+          dz[e] = dr * u * dsw;
           dx[e] = du[e] * Dh;
-          accD[c] = fmaf(du[e], x[e], accD[c]);
-          dw[c][e] = fmaf(gy[e], n, dw[c][e]);
+          aD = fmaf(du[e], x, aD);
+          gn[e] = gy * n;
         }
         store8((T*)A.g.d_o + row + e0, du);
-        if (A.t.x) store8((T*)A.g.dx + row + e0, dx);
-        if (A.t.gate) store8((T*)A.g.dgate + row + e0, dz);
+        if (has_x) store8((T*)A.g.dx + row + e0, dx);
+        if (has_gate) store8((T*)A.g.dgate + row + e0, dz);
+        f32x4 s0 = *(const f32x4*)(mine + e0), s1 = *(const f32x4*)(mine + e0 + 4);
+        s0 += f32x4{gn[0], gn[1], gn[2], gn[3]};
+        s1 += f32x4{gn[4], gn[5], gn[6], gn[7]};
+        *(f32x4*)(mine + e0) = s0;
+        *(f32x4*)(mine + e0 + 4) = s1;
+        mine[HD + (e0 >> 3)] += aD;
       }
-    }
-  }
-  const int per_wave = HD + (HD >> 3);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (KEEP) {
 #pragma unroll
-  for (int c = 0; c < kHeadsMaxCh; ++c) {
-    const int e0 = 512 * c + 8 * lane;
-    if (c < nch && e0 < HD) {
-      float* pw = sPartial + w * per_wave + e0;
-      *(f32x4*)pw = f32x4{dw[c][0], dw[c][1], dw[c][2], dw[c][3]};
-      *(f32x4*)(pw + 4) = f32x4{dw[c][4], dw[c][5], dw[c][6], dw[c][7]};
-      sPartial[w * per_wave + HD + (e0 >> 3)] = accD[c];
+      for (int c = 0; c < NCH; ++c) pass2(c);
+    } else {
+#pragma unroll 1
+      for (int c = 0; c < nch; ++c) pass2(c);
     }
   }
   __syncthreads();
@@ -590,6 +718,23 @@ __global__ __launch_bounds__(256) void epilogue_heads_bwd_kernel(EpilogueArgs A)
     const float tot = (sPartial[e] + sPartial[per_wave + e]) + (sPartial[2 * per_wave + e] + sPartial[3 * per_wave + e]);
     if (e < HD) A.part_w[(int64_t)blockIdx.x * HD + e] = tot;
     else A.part_D[(int64_t)blockIdx.x * (HD >> 3) + (e - HD)] = tot;
+  }
+}
+
+template <typename T, int NCH>
+static int launch_heads_bwd(const EpilogueArgs& A, int nblk, size_t lds, hipStream_t hs) {
+  if (int rc = allow_lds((const void*)&epilogue_heads_bwd_kernel<T, NCH>, lds)) return rc;
+  PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, (epilogue_heads_bwd_kernel<T, NCH>), dim3(nblk), dim3(256), lds, hs, A);
+  return PAL_OK;
+}
+template <typename T>
+static int launch_heads_bwd_nch(int nch, const EpilogueArgs& A, int nblk, size_t lds, hipStream_t hs) {
+  switch (nch) {
+    case 1: return launch_heads_bwd<T, 1>(A, nblk, lds, hs);
+    case 2: return launch_heads_bwd<T, 2>(A, nblk, lds, hs);
+    case 3: return launch_heads_bwd<T, 3>(A, nblk, lds, hs);
+    case 4: return launch_heads_bwd<T, 4>(A, nblk, lds, hs);
+    default: return launch_heads_bwd<T, 0>(A, nblk, lds, hs);
   }
 }
 
@@ -813,13 +958,10 @@ extern "C" int pal_epilogue_bwd(const PalGlueDims* d, const PalEpilogueTensors* 
     A.part_D = (float*)((char*)workspace + up256(sizeof(float) * (size_t)nblk * HD));
     hipStream_t hs = (hipStream_t)stream;
     const size_t lds = sizeof(float) * 4 * (HD + HD / 8);
-    if (d->dtype == PAL_DTYPE_BF16) {
-      if (int rc = allow_lds((const void*)&epilogue_heads_bwd_kernel<bf16_t>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, epilogue_heads_bwd_kernel<bf16_t>, dim3(nblk), dim3(256), lds, hs, A);
-    } else {
-      if (int rc = allow_lds((const void*)&epilogue_heads_bwd_kernel<float>, lds)) return rc;
-      PAL_TIMED_LAUNCH(kKernEpilogueBwd, hs, epilogue_heads_bwd_kernel<float>, dim3(nblk), dim3(256), lds, hs, A);
-    }
+    const int nch = (int)((HD + 511) / 512);
+    if (int rc = d->dtype == PAL_DTYPE_BF16 ? launch_heads_bwd_nch<bf16_t>(nch, A, nblk, lds, hs)
+                                            : launch_heads_bwd<float, 0>(A, nblk, lds, hs))
+      return rc;
     PAL_HIP_LAUNCH_CHECK();
     hipLaunchKernelGGL(epilogue_heads_reduce_kernel, dim3((unsigned)((HD + 63) / 64 + d->n_heads)), dim3(64 * kRedWaves), 0, hs, A, nblk);
     PAL_HIP_LAUNCH_CHECK();

@@ -253,6 +253,7 @@ MAMBA_SHAPES = [
     ((5,), 2, 256, torch.bfloat16),
     ((2, 40), 4, 64, torch.float32),
     ((2, 300), 16, 96, torch.bfloat16),     # more tokens than one workgroup takes
+    ((2, 21), 16, 128, torch.bfloat16),     # 2048 entries: the longest token the backward keeps in registers
 ]
 
 
