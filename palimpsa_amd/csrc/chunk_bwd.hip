@@ -739,14 +739,18 @@ __global__ __launch_bounds__(256) void chunk_bwd_carry_scan_kernel(BwdArgs A) {
 // PREC (fp32 rows): operands as two bf16 halves, three matrix instructions per product; the transposed copy of the
 // carries then holds a second plane with the lo halves (never shared with a result buffer).
 // (second launch bound: at most 256 registers per lane, so matrix results stay in ordinary vector registers)
+// The kernel is a chain of phases, each of which starts with fetches from global memory (the carries, the operand
+// rows, the gradients it adds to); taken in turn their latencies add up to most of the kernel's time.  So every fetch
+// is issued as early as its address is known: the operand rows of all four products before the carries are staged,
+// the gradients that a phase adds to before the matrix instructions of that phase.  Every wave scans the gates
+// itself (the decay a_s of its own token rows), so the operands do not wait for another wave.
 template <typename TIn, int KSMAX, bool SEQ, bool PREC>
 __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A) {
   const ChunkArgs& a = A.c;
   extern __shared__ float smem[];
   const int H = a.H, dk = a.dk, dv = a.dv;
   const int dmax = dk > dv ? dk : dv;
-  float* sAs = smem;                       // [64] decay from token s to the end of the tile
-  float* sW4 = sAs + kC;                   // [8]
+  float* sW4 = smem + kC;                  // [8]
   float* sBt = sW4 + 8;                    // [64][dv/8] beta of the carry terms, one slot per work item
   float* sO1 = sBt + kC * (dv >> 3);       // [64][OS] dk^carry, later dv^carry
   float* sO2 = SEQ ? sO1 : sO1 + kC * (dmax + 4);   // [64][OS] db^carry (SEQ: after dv^carry has been applied)
@@ -765,17 +769,20 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
   int bos, len, cbase;
   seq_lookup(a, seq, bos, len, cbase);
   const bool last = cis == (len + kC - 1) / kC - 1;
+  // the gates of the tile's tokens (every wave), and for wave 0 the local part of d log f
+  const bool tok_ok = lane < clen;
+  const int64_t tokL = (int64_t)t0 + lane;
+  const float gt_l = tok_ok ? load_gate(a.gt, tokL * H + h, a.gate_bf16) : 0.f;
+  float e_l = 0.f;
+  if (w == 0 && tok_ok) e_l = A.wE[(int64_t)h * A.tokens + tokL];
   // Gate gradient of the tile's tokens, by wave 0 once the carry terms are known:
   //   d log f_t = (local part, from the tile kernel) + (carry terms of the earlier tokens of the tile) + (boundary term),
   //   dgt_t = -g d log f_t, and the tile's share of dg = -sum_t gt_t d log f_t.
   auto gate_grad = [&](float bc, float bnd) {
-    const bool ok = lane < clen;
     const float pre = wave_inclusive_scan(bc, lane) - bc;
-    const int64_t tok = (int64_t)t0 + lane;
-    const float dlogf = ok ? A.wE[(int64_t)h * A.tokens + tok] + pre + bnd : 0.f;
-    const float gt = ok ? load_gate(a.gt, tok * H + h, a.gate_bf16) : 0.f;
-    if (ok) A.dgt[tok * H + h] = -a.g[h] * dlogf;
-    const float share = wave_sum(-gt * dlogf);
+    const float dlogf = tok_ok ? e_l + pre + bnd : 0.f;
+    if (tok_ok) A.dgt[tokL * H + h] = -a.g[h] * dlogf;
+    const float share = wave_sum(-gt_l * dlogf);
     if (lane == 0) A.wDgTile[(int64_t)cidx * H + h] = share;
   };
   if (last) {  // nothing flows in from beyond the end of the sequence (uniform for the block)
@@ -783,65 +790,25 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
     return;
   }
   const float gh = a.g[h] * kLog2e;
-  if (w == 0) {
-    const float gt = (lane < clen) ? load_gate(a.gt, (int64_t)(t0 + lane) * H + h, a.gate_bf16) : 0.f;
-    const float c = wave_inclusive_scan(-gt * gh, lane);
-    const float tot = __shfl(c, 63);
-    sAs[lane] = fast_exp2(tot - c);
-    if (lane == 0) sW4[4] = fast_exp2(tot);
-  }
-  const int64_t E = (int64_t)dv * dk;
-  const TIn* RM = (const TIn*)A.wDM + ((int64_t)cidx * H + h) * E;
-  const TIn* RJ = (const TIn*)A.wDJ + ((int64_t)cidx * H + h) * E;
-  {
-    // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile; the same
-    // pass leaves R^T in LDS for the products that contract over the value rows
-    const float* smu = a.chunk_mu + ((int64_t)cidx * H + h) * E;
-    const float* sI = a.chunk_I + ((int64_t)cidx * H + h) * E;
-    const float Ipb = a.Ip[h];
-    float acc = 0.f;
-    // a wave instruction covers 16 value rows x 64 bytes, and a wave walks along the rows before it
-    // moves to other rows, so that both halves of a 128-byte line are used while it is still in L1
-    const int nc = dk >> 4, nblk = (dv >> 4) * nc, per = (nblk + 3) >> 2;
-    for (int j = 0; j < per; ++j) {
-      const int blk = w * per + j;
-      if (blk >= nblk) break;
-      const int d = 16 * (blk / nc) + i, c4 = 4 * (blk % nc) + g;
-      const int64_t e = (int64_t)d * dk + 4 * c4;
-      float rm[4], rj[4];
-      load_vec<4>(RM + e, rm);
-      load_vec<4>(RJ + e, rj);
-      const f32x4 mu = *(const f32x4*)(smu + e), I = *(const f32x4*)(sI + e);
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        acc = fmaf(rm[x], mu[x] * I[x], acc);
-        acc = fmaf(rj[x], I[x] - Ipb, acc);
-        const bf16_t mh = (bf16_t)rm[x], jh = (bf16_t)rj[x];
-        sRT[(4 * c4 + x) * RS + d] = mh;
-        sRT[(dk + 4 * c4 + x) * RS + d] = jh;
-        if constexpr (PREC) {
-          sRTl[(4 * c4 + x) * RS + d] = (bf16_t)(rm[x] - (float)mh);
-          sRTl[(dk + 4 * c4 + x) * RS + d] = (bf16_t)(rj[x] - (float)jh);
-        }
-      }
-    }
-    acc = wave_sum(acc);
-    if (lane == 0) sW4[w] = acc;
-  }
-  __syncthreads();
-  const float bnd = sW4[4] * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);   // every thread; the slots are rewritten only after later barriers
-
   const int srow = 16 * w + i;            // operand row (token) of this lane
   const bool row_ok = srow < clen;
-  const float as = sAs[srow];
+  float as, Ftot;                         // decay from token srow to the end of the tile, and over the whole tile
+  {
+    const float c = wave_inclusive_scan(-gt_l * gh, lane);
+    const float tot = __shfl(c, 63);
+    as = fast_exp2(tot - __shfl(c, srow));
+    Ftot = fast_exp2(tot);
+  }
   const int64_t tokA = ((int64_t)(t0 + (row_ok ? srow : 0)) * H + h);
   const int64_t tok0 = ((int64_t)t0 * H + h);
 
-  // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
-  {
+  // operands of the four products: rows a_s v_s, a_s b_s (contraction over the value rows) and a_s k_s, a_s k_s^2
+  // (over the key columns) of this lane's token.  EARLY: built before anything else (the registers are there).
+  constexpr bool EARLY = (PREC ? 2 : 1) * KSMAX <= 4;
+  bf16x8 A3[KSMAX], A4[KSMAX], A1[KSMAX], A2[KSMAX];
+  bf16x8 A3l[PREC ? KSMAX : 1], A4l[PREC ? KSMAX : 1], A1l[PREC ? KSMAX : 1], A2l[PREC ? KSMAX : 1];
+  auto build_vb = [&]() {
     const int KS = (dv + 31) / 32;
-    bf16x8 A3[KSMAX], A4[KSMAX];
-    bf16x8 A3l[PREC ? KSMAX : 1], A4l[PREC ? KSMAX : 1];
     const TIn* vp = (const TIn*)a.v + tokA * dv;
     const TIn* bp = (const TIn*)a.b + tokA * dv;
 #pragma unroll
@@ -863,13 +830,119 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
           split_bf16(bb, A4[ks], A4l[ks]);
         } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          A3[ks][j] = (bf16_t)(as * vv[j]);
-          A4[ks][j] = (bf16_t)(as * bb[j]);
-        }
+          for (int j = 0; j < 8; ++j) {
+            A3[ks][j] = (bf16_t)(as * vv[j]);
+            A4[ks][j] = (bf16_t)(as * bb[j]);
+          }
         }
       }
     }
+  };
+  auto build_k = [&]() {
+    const int KS = (dk + 31) / 32;
+    const TIn* kp = (const TIn*)a.k + qk_row(a, t0 + (row_ok ? srow : 0), h);
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      if (ks < KS) {
+        const int n0 = 8 * g + 32 * ks;
+        float kv[8];
+        if (row_ok && n0 < dk) {
+          load_vec<4>(kp + n0, kv);
+          load_vec<4>(kp + n0 + 4, kv + 4);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) kv[j] = 0.f;
+        }
+        if constexpr (PREC) {
+          float k1[8], k2[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { k1[j] = as * kv[j]; k2[j] = k1[j] * kv[j]; }
+          split_bf16(k1, A1[ks], A1l[ks]);
+          split_bf16(k2, A2[ks], A2l[ks]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            A1[ks][j] = (bf16_t)(as * kv[j]);
+            A2[ks][j] = (bf16_t)(as * kv[j] * kv[j]);
+          }
+        }
+      }
+    }
+  };
+  build_vb();
+  if constexpr (EARLY) build_k();
+
+  const int64_t E = (int64_t)dv * dk;
+  const TIn* RM = (const TIn*)A.wDM + ((int64_t)cidx * H + h) * E;
+  const TIn* RJ = (const TIn*)A.wDJ + ((int64_t)cidx * H + h) * E;
+  {
+    // F_C (<R_M, M_0> + <R_J, J_0>) with (M_0, J_0) the state at the start of this tile; the same
+    // pass leaves R^T in LDS for the products that contract over the value rows
+    const float* smu = a.chunk_mu + ((int64_t)cidx * H + h) * E;
+    const float* sI = a.chunk_I + ((int64_t)cidx * H + h) * E;
+    const float Ipb = a.Ip[h];
+    float acc = 0.f;
+    // a wave instruction covers 16 value rows x 64 bytes, and a wave walks along the rows before it
+    // moves to other rows, so that both halves of a 128-byte line are used while it is still in L1;
+    // four blocks are fetched before the first is used
+    const int nc = dk >> 4, nblk = (dv >> 4) * nc, per = (nblk + 3) >> 2;
+    for (int j0 = 0; j0 < per; j0 += 4) {
+      float rm[4][4], rj[4][4];
+      f32x4 mu[4], I[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int blk = w * per + j0 + u;
+        if (j0 + u < per && blk < nblk) {
+          const int64_t e = (int64_t)(16 * (blk / nc) + i) * dk + 4 * (4 * (blk % nc) + g);
+          load_vec<4>(RM + e, rm[u]);
+          load_vec<4>(RJ + e, rj[u]);
+          mu[u] = *(const f32x4*)(smu + e);
+          I[u] = *(const f32x4*)(sI + e);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int blk = w * per + j0 + u;
+        if (j0 + u < per && blk < nblk) {
+          const int d = 16 * (blk / nc) + i, c4 = 4 * (blk % nc) + g;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            acc = fmaf(rm[u][x], mu[u][x] * I[u][x], acc);
+            acc = fmaf(rj[u][x], I[u][x] - Ipb, acc);
+            const bf16_t mh = (bf16_t)rm[u][x], jh = (bf16_t)rj[u][x];
+            sRT[(4 * c4 + x) * RS + d] = mh;
+            sRT[(dk + 4 * c4 + x) * RS + d] = jh;
+            if constexpr (PREC) {
+              sRTl[(4 * c4 + x) * RS + d] = (bf16_t)(rm[u][x] - (float)mh);
+              sRTl[(dk + 4 * c4 + x) * RS + d] = (bf16_t)(rj[u][x] - (float)jh);
+            }
+          }
+        }
+      }
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) sW4[w] = acc;
+  }
+  // gradients this kernel adds to, as fetched: item m of a thread is (token s, eight consecutive entries c8) with
+  // s * groups + c8 = tid + 256 m; a row has at most 4 KSMAX groups of eight, so a thread has at most KSMAX items
+  // PRE: fetched a phase ahead, where the registers are there for it (else right before they are used)
+  constexpr bool PRE = KSMAX <= 2 || (KSMAX == 4 && SEQ && !PREC && sizeof(TIn) == 2);
+  Raw8<TIn> old1[KSMAX], old2[KSMAX], in1[KSMAX], in2[KSMAX];
+  auto fetch_items = [&](const TIn* p, int groups, int row_len, Raw8<TIn>* dst) {
+#pragma unroll
+    for (int m = 0; m < KSMAX; ++m) {
+      const int idx = tid + 256 * m, c8 = idx % groups, s = idx / groups;
+      if (idx < kC * groups && s < clen) dst[m].load(p + (int64_t)s * H * row_len + 8 * c8);
+    }
+  };
+  TIn* dko = (TIn*)A.dk + tok0 * dk;
+  if constexpr (PRE) fetch_items(dko, dk >> 3, dk, old1);
+  __syncthreads();
+  const float bnd = Ftot * (sW4[0] + sW4[1] + sW4[2] + sW4[3]);   // every thread; the slots are not written again
+
+  // ---- dk: out[s, n] = sum_d (a_s v_s[d]) R_M[d, n] + 2 k_s[n] sum_d (a_s b_s[d]) R_J[d, n]
+  {
+    const int KS = (dv + 31) / 32;
     const TIn* kin = (const TIn*)a.k + qk_row(a, t0, h);
     // k of the result entries (row s = 16w + 4g + r, column n = 16nbk + i), fetched one step ahead
     auto load_k4 = [&](int nbk, float* kv) {
@@ -906,8 +979,8 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
             accM = mfma16_split(A3[ks], A3l[ks], B3, B3l, accM);
             accJ = mfma16_split(A4[ks], A4l[ks], B4, B4l, accJ);
           } else {
-          accM = mfma16(A3[ks], B3, accM);
-          accJ = mfma16(A4[ks], B4, accJ);
+            accM = mfma16(A3[ks], B3, accM);
+            accJ = mfma16(A4[ks], B4, accJ);
           }
         }
       }
@@ -920,62 +993,51 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
       }
     }
   }
+  if constexpr (!EARLY) build_k();
+  const int vgroups = dv >> 3;   // work item = (token, 8 value rows); the items of a token sit in adjacent lanes
+  const TIn* vin = (const TIn*)a.v + tok0 * dv;
+  const TIn* bin = (const TIn*)a.b + tok0 * dv;
+  TIn* dvo = (TIn*)A.dv + tok0 * dv;
+  TIn* dbo = (TIn*)A.db + tok0 * dv;
+  // dv and its v rows for the next phase (SEQ: db and b before the second pass)
+  if constexpr (PRE) {
+    fetch_items(vin, vgroups, dv, in1);
+    fetch_items(dvo, vgroups, dv, old2);
+  }
   __syncthreads();
   {
     const int groups = dk >> 3;
-    TIn* dko = (TIn*)A.dk + tok0 * dk;
-    for (int idx = tid; idx < kC * groups; idx += 256) {
-      const int c8 = idx % groups, s = idx / groups;
-      if (s < clen) {
-        const int64_t off = (int64_t)s * H * dk + 8 * c8;
+    auto item = [&](int m) {
+      const int idx = tid + 256 * m, c8 = idx % groups, s = idx / groups;
+      if (idx < kC * groups && s < clen) {
+        TIn* o = dko + (int64_t)s * H * dk + 8 * c8;
+        Raw8<TIn> now;
+        if constexpr (!PRE) now.load(o);
+        const Raw8<TIn>& was = PRE ? old1[m] : now;
         float gk[8];
-        load_vec<4>(dko + off, gk); load_vec<4>(dko + off + 4, gk + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) gk[e] += sO1[s * OS + 8 * c8 + e];
-        store_vec<4>(dko + off, gk); store_vec<4>(dko + off + 4, gk + 4);
+        for (int e = 0; e < 8; ++e) gk[e] = was.get(e) + sO1[s * OS + 8 * c8 + e];
+        store_vec<4>(o, gk); store_vec<4>(o + 4, gk + 4);
       }
+    };
+    if constexpr (PRE) {
+#pragma unroll
+      for (int m = 0; m < KSMAX; ++m) item(m);
+    } else {
+#pragma unroll 1
+      for (int m = 0; m < KSMAX; ++m) item(m);
     }
+  }
+  if constexpr (PRE && !SEQ) {
+    fetch_items(bin, vgroups, dv, in2);
+    fetch_items(dbo, vgroups, dv, old1);
   }
   __syncthreads();   // sO1 is free again
 
   // ---- dv, db: out[s, d] = sum_n (a_s k_s[n]) R_M[d, n]
   {
     const int KS = (dk + 31) / 32;
-    bf16x8 A1[KSMAX], A2[KSMAX];
-    bf16x8 A1l[PREC ? KSMAX : 1], A2l[PREC ? KSMAX : 1];
-    const TIn* kp = (const TIn*)a.k + qk_row(a, t0 + (row_ok ? srow : 0), h);
-#pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks) {
-      if (ks < KS) {
-        const int n0 = 8 * g + 32 * ks;
-        float kv[8];
-        if (row_ok && n0 < dk) {
-          load_vec<4>(kp + n0, kv);
-          load_vec<4>(kp + n0 + 4, kv + 4);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) kv[j] = 0.f;
-        }
-        if constexpr (PREC) {
-          float k1[8], k2[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) { k1[j] = as * kv[j]; k2[j] = k1[j] * kv[j]; }
-          split_bf16(k1, A1[ks], A1l[ks]);
-          split_bf16(k2, A2[ks], A2l[ks]);
-        } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          A1[ks][j] = (bf16_t)(as * kv[j]);
-          A2[ks][j] = (bf16_t)(as * kv[j] * kv[j]);
-        }
-        }
-      }
-    }
-    const int groups = dv >> 3;   // work item = (token, 8 value rows); the items of a token sit in adjacent lanes
-    const TIn* vin = (const TIn*)a.v + tok0 * dv;
-    const TIn* bin = (const TIn*)a.b + tok0 * dv;
-    TIn* dvo = (TIn*)A.dv + tok0 * dv;
-    TIn* dbo = (TIn*)A.db + tok0 * dv;
+    const int groups = vgroups;
     constexpr int NPASS = SEQ ? 2 : 1;
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
@@ -1035,44 +1097,62 @@ __global__ __launch_bounds__(256, 2) void chunk_bwd_carry_apply_kernel(BwdArgs A
       }
       __syncthreads();
       // add to the tile-local dv, db; beta_s = <v_s, dv^carry_s> + <b_s, db^carry_s>
-      for (int idx = tid; idx < kC * groups; idx += 256) {
-        const int c8 = idx % groups, s = idx / groups;
-        float beta = 0.f;
-        if (s < clen) {
-          const int64_t off = (int64_t)s * H * dv + 8 * c8;
-          if (doV) {
-            float xv[8], gv[8];
-            load_vec<4>(vin + off, xv); load_vec<4>(vin + off + 4, xv + 4);
-            load_vec<4>(dvo + off, gv); load_vec<4>(dvo + off + 4, gv + 4);
+      // (SEQ: the rows of the pass are in in1/old2; else v, dv in in1/old2 and b, db in in2/old1)
+      auto item = [&](int m) {
+        const int idx = tid + 256 * m, c8 = idx % groups, s = idx / groups;
+        if (idx < kC * groups) {
+          float beta = 0.f;
+          if (s < clen) {
+            const int64_t off = (int64_t)s * H * dv + 8 * c8;
+            if (doV) {
+              Raw8<TIn> x_now, g_now;
+              if constexpr (!PRE) { x_now.load(vin + off); g_now.load(dvo + off); }
+              const Raw8<TIn>& xv = PRE ? in1[m] : x_now;
+              const Raw8<TIn>& gvo = PRE ? old2[m] : g_now;
+              float gv[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float cv = sO1[s * OS + 8 * c8 + e];
-              beta = fmaf(xv[e], cv, beta);
-              gv[e] += cv;
+              for (int e = 0; e < 8; ++e) {
+                const float cv = sO1[s * OS + 8 * c8 + e];
+                beta = fmaf(xv.get(e), cv, beta);
+                gv[e] = gvo.get(e) + cv;
+              }
+              store_vec<4>(dvo + off, gv); store_vec<4>(dvo + off + 4, gv + 4);
             }
-            store_vec<4>(dvo + off, gv); store_vec<4>(dvo + off + 4, gv + 4);
-          }
-          if (doB) {
-            float xb[8], gb[8];
-            load_vec<4>(bin + off, xb); load_vec<4>(bin + off + 4, xb + 4);
-            load_vec<4>(dbo + off, gb); load_vec<4>(dbo + off + 4, gb + 4);
+            if (doB) {
+              Raw8<TIn> x_now, g_now;
+              if constexpr (!PRE) { x_now.load(bin + off); g_now.load(dbo + off); }
+              const Raw8<TIn>& xb = PRE ? (SEQ ? in1[m] : in2[m]) : x_now;
+              const Raw8<TIn>& gbo = PRE ? (SEQ ? old2[m] : old1[m]) : g_now;
+              float gb[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float cb = sO2[s * OS + 8 * c8 + e];
-              beta = fmaf(xb[e], cb, beta);
-              gb[e] += cb;
+              for (int e = 0; e < 8; ++e) {
+                const float cb = sO2[s * OS + 8 * c8 + e];
+                beta = fmaf(xb.get(e), cb, beta);
+                gb[e] = gbo.get(e) + cb;
+              }
+              store_vec<4>(dbo + off, gb); store_vec<4>(dbo + off + 4, gb + 4);
             }
-            store_vec<4>(dbo + off, gb); store_vec<4>(dbo + off + 4, gb + 4);
           }
+          // the second pass of SEQ adds to the share the same thread left in the first
+          sBt[idx] = (SEQ && pass == 1) ? sBt[idx] + beta : beta;
         }
-        // the second pass of SEQ adds to the share the same thread left in the first
-        sBt[idx] = (SEQ && pass == 1) ? sBt[idx] + beta : beta;
+      };
+      if constexpr (PRE) {
+#pragma unroll
+        for (int m = 0; m < KSMAX; ++m) item(m);
+      } else {
+#pragma unroll 1
+        for (int m = 0; m < KSMAX; ++m) item(m);
+      }
+      if (PRE && SEQ && pass == 0) {
+        fetch_items(bin, groups, dv, in1);
+        fetch_items(dbo, groups, dv, old2);
       }
       __syncthreads();   // SEQ: the result buffer is free for the next pass; last pass: sBt is complete
     }
     if (w == 0) {
       float bsum = 0.f;
-      if (lane < clen)
+      if (tok_ok)
         for (int c8 = 0; c8 < groups; ++c8) bsum += sBt[lane * groups + c8];   // fixed order
       gate_grad(bsum, bnd);
     }

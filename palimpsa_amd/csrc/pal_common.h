@@ -95,6 +95,21 @@ __device__ __forceinline__ void load_vec(const bf16_t* p, float* out) {
     out[0] = (float)*p;
   }
 }
+// eight consecutive elements of a row as fetched (two 8- or 16-byte accesses), converted when they are used
+template <typename T>
+struct Raw8;
+template <>
+struct Raw8<bf16_t> {
+  bf16x4 lo, hi;
+  __device__ __forceinline__ void load(const bf16_t* p) { lo = *(const bf16x4*)p; hi = *(const bf16x4*)(p + 4); }
+  __device__ __forceinline__ float get(int e) const { return (float)(e < 4 ? lo[e & 3] : hi[e & 3]); }
+};
+template <>
+struct Raw8<float> {
+  f32x4 lo, hi;
+  __device__ __forceinline__ void load(const float* p) { lo = *(const f32x4*)p; hi = *(const f32x4*)(p + 4); }
+  __device__ __forceinline__ float get(int e) const { return e < 4 ? lo[e & 3] : hi[e & 3]; }
+};
 template <int VW>
 __device__ __forceinline__ void store_vec(float* p, const float* in) {
   if constexpr (VW == 4) {
